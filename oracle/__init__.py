@@ -1,0 +1,236 @@
+"""CPU oracle for the linear-recurrence scan -- TEST INFRASTRUCTURE ONLY.
+
+Importable from ``tests/``, ``__graft_entry__.smoke()`` and the ``cpu_baseline``
+leg of ``bench.py``; the shipped package never imports it.
+
+Thin ``ctypes``/NumPy binding of ``oracle/scan_oracle.c`` (a restatement of
+``sequential_scan/common.py:46-59`` and
+``csrc/include/sequential_scan_cpu.hpp:5-115`` of the reference) and, when it
+has been built, of ``oracle/_ref/libref_scan.so`` -- the reference's own C++
+header compiled unchanged.
+
+All arrays are C-contiguous ``(bs, seq, d)``.  bf16 tensors travel as
+``uint16`` bit patterns.
+"""
+from __future__ import annotations
+
+import ctypes
+import os
+import subprocess
+from typing import List, Optional, Tuple
+
+import numpy as np
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+_LIB_PATH = os.path.join(_HERE, "_build", "liboracle.so")
+_REF_PATH = os.path.join(_HERE, "_ref", "libref_scan.so")
+
+_i64 = ctypes.c_int64
+_ptr = ctypes.c_void_p
+
+
+def build(with_ref: Optional[bool] = None, reference_dir: str = "/root/reference") -> None:
+    """Compile the oracle; also the reference driver when the checkout exists."""
+    subprocess.run(["make", "-C", _HERE, "-B", "all"], check=True, capture_output=True)
+    if with_ref is None:
+        with_ref = os.path.isfile(
+            os.path.join(reference_dir, "csrc", "include", "sequential_scan_cpu.hpp")
+        )
+    if with_ref:
+        subprocess.run(
+            ["make", "-C", _HERE, "-B", "ref", f"REFERENCE_DIR={reference_dir}"],
+            check=True,
+            capture_output=True,
+        )
+
+
+_lib = None
+_ref = None
+
+
+def _load() -> ctypes.CDLL:
+    global _lib
+    if _lib is None:
+        if not os.path.isfile(_LIB_PATH):
+            build(with_ref=False)
+        _lib = ctypes.CDLL(_LIB_PATH)
+    return _lib
+
+
+def _c(a: np.ndarray, dtype) -> np.ndarray:
+    a = np.ascontiguousarray(a, dtype=dtype)
+    if a.ndim != 3:
+        raise ValueError(f"expected a (bs, seq, d) array, got shape {a.shape}")
+    return a
+
+
+def _p(a: np.ndarray) -> _ptr:
+    return _ptr(a.ctypes.data)
+
+
+def _dims(a: np.ndarray) -> Tuple[_i64, _i64, _i64]:
+    return _i64(a.shape[0]), _i64(a.shape[1]), _i64(a.shape[2])
+
+
+def _same_shape(*arrays: np.ndarray) -> None:
+    s = arrays[0].shape
+    for a in arrays[1:]:
+        if a.shape != s:
+            raise ValueError(f"shape mismatch: {s} vs {a.shape}")
+
+
+# --------------------------------------------------------------- fp32 / fp64
+
+
+def scan_fwd_f32(alpha, beta, fused: bool = False) -> np.ndarray:
+    a, b = _c(alpha, np.float32), _c(beta, np.float32)
+    _same_shape(a, b)
+    h = np.empty_like(a)
+    _load().oracle_scan_fwd_f32(_p(a), _p(b), _p(h), *_dims(a), ctypes.c_int(int(fused)))
+    return h
+
+
+def scan_bwd_f32(alpha, h, dout, fused: bool = False) -> Tuple[np.ndarray, np.ndarray]:
+    a, hh, do = _c(alpha, np.float32), _c(h, np.float32), _c(dout, np.float32)
+    _same_shape(a, hh, do)
+    ga, gb = np.empty_like(a), np.empty_like(a)
+    _load().oracle_scan_bwd_f32(
+        _p(a), _p(hh), _p(do), _p(ga), _p(gb), *_dims(a), ctypes.c_int(int(fused))
+    )
+    return ga, gb
+
+
+def scan_fwd_f64(alpha, beta) -> np.ndarray:
+    a, b = _c(alpha, np.float64), _c(beta, np.float64)
+    _same_shape(a, b)
+    h = np.empty_like(a)
+    _load().oracle_scan_fwd_f64(_p(a), _p(b), _p(h), *_dims(a))
+    return h
+
+
+def scan_bwd_f64(alpha, h, dout) -> Tuple[np.ndarray, np.ndarray]:
+    a, hh, do = _c(alpha, np.float64), _c(h, np.float64), _c(dout, np.float64)
+    _same_shape(a, hh, do)
+    ga, gb = np.empty_like(a), np.empty_like(a)
+    _load().oracle_scan_bwd_f64(_p(a), _p(hh), _p(do), _p(ga), _p(gb), *_dims(a))
+    return ga, gb
+
+
+# ---------------------------------------------------------------------- bf16
+
+
+def scan_fwd_bf16(alpha_bits, beta_bits, fused: bool = False) -> np.ndarray:
+    """bf16 bits in, bf16 bits out, fp32 carry."""
+    a, b = _c(alpha_bits, np.uint16), _c(beta_bits, np.uint16)
+    _same_shape(a, b)
+    h = np.empty_like(a)
+    _load().oracle_scan_fwd_bf16(_p(a), _p(b), _p(h), *_dims(a), ctypes.c_int(int(fused)))
+    return h
+
+
+def scan_bwd_bf16(alpha_bits, h_bits, dout_bits, fused: bool = False):
+    """bf16 bits in (h = stored forward output), bf16 bits out, fp32 carry."""
+    a, hh, do = _c(alpha_bits, np.uint16), _c(h_bits, np.uint16), _c(dout_bits, np.uint16)
+    _same_shape(a, hh, do)
+    ga, gb = np.empty_like(a), np.empty_like(a)
+    _load().oracle_scan_bwd_bf16(
+        _p(a), _p(hh), _p(do), _p(ga), _p(gb), *_dims(a), ctypes.c_int(int(fused))
+    )
+    return ga, gb
+
+
+def scan_fwd_bf16_f32out(alpha_bits, beta_bits) -> np.ndarray:
+    """Grading oracle: bf16 inputs, everything after the load in fp32."""
+    a, b = _c(alpha_bits, np.uint16), _c(beta_bits, np.uint16)
+    _same_shape(a, b)
+    h = np.empty(a.shape, dtype=np.float32)
+    _load().oracle_scan_fwd_bf16_f32out(_p(a), _p(b), _p(h), *_dims(a))
+    return h
+
+
+def scan_bwd_bf16_f32out(alpha_bits, h_f32, dout_bits):
+    a, do = _c(alpha_bits, np.uint16), _c(dout_bits, np.uint16)
+    hh = _c(h_f32, np.float32)
+    _same_shape(a, hh, do)
+    ga = np.empty(a.shape, dtype=np.float32)
+    gb = np.empty(a.shape, dtype=np.float32)
+    _load().oracle_scan_bwd_bf16_f32out(_p(a), _p(hh), _p(do), _p(ga), _p(gb), *_dims(a))
+    return ga, gb
+
+
+def f32_to_bf16_bits(x) -> np.ndarray:
+    x = np.ascontiguousarray(x, dtype=np.float32)
+    out = np.empty(x.shape, dtype=np.uint16)
+    _load().oracle_f32_to_bf16(_p(x), _p(out), _i64(x.size))
+    return out
+
+
+def bf16_bits_to_f32(bits) -> np.ndarray:
+    bits = np.ascontiguousarray(bits, dtype=np.uint16)
+    out = np.empty(bits.shape, dtype=np.float32)
+    _load().oracle_bf16_to_f32(_p(bits), _p(out), _i64(bits.size))
+    return out
+
+
+# torch <-> bit-pattern helpers (torch imported lazily: the oracle itself is NumPy)
+
+
+def torch_bf16_to_bits(t) -> np.ndarray:
+    import torch
+
+    assert t.dtype == torch.bfloat16
+    return t.detach().cpu().contiguous().view(torch.int16).numpy().view(np.uint16)
+
+
+def bits_to_torch_bf16(bits):
+    import torch
+
+    return torch.from_numpy(np.ascontiguousarray(bits).view(np.int16).copy()).view(torch.bfloat16)
+
+
+# ------------------------------------------- the reference's own C++ CPU scan
+
+
+def ref_available() -> bool:
+    return os.path.isfile(_REF_PATH)
+
+
+def _load_ref() -> ctypes.CDLL:
+    global _ref
+    if _ref is None:
+        if not ref_available():
+            raise FileNotFoundError(
+                f"{_REF_PATH} is not built (make -C oracle ref needs the reference checkout)"
+            )
+        _ref = ctypes.CDLL(_REF_PATH)
+    return _ref
+
+
+def ref_shapes() -> List[Tuple[int, int, int]]:
+    lib = _load_ref()
+    out = []
+    for i in range(lib.ref_scan_num_shapes()):
+        bs, seq, d = _i64(), _i64(), _i64()
+        lib.ref_scan_shape(i, ctypes.byref(bs), ctypes.byref(seq), ctypes.byref(d))
+        out.append((bs.value, seq.value, d.value))
+    return out
+
+
+def ref_scan_fwd(alpha, beta) -> np.ndarray:
+    a, b = _c(alpha, np.float32), _c(beta, np.float32)
+    _same_shape(a, b)
+    h = np.empty_like(a)
+    rc = _load_ref().ref_scan_fwd(_p(a), _p(b), _p(h), *_dims(a))
+    if rc != 0:
+        raise ValueError(f"shape {a.shape} is not instantiated in oracle/ref_driver.cpp")
+    return h
+
+
+def ref_scan_bwd(alpha, h, dout):
+    a, hh, do = _c(alpha, np.float32), _c(h, np.float32), _c(dout, np.float32)
+    _same_shape(a, hh, do)
+    ga, gb = np.empty_like(a), np.empty_like(a)
+    rc = _load_ref().ref_scan_bwd(_p(a), _p(hh), _p(do), _p(ga), _p(gb), *_dims(a))
+    if rc != 0:
+        raise ValueError(f"shape {a.shape} is not instantiated in oracle/ref_driver.cpp")
+    return ga, gb
