@@ -1,0 +1,134 @@
+"""ctypes binding of the C ABI declared in include/fss_scan.h.
+
+The shared library is the only implementation: when it cannot be loaded every
+entry point of the package raises, there is no fallback path.
+"""
+from __future__ import annotations
+
+import ctypes
+import os
+import threading
+from typing import Optional, Tuple
+
+PKG_DIR = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(PKG_DIR, "_lib", "libfss_scan.so")
+
+FSS_BF16, FSS_F32 = 0, 1
+FSS_FWD, FSS_BWD = 0, 1
+FSS_OK = 0
+FSS_ERR_CHAIN_TIMEOUT = 7
+
+EXPORTED_SYMBOLS = (
+    "fss_abi_version",
+    "fss_strerror",
+    "fss_last_hip_error",
+    "fss_workspace_bytes",
+    "fss_workspace_bytes_max",
+    "fss_workspace_init",
+    "fss_workspace_status",
+    "fss_choose_config",
+    "fss_scan_fwd_bf16",
+    "fss_scan_bwd_bf16",
+    "fss_scan_fwd_f32",
+    "fss_scan_bwd_f32",
+    "fss_scan_fwd_ex",
+    "fss_scan_bwd_ex",
+    "fss_copy_bytes",
+)
+
+
+class FssConfig(ctypes.Structure):
+    _fields_ = [
+        ("vec", ctypes.c_int32),
+        ("steps", ctypes.c_int32),
+        ("waves", ctypes.c_int32),
+        ("reserved", ctypes.c_int32),
+    ]
+
+
+class NativeLibraryMissing(RuntimeError):
+    pass
+
+
+class FssError(RuntimeError):
+    def __init__(self, status: int, message: str):
+        super().__init__(f"fss_scan status {status}: {message}")
+        self.status = status
+
+
+_lock = threading.Lock()
+_lib: Optional[ctypes.CDLL] = None
+
+_vp, _i64, _sz, _int = ctypes.c_void_p, ctypes.c_int64, ctypes.c_size_t, ctypes.c_int
+_cfgp = ctypes.POINTER(FssConfig)
+
+
+def _declare(lib: ctypes.CDLL) -> None:
+    lib.fss_abi_version.restype = _int
+    lib.fss_abi_version.argtypes = []
+    lib.fss_strerror.restype = ctypes.c_char_p
+    lib.fss_strerror.argtypes = [_int]
+    lib.fss_last_hip_error.restype = _int
+    lib.fss_last_hip_error.argtypes = []
+    lib.fss_workspace_bytes.restype = _sz
+    lib.fss_workspace_bytes.argtypes = [_i64, _i64, _i64, _int, _int, _cfgp]
+    lib.fss_workspace_bytes_max.restype = _sz
+    lib.fss_workspace_bytes_max.argtypes = [_i64, _i64, _i64]
+    lib.fss_workspace_init.restype = _int
+    lib.fss_workspace_init.argtypes = [_vp, _sz, _vp]
+    lib.fss_workspace_status.restype = _int
+    lib.fss_workspace_status.argtypes = [_vp, _vp]
+    lib.fss_choose_config.restype = _int
+    lib.fss_choose_config.argtypes = [_i64, _i64, _i64, _int, _int, _sz, _cfgp]
+    fwd = [_vp, _vp, _vp, _i64, _i64, _i64, _vp, _sz, _vp]
+    bwd = [_vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _vp, _sz, _vp]
+    for name in ("fss_scan_fwd_bf16", "fss_scan_fwd_f32"):
+        getattr(lib, name).restype = _int
+        getattr(lib, name).argtypes = fwd
+    for name in ("fss_scan_bwd_bf16", "fss_scan_bwd_f32"):
+        getattr(lib, name).restype = _int
+        getattr(lib, name).argtypes = bwd
+    lib.fss_scan_fwd_ex.restype = _int
+    lib.fss_scan_fwd_ex.argtypes = [_int] + fwd + [_cfgp]
+    lib.fss_scan_bwd_ex.restype = _int
+    lib.fss_scan_bwd_ex.argtypes = [_int] + bwd + [_cfgp]
+    lib.fss_copy_bytes.restype = _int
+    lib.fss_copy_bytes.argtypes = [_vp, _vp, _sz, _vp]
+
+
+def lib() -> ctypes.CDLL:
+    """The loaded library; raises NativeLibraryMissing when it has not been built."""
+    global _lib
+    if _lib is None:
+        with _lock:
+            if _lib is None:
+                if not os.path.isfile(LIB_PATH):
+                    raise NativeLibraryMissing(
+                        f"{LIB_PATH} not found: build it with `python -m fast_sequential_scan_amd.build` "
+                        "(there is no non-HIP fallback)"
+                    )
+                loaded = ctypes.CDLL(LIB_PATH)
+                _declare(loaded)
+                _lib = loaded
+    return _lib
+
+
+def strerror(status: int) -> str:
+    return lib().fss_strerror(status).decode()
+
+
+def check(status: int) -> None:
+    if status != FSS_OK:
+        msg = strerror(status)
+        hip = lib().fss_last_hip_error()
+        if hip:
+            msg += f" (hipError_t {hip})"
+        raise FssError(status, msg)
+
+
+def make_config(cfg: Optional[Tuple[int, int, int]]):
+    """(vec, steps, waves) -> pointer for the *_ex entry points; None -> NULL."""
+    if cfg is None:
+        return None
+    vec, steps, waves = cfg
+    return ctypes.byref(FssConfig(int(vec), int(steps), int(waves), 0))

@@ -1,0 +1,68 @@
+"""Autograd Functions over the HIP scan, with the public surface of the
+reference's sequential_scan/scan_cuda.py: ``SequentialScan`` (bf16, autocast
+aware), ``SequentialScanSingle`` (fp32), ``scan`` and ``scan_single``.
+
+Both Functions save ``(alpha, h)`` - the output itself, no extra activation
+memory (reference scan_cuda.py:20,42) - and the backward returns
+``(grad_alpha, grad_beta)``.
+"""
+from __future__ import annotations
+
+from typing import Any, Tuple
+
+import torch
+from torch.autograd import Function
+from torch.autograd.function import once_differentiable
+
+from . import sequential_scan_cuda as _ext
+
+__all__ = ["SequentialScan", "SequentialScanSingle", "scan", "scan_single"]
+
+
+class SequentialScan(Function):
+    """bf16 scan.  Under ``torch.autocast('cuda')`` floating inputs are cast to
+    bf16 and autocast is switched off inside, as the reference's
+    ``custom_fwd(cast_inputs=torch.bfloat16)`` does (scan_cuda.py:15); outside
+    autocast a non-bf16 input is an error, as it is there."""
+
+    @staticmethod
+    @torch.amp.custom_fwd(device_type="cuda", cast_inputs=torch.bfloat16)
+    def forward(ctx: Any, input_alpha: torch.Tensor, input_beta: torch.Tensor) -> torch.Tensor:
+        h = _ext.scan_forward_half(input_alpha, input_beta)
+        ctx.save_for_backward(input_alpha, h)
+        return h
+
+    @staticmethod
+    @torch.amp.custom_bwd(device_type="cuda")
+    @once_differentiable
+    def backward(ctx: Any, grad_output: torch.Tensor) -> Tuple[torch.Tensor, torch.Tensor]:
+        input_alpha, h = ctx.saved_tensors
+        alpha_grad, beta_grad = _ext.scan_backward_half(input_alpha, h, grad_output)
+        return alpha_grad, beta_grad
+
+
+class SequentialScanSingle(Function):
+    """fp32 scan (reference scan_cuda.py:36-54)."""
+
+    @staticmethod
+    def forward(ctx: Any, input_alpha: torch.Tensor, input_beta: torch.Tensor) -> torch.Tensor:
+        h = _ext.scan_forward(input_alpha, input_beta)
+        ctx.save_for_backward(input_alpha, h)
+        return h
+
+    @staticmethod
+    @once_differentiable
+    def backward(ctx: Any, grad_output: torch.Tensor) -> Tuple[torch.Tensor, torch.Tensor]:
+        input_alpha, h = ctx.saved_tensors
+        alpha_grad, beta_grad = _ext.scan_backward(input_alpha, h, grad_output)
+        return alpha_grad, beta_grad
+
+
+def scan(alpha: torch.Tensor, beta: torch.Tensor) -> torch.Tensor:
+    """h[:,0] = beta[:,0]; h[:,t] = alpha[:,t]*h[:,t-1] + beta[:,t]  (bf16, fp32 carry)."""
+    return SequentialScan.apply(alpha, beta)
+
+
+def scan_single(alpha: torch.Tensor, beta: torch.Tensor) -> torch.Tensor:
+    """The same recurrence on fp32 tensors."""
+    return SequentialScanSingle.apply(alpha, beta)

@@ -1,0 +1,152 @@
+"""The four callees the reference's autograd Functions import from its compiled
+extension (``from sequential_scan_cuda import scan_forward, scan_backward,
+scan_forward_half, scan_backward_half``: sequential_scan/scan_cuda.py:4-9,
+registered in csrc/sequential_scan.cpp:15-22), here as thin torch-tensor
+wrappers over the C ABI of the HIP library.
+
+Same names, argument order and return structure.  Differences, all supersets:
+  * any ``d_model`` and any ``seq >= 1`` (the reference throws for d outside
+    {512,768,1024,1536,2048}: csrc/sequential_scan_kernel.cu:54);
+  * inputs are validated (device, dtype, rank, equal shapes) and made contiguous;
+    the reference checks nothing;
+  * kernels run on the current torch stream, not the legacy default stream;
+  * ``scan_backward_half`` returns a fresh ``grad_beta``; the reference returns
+    ``h_saved`` overwritten in place (csrc/sequential_scan_kernel.cu:197).
+"""
+from __future__ import annotations
+
+from typing import Dict, List, Optional, Tuple
+
+import torch
+
+from . import _native
+
+__all__ = ["scan_forward", "scan_backward", "scan_forward_half", "scan_backward_half"]
+
+_DTYPE_CODE = {torch.bfloat16: _native.FSS_BF16, torch.float32: _native.FSS_F32}
+
+# one workspace per (device, stream): calls on one stream are ordered, calls on
+# different streams must not share the chaining words
+_workspaces: Dict[Tuple[int, int], "_Workspace"] = {}
+
+# the validity tags in a workspace are a 32-bit launch counter: reset long before it wraps
+_REINIT_AFTER_LAUNCHES = 1 << 31
+
+
+class _Workspace:
+    __slots__ = ("buf", "launches")
+
+    def __init__(self, buf: torch.Tensor):
+        self.buf = buf
+        self.launches = 0
+
+
+def _validate(expected: torch.dtype, **tensors: torch.Tensor) -> Tuple[int, int, int]:
+    first_name, first = next(iter(tensors.items()))
+    for name, t in tensors.items():
+        if not isinstance(t, torch.Tensor):
+            raise TypeError(f"{name} must be a torch.Tensor, got {type(t).__name__}")
+        if not t.is_cuda:
+            raise RuntimeError(f"{name} must live on a GPU (got device {t.device})")
+        if t.dtype != expected:
+            raise RuntimeError(f"expected scalar type {expected} for {name} but found {t.dtype}")
+        if t.dim() != 3:
+            raise RuntimeError(f"{name} must have shape (bs, seq, d_model), got {tuple(t.shape)}")
+        if t.device != first.device:
+            raise RuntimeError(f"{name} is on {t.device} but {first_name} is on {first.device}")
+        if t.shape != first.shape:
+            raise RuntimeError(
+                f"{name} has shape {tuple(t.shape)} but {first_name} has shape {tuple(first.shape)}"
+            )
+    bs, seq, d = first.shape
+    return int(bs), int(seq), int(d)
+
+
+def _workspace(device: torch.device, stream: torch.cuda.Stream, need: int) -> torch.Tensor:
+    key = (device.index if device.index is not None else torch.cuda.current_device(), stream.cuda_stream)
+    ws = _workspaces.get(key)
+    if ws is None or ws.buf.numel() < need:
+        ws = _Workspace(torch.empty(max(need, 1 << 20), dtype=torch.uint8, device=device))
+        _native.check(_native.lib().fss_workspace_init(ws.buf.data_ptr(), ws.buf.numel(), stream.cuda_stream))
+        _workspaces[key] = ws
+    elif ws.launches >= _REINIT_AFTER_LAUNCHES:
+        _native.check(_native.lib().fss_workspace_init(ws.buf.data_ptr(), ws.buf.numel(), stream.cuda_stream))
+        ws.launches = 0
+    ws.launches += 1
+    return ws.buf
+
+
+def workspace_status(device: Optional[torch.device] = None) -> None:
+    """Synchronises the current stream and raises if a chained scan timed out (debug aid)."""
+    device = torch.device("cuda", torch.cuda.current_device()) if device is None else device
+    with torch.cuda.device(device):
+        stream = torch.cuda.current_stream()
+        ws = _workspaces.get((device.index, stream.cuda_stream))
+        if ws is not None:
+            _native.check(_native.lib().fss_workspace_status(ws.buf.data_ptr(), stream.cuda_stream))
+
+
+def _forward(dtype: torch.dtype, alpha: torch.Tensor, beta: torch.Tensor, config=None) -> torch.Tensor:
+    bs, seq, d = _validate(dtype, alpha=alpha, beta=beta)
+    alpha, beta = alpha.contiguous(), beta.contiguous()
+    out = torch.empty_like(alpha, memory_format=torch.contiguous_format)
+    if out.numel() == 0:
+        return out
+    lib = _native.lib()
+    code = _DTYPE_CODE[dtype]
+    with torch.cuda.device(alpha.device):
+        stream = torch.cuda.current_stream()
+        need = lib.fss_workspace_bytes(bs, seq, d, code, _native.FSS_FWD, _native.make_config(config))
+        ws = _workspace(alpha.device, stream, need)
+        _native.check(
+            lib.fss_scan_fwd_ex(
+                code, alpha.data_ptr(), beta.data_ptr(), out.data_ptr(), bs, seq, d,
+                ws.data_ptr(), ws.numel(), stream.cuda_stream, _native.make_config(config),
+            )
+        )
+    return out
+
+
+def _backward(
+    dtype: torch.dtype, alpha_saved: torch.Tensor, h_saved: torch.Tensor, grad_out: torch.Tensor, config=None
+) -> List[torch.Tensor]:
+    bs, seq, d = _validate(dtype, alpha_saved=alpha_saved, h_saved=h_saved, grad_out=grad_out)
+    alpha_saved, h_saved, grad_out = alpha_saved.contiguous(), h_saved.contiguous(), grad_out.contiguous()
+    grad_alpha = torch.empty_like(alpha_saved, memory_format=torch.contiguous_format)
+    grad_beta = torch.empty_like(alpha_saved, memory_format=torch.contiguous_format)
+    if grad_alpha.numel() == 0:
+        return [grad_alpha, grad_beta]
+    lib = _native.lib()
+    code = _DTYPE_CODE[dtype]
+    with torch.cuda.device(alpha_saved.device):
+        stream = torch.cuda.current_stream()
+        need = lib.fss_workspace_bytes(bs, seq, d, code, _native.FSS_BWD, _native.make_config(config))
+        ws = _workspace(alpha_saved.device, stream, need)
+        _native.check(
+            lib.fss_scan_bwd_ex(
+                code, alpha_saved.data_ptr(), h_saved.data_ptr(), grad_out.data_ptr(),
+                grad_alpha.data_ptr(), grad_beta.data_ptr(), bs, seq, d,
+                ws.data_ptr(), ws.numel(), stream.cuda_stream, _native.make_config(config),
+            )
+        )
+    return [grad_alpha, grad_beta]
+
+
+def scan_forward(alpha: torch.Tensor, beta: torch.Tensor) -> torch.Tensor:
+    """fp32 forward: csrc/sequential_scan.cpp:15 / sequential_scan_kernel.cu:7-58."""
+    return _forward(torch.float32, alpha, beta)
+
+
+def scan_backward(alpha_saved: torch.Tensor, h_saved: torch.Tensor, grad_out: torch.Tensor) -> List[torch.Tensor]:
+    """fp32 backward -> [grad_alpha, grad_beta]: csrc/sequential_scan.cpp:17 / sequential_scan_kernel.cu:60-124."""
+    return _backward(torch.float32, alpha_saved, h_saved, grad_out)
+
+
+def scan_forward_half(alpha: torch.Tensor, beta: torch.Tensor) -> torch.Tensor:
+    """bf16 forward: csrc/sequential_scan.cpp:19 / sequential_scan_kernel.cu:126-187."""
+    return _forward(torch.bfloat16, alpha, beta)
+
+
+def scan_backward_half(alpha_saved: torch.Tensor, h_saved: torch.Tensor, grad_out: torch.Tensor) -> List[torch.Tensor]:
+    """bf16 backward -> [grad_alpha, grad_beta]: csrc/sequential_scan.cpp:21 / sequential_scan_kernel.cu:189-268."""
+    return _backward(torch.bfloat16, alpha_saved, h_saved, grad_out)

@@ -1,0 +1,55 @@
+"""Seeded synthetic workloads: shared by the parity tests, the smoke entry and the bench.
+
+The five recipes are the workload configurations this build is measured on:
+  C1  bs 2, seq 1024, d 768;  alpha, beta ~ N(0,1)
+  C2  bs 16, seq 2048, d 512; alpha = sigmoid(N(0,1)), beta = N(0,1)*sqrt(1-alpha^2)
+  C3  bs 8, d 1024, seq in {512,1000,2048,3000,4096,8192}; alpha = sigmoid(N(0,1)), beta ~ N(0,1)
+  C4  bs 4, seq 8192, d 2048; alpha = sigmoid(N(0,1)+2), beta ~ N(0,1)
+  C5  bs 1, seq 65521 (prime), d 256; alpha = sigmoid(N(0,1)), beta ~ N(0,1)
+The upstream gradient is N(0,1) everywhere.  Values are drawn in fp32 on the CPU
+from a fixed seed and then rounded to the storage dtype, so the device kernel
+and the CPU oracle see bit-identical inputs.
+"""
+from __future__ import annotations
+
+from typing import Tuple
+
+import torch
+
+RECIPES = ("normal", "hawk", "sigmoid", "sigmoid_plus2")
+
+BASELINE_CASES = {
+    "C1": ("normal", 2, 1024, 768),
+    "C2": ("hawk", 16, 2048, 512),
+    "C3_512": ("sigmoid", 8, 512, 1024),
+    "C3_1000": ("sigmoid", 8, 1000, 1024),
+    "C3_2048": ("sigmoid", 8, 2048, 1024),
+    "C3_3000": ("sigmoid", 8, 3000, 1024),
+    "C3_4096": ("sigmoid", 8, 4096, 1024),
+    "C3_8192": ("sigmoid", 8, 8192, 1024),
+    "C4": ("sigmoid_plus2", 4, 8192, 2048),
+    "C5": ("sigmoid", 1, 65521, 256),
+}
+
+
+def make_inputs(
+    recipe: str, bs: int, seq: int, d: int, dtype: torch.dtype = torch.bfloat16, seed: int = 0
+) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
+    """(alpha, beta, dout) on the CPU in `dtype`."""
+    g = torch.Generator().manual_seed(1000 + seed)
+    shape = (bs, seq, d)
+    x = torch.randn(shape, generator=g, dtype=torch.float32)
+    beta = torch.randn(shape, generator=g, dtype=torch.float32)
+    dout = torch.randn(shape, generator=g, dtype=torch.float32)
+    if recipe == "normal":
+        alpha = x
+    elif recipe == "hawk":
+        alpha = torch.sigmoid(x)
+        beta = beta * torch.sqrt(1.0 - alpha * alpha)
+    elif recipe == "sigmoid":
+        alpha = torch.sigmoid(x)
+    elif recipe == "sigmoid_plus2":
+        alpha = torch.sigmoid(x + 2.0)
+    else:
+        raise ValueError(recipe)
+    return alpha.to(dtype), beta.to(dtype), dout.to(dtype)

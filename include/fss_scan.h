@@ -1,0 +1,167 @@
+/*
+ * fss_scan.h - C ABI of the MI355X (gfx950) linear-recurrence scan library.
+ *
+ * Computes, independently for each of the bs*d channels of row-major
+ * contiguous (bs, seq, d) tensors,
+ *
+ *   forward    h[0] = beta[0];  h[t] = alpha[t]*h[t-1] + beta[t]      (t = 1..seq-1)
+ *   backward   g[seq-1] = dout[seq-1];  g[t] = alpha[t+1]*g[t+1] + dout[t]
+ *              grad_beta[t] = g[t];  grad_alpha[t] = g[t]*h[t-1] (t >= 1);  grad_alpha[0] = 0
+ *
+ * with fp32 carries in both directions.  alpha[:,0,:] is never read.
+ *
+ * This header replaces, for a host written in any language, the pybind11 module
+ * `sequential_scan_cuda` of the reference (csrc/sequential_scan.cpp:13-22) and
+ * the host launchers behind it (csrc/sequential_scan_kernel.cu).  The entry
+ * points take plain device pointers, sizes and a HIP stream; no torch types.
+ *
+ * Conventions
+ *   - Every pointer is a device pointer on the current HIP device.
+ *   - The library never allocates or frees device memory.  Outputs and the
+ *     workspace are the caller's.
+ *   - Calls are asynchronous on `stream` (a hipStream_t passed as void*; NULL is
+ *     the null stream).  No entry point synchronises except fss_workspace_status.
+ *   - Every entry point returns an fss_status (0 = ok); nothing throws.
+ *   - Any seq >= 1 and any d >= 1 are accepted (the reference needs seq >= 2/3 and
+ *     d in {512,768,1024,1536,2048}: csrc/sequential_scan_kernel.cu:136-184).
+ *     Tensors need only their element alignment; 4/8/16-byte aligned tensors
+ *     with d a multiple of 2/4/8 elements take the vectorised paths.
+ *   - Offsets are 64-bit (the reference's are 32-bit:
+ *     csrc/include/sequential_scan_kernel_bf16.cuh:63-70).
+ *
+ * Workspace
+ *   When the sequence is split into more than one chunk the kernels chain the
+ *   chunks through a small workspace (per-chunk carries with validity tags, a
+ *   ticket counter).  Size it with fss_workspace_bytes, zero it ONCE with
+ *   fss_workspace_init; after that every scan call leaves it ready for the
+ *   next one, so steady-state calls launch exactly one kernel.  One workspace
+ *   must not be used by two calls that may run concurrently (use one per
+ *   stream).  A workspace sized for one shape serves any shape whose
+ *   fss_workspace_bytes is not larger.  Validity tags are a 32-bit launch
+ *   counter kept in the workspace: call fss_workspace_init again before a
+ *   workspace has served 2^32-1 chained launches.
+ */
+#ifndef FSS_SCAN_H_
+#define FSS_SCAN_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define FSS_ABI_VERSION 1
+
+typedef enum fss_status {
+  FSS_OK = 0,
+  FSS_ERR_NULL_POINTER = 1,    /* a required pointer is NULL                      */
+  FSS_ERR_BAD_SHAPE = 2,       /* bs, seq or d < 0, or a product overflows        */
+  FSS_ERR_MISALIGNED = 3,      /* a tensor is not aligned to its element size     */
+  FSS_ERR_WORKSPACE_SMALL = 4, /* workspace NULL or smaller than fss_workspace_bytes */
+  FSS_ERR_BAD_CONFIG = 5,      /* explicit launch configuration not supported     */
+  FSS_ERR_LAUNCH = 6,          /* HIP reported an error at launch (see fss_last_hip_error) */
+  FSS_ERR_CHAIN_TIMEOUT = 7,   /* reported by fss_workspace_status: a chunk gave up waiting */
+  FSS_ERR_UNSUPPORTED_DEVICE = 8 /* current device is not gfx950                  */
+} fss_status;
+
+typedef enum fss_dtype { FSS_BF16 = 0, FSS_F32 = 1 } fss_dtype;
+typedef enum fss_dir { FSS_FWD = 0, FSS_BWD = 1 } fss_dir;
+
+/*
+ * Launch configuration.  Zero in a field means "choose for me".
+ *   vec    channels per lane (bf16: 1,2,4,8; fp32: 1,2,4); needs d % vec == 0 and
+ *          tensors aligned to vec elements
+ *   steps  timesteps each lane keeps in registers (8, 16 or 32; vec*steps bounded
+ *          by the register budget of the direction)
+ *   waves  wavefronts per workgroup (1..16); one workgroup scans waves*steps
+ *          consecutive timesteps of 64*vec channels
+ * Results do not depend on the configuration beyond fp32 rounding of the
+ * carries handed between chunks.
+ */
+typedef struct fss_config {
+  int32_t vec;
+  int32_t steps;
+  int32_t waves;
+  int32_t reserved;
+} fss_config;
+
+int fss_abi_version(void);
+const char *fss_strerror(int status);
+/* hipError_t of the most recent failed HIP call made by this thread, 0 if none */
+int fss_last_hip_error(void);
+
+/* Bytes of workspace a scan of this shape needs (a multiple of 256, never 0).
+ * cfg may be NULL. */
+size_t fss_workspace_bytes(int64_t bs, int64_t seq, int64_t d, int dtype, int dir,
+                           const fss_config *cfg);
+/* Upper bound over both directions, both dtypes and every configuration the
+ * library may choose by itself. */
+size_t fss_workspace_bytes_max(int64_t bs, int64_t seq, int64_t d);
+/* Resets the workspace with a fill kernel on `stream` (graph-capturable). */
+int fss_workspace_init(void *workspace, size_t bytes, void *stream);
+/* Synchronises `stream`, then reports FSS_OK or FSS_ERR_CHAIN_TIMEOUT and clears
+ * the sticky error word.  For tests and debugging. */
+int fss_workspace_status(void *workspace, void *stream);
+
+/* The configuration the library would choose for this shape (for reporting). */
+int fss_choose_config(int64_t bs, int64_t seq, int64_t d, int dtype, int dir,
+                      size_t align_bytes, fss_config *out);
+
+/*
+ * bf16 forward.  Replaces scan_forward_half
+ * (csrc/sequential_scan.cpp:19, csrc/sequential_scan_kernel.cu:126-187, kernel
+ * csrc/include/sequential_scan_kernel_bf16.cuh:58-167).  h is written in full.
+ */
+int fss_scan_fwd_bf16(const void *alpha, const void *beta, void *h, int64_t bs,
+                      int64_t seq, int64_t d, void *workspace,
+                      size_t workspace_bytes, void *stream);
+
+/*
+ * bf16 backward.  Replaces scan_backward_half
+ * (csrc/sequential_scan.cpp:21, csrc/sequential_scan_kernel.cu:189-268, kernel
+ * csrc/include/sequential_scan_kernel_bf16.cuh:169-390).  `h` is the stored
+ * forward output.  The five tensors must not overlap: the reference writes
+ * grad_beta over `h` (csrc/sequential_scan_kernel.cu:197), which is only safe
+ * when one thread walks a channel's whole sequence in order; here neighbouring
+ * chunks of a sequence run concurrently and each reads the last row of `h`
+ * before its own chunk.
+ */
+int fss_scan_bwd_bf16(const void *alpha, const void *h, const void *dout,
+                      void *grad_alpha, void *grad_beta, int64_t bs, int64_t seq,
+                      int64_t d, void *workspace, size_t workspace_bytes,
+                      void *stream);
+
+/* fp32 forward.  Replaces scan_forward (csrc/sequential_scan.cpp:15,
+ * csrc/sequential_scan_kernel.cu:7-58, csrc/include/sequential_scan_kernel.cuh:35-129). */
+int fss_scan_fwd_f32(const void *alpha, const void *beta, void *h, int64_t bs,
+                     int64_t seq, int64_t d, void *workspace,
+                     size_t workspace_bytes, void *stream);
+
+/* fp32 backward.  Replaces scan_backward (csrc/sequential_scan.cpp:17,
+ * csrc/sequential_scan_kernel.cu:60-124, csrc/include/sequential_scan_kernel.cuh:131-301). */
+int fss_scan_bwd_f32(const void *alpha, const void *h, const void *dout,
+                     void *grad_alpha, void *grad_beta, int64_t bs, int64_t seq,
+                     int64_t d, void *workspace, size_t workspace_bytes,
+                     void *stream);
+
+/* Same four operations with an explicit dtype and launch configuration (tuning,
+ * and tests that results do not depend on how the sequence is chunked). */
+int fss_scan_fwd_ex(int dtype, const void *alpha, const void *beta, void *h,
+                    int64_t bs, int64_t seq, int64_t d, void *workspace,
+                    size_t workspace_bytes, void *stream, const fss_config *cfg);
+int fss_scan_bwd_ex(int dtype, const void *alpha, const void *h, const void *dout,
+                    void *grad_alpha, void *grad_beta, int64_t bs, int64_t seq,
+                    int64_t d, void *workspace, size_t workspace_bytes,
+                    void *stream, const fss_config *cfg);
+
+/* Plain device-to-device copy kernel of `bytes` bytes (a multiple of 16; both
+ * pointers 16-byte aligned).  Exists so that hardware counters read for the
+ * scan kernels can be scaled by what the same counters read for a transfer of
+ * known size. */
+int fss_copy_bytes(const void *src, void *dst, size_t bytes, void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* FSS_SCAN_H_ */

@@ -1,0 +1,157 @@
+"""CPU-side checks: the C-ABI library loads and exports what include/fss_scan.h
+declares, launch planning is sane, the torch wrappers validate their arguments,
+and the autograd glue behaves like the reference's (with a CPU stand-in behind
+the four extension names, so no kernel runs here)."""
+import ctypes
+import os
+import re
+
+import numpy as np
+import pytest
+import torch
+
+from fast_sequential_scan_amd import _native, scan_cuda
+from fast_sequential_scan_amd import sequential_scan_cuda as ext
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def test_library_exports_every_declared_symbol():
+    header = open(os.path.join(ROOT, "include", "fss_scan.h")).read()
+    declared = set(re.findall(r"^(?:int|size_t|const char \*)\s*(fss_[a-z0-9_]+)\(", header, flags=re.M))
+    assert declared == set(_native.EXPORTED_SYMBOLS)
+    lib = ctypes.CDLL(_native.LIB_PATH)
+    for name in declared:
+        assert hasattr(lib, name), name
+    assert _native.lib().fss_abi_version() == 1
+    assert _native.strerror(0) == "ok"
+    assert "workspace" in _native.strerror(4)
+
+
+def test_workspace_sizing_and_config_choice():
+    lib = _native.lib()
+    cfg = _native.FssConfig()
+    for dtype in (0, 1):
+        for direction in (0, 1):
+            for bs, seq, d in [(8, 4096, 1024), (2, 1024, 768), (1, 65521, 256), (16, 2048, 512), (4, 8192, 2048), (3, 1, 7)]:
+                assert lib.fss_choose_config(bs, seq, d, dtype, direction, 16, ctypes.byref(cfg)) == 0
+                assert d % cfg.vec == 0 and cfg.steps in (8, 16, 32) and 1 <= cfg.waves <= 16
+                need = lib.fss_workspace_bytes(bs, seq, d, dtype, direction, None)
+                assert need >= 256 and need % 256 == 0
+                assert need <= lib.fss_workspace_bytes_max(bs, seq, d)
+                chunks = -(-seq // (cfg.steps * cfg.waves))
+                tiles = bs * -(-d // (64 * cfg.vec)) * chunks
+                expect = 256 + (tiles * 3 * 64 * cfg.vec * 8 if chunks > 1 else 0)
+                assert need == expect
+    # odd d forces the scalar path; 2-byte alignment too
+    assert lib.fss_choose_config(2, 100, 77, 0, 0, 16, ctypes.byref(cfg)) == 0 and cfg.vec == 1
+    assert lib.fss_choose_config(2, 100, 64, 0, 0, 2, ctypes.byref(cfg)) == 0 and cfg.vec == 1
+    # explicit configurations: bad ones are refused, good ones size the workspace
+    bad = _native.FssConfig(3, 8, 1, 0)
+    assert lib.fss_workspace_bytes(2, 100, 64, 0, 0, ctypes.byref(bad)) == 256
+    good = _native.FssConfig(2, 8, 2, 0)
+    assert lib.fss_workspace_bytes(2, 100, 64, 0, 0, ctypes.byref(good)) == 256 + 2 * 1 * 7 * 3 * 128 * 8
+    assert lib.fss_choose_config(-1, 4, 4, 0, 0, 16, ctypes.byref(cfg)) == 2
+
+
+def test_entry_points_reject_bad_arguments_without_a_gpu():
+    lib = _native.lib()
+    buf = (ctypes.c_char * 4096)()
+    p = ctypes.addressof(buf)
+    assert lib.fss_scan_fwd_bf16(None, p, p, 1, 4, 8, None, 0, None) == 1
+    assert lib.fss_scan_fwd_bf16(p, p, p, 1, -4, 8, None, 0, None) == 2
+    assert lib.fss_scan_bwd_bf16(p, None, p, p, p, 1, 4, 8, None, 0, None) == 1
+    assert lib.fss_scan_fwd_f32(p + 2, p, p, 1, 4, 8, None, 0, None) == 3
+    assert lib.fss_scan_fwd_bf16(p, p, p, 0, 4, 8, None, 0, None) == 0  # empty: nothing to do
+    assert lib.fss_scan_fwd_ex(7, p, p, p, 1, 4, 8, None, 0, None, None) == 5
+    assert lib.fss_workspace_init(None, 1024, None) == 1
+    assert lib.fss_copy_bytes(p, p + 1, 16, None) == 3
+    two_chunks = _native.FssConfig(1, 8, 1, 0)
+    assert lib.fss_scan_fwd_ex(0, p, p, p, 1, 9, 8, None, 0, None, ctypes.byref(two_chunks)) == 4
+
+
+def test_wrappers_validate_tensors():
+    a = torch.zeros(2, 4, 8, dtype=torch.bfloat16)
+    with pytest.raises(RuntimeError, match="GPU"):
+        ext.scan_forward_half(a, a)
+    with pytest.raises(TypeError):
+        ext.scan_forward_half(a.numpy() if False else None, a)
+    meta = torch.device("meta")
+    with pytest.raises(RuntimeError):
+        ext.scan_forward(torch.zeros(2, 4, 8, device=meta), torch.zeros(2, 4, 8, device=meta))
+
+
+class _CudaLike:
+    """Lets the validation run on CPU tensors that claim to be on a GPU."""
+
+    def __init__(self, t):
+        self.t = t
+
+
+def test_validation_messages(monkeypatch):
+    class Fake(torch.Tensor):
+        @property
+        def is_cuda(self):
+            return True
+
+    def fake(*shape, dtype=torch.bfloat16):
+        return torch.zeros(*shape, dtype=dtype).as_subclass(Fake)
+
+    with pytest.raises(RuntimeError, match="expected scalar type torch.bfloat16"):
+        ext._validate(torch.bfloat16, alpha=fake(2, 4, 8, dtype=torch.float32), beta=fake(2, 4, 8))
+    with pytest.raises(RuntimeError, match=r"\(bs, seq, d_model\)"):
+        ext._validate(torch.bfloat16, alpha=fake(4, 8), beta=fake(4, 8))
+    with pytest.raises(RuntimeError, match="has shape"):
+        ext._validate(torch.bfloat16, alpha=fake(2, 4, 8), beta=fake(2, 5, 8))
+    assert ext._validate(torch.bfloat16, alpha=fake(2, 4, 8), beta=fake(2, 4, 8)) == (2, 4, 8)
+
+
+def _install_cpu_stand_in(monkeypatch, oracle):
+    def fwd(alpha, beta):
+        return torch.from_numpy(oracle.scan_fwd_f32(alpha.detach().numpy(), beta.detach().numpy()))
+
+    def bwd(alpha, h, dout):
+        ga, gb = oracle.scan_bwd_f32(alpha.detach().numpy(), h.detach().numpy(), dout.detach().numpy())
+        return [torch.from_numpy(ga), torch.from_numpy(gb)]
+
+    monkeypatch.setattr(scan_cuda._ext, "scan_forward", fwd)
+    monkeypatch.setattr(scan_cuda._ext, "scan_backward", bwd)
+
+
+def test_autograd_glue_with_cpu_stand_in(monkeypatch, oracle):
+    """SequentialScanSingle wires (alpha, h) into the backward and returns two grads,
+    as sequential_scan/scan_cuda.py:36-54 does; checked against autograd through a loop."""
+    _install_cpu_stand_in(monkeypatch, oracle)
+    g = torch.Generator().manual_seed(0)
+    alpha = torch.randn(2, 12, 5, generator=g, requires_grad=True)
+    beta = torch.randn(2, 12, 5, generator=g, requires_grad=True)
+    dy = torch.randn(2, 12, 5, generator=g)
+    out = scan_cuda.scan_single(alpha, beta)
+    out.backward(dy)
+    ga, gb = alpha.grad.clone(), beta.grad.clone()
+    alpha.grad = beta.grad = None
+    hs = [beta[:, 0]]
+    for t in range(1, 12):
+        hs.append(hs[-1] * alpha[:, t] + beta[:, t])
+    ref = torch.stack(hs, 1)
+    ref.backward(dy)
+    np.testing.assert_allclose(out.detach().numpy(), ref.detach().numpy(), rtol=1e-5, atol=1e-6)
+    np.testing.assert_allclose(ga.numpy(), alpha.grad.numpy(), rtol=1e-4, atol=1e-5)
+    np.testing.assert_allclose(gb.numpy(), beta.grad.numpy(), rtol=1e-4, atol=1e-5)
+
+
+def test_public_names():
+    import fast_sequential_scan_amd as pkg
+    import sequential_scan
+
+    assert sequential_scan.scan_cu is pkg.scan_cu and sequential_scan.scan_cu_single is pkg.scan_cu_single
+    assert pkg.scan_cu is scan_cuda.scan and pkg.scan_cu_single is scan_cuda.scan_single
+    with pytest.raises(NotImplementedError):
+        pkg.scan_tr(None, None)
+
+
+def test_missing_library_is_an_error(monkeypatch, tmp_path):
+    monkeypatch.setattr(_native, "_lib", None)
+    monkeypatch.setattr(_native, "LIB_PATH", str(tmp_path / "nope.so"))
+    with pytest.raises(_native.NativeLibraryMissing):
+        _native.lib()

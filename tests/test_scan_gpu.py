@@ -1,0 +1,336 @@
+"""GPU parity tests: the HIP kernels, called through the C ABI, against the CPU oracle.
+
+Bars
+  * grading bar: every output within rtol = atol = 1e-2 of the fp32-accumulated
+    sequential scan fed the same seeded bf16 inputs (oracle.*_f32out);
+  * tight bar: bf16 outputs within 2 bf16 ulps of the oracle that rounds exactly
+    where the kernel does (fp32 carry, fused multiply-add, round-to-nearest-even
+    on store, backward fed the same stored h) - bit-exact when one wave scans
+    the whole sequence, because then the operation order is identical;
+  * fp32: relative L2 error < 1e-6, the reference's SINGLE_TOL
+    (sequential_scan/common.py:6,14-17).
+"""
+import numpy as np
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+from fast_sequential_scan_amd import _native, scan_cu, scan_cu_single  # noqa: E402
+from fast_sequential_scan_amd import sequential_scan_cuda as ext  # noqa: E402
+from fast_sequential_scan_amd.workloads import BASELINE_CASES, make_inputs  # noqa: E402
+
+DEV = "cuda:0"
+RTOL = ATOL = 1e-2
+
+
+def bits(t: torch.Tensor) -> np.ndarray:
+    return t.detach().cpu().contiguous().view(torch.int16).numpy().view(np.uint16)
+
+
+def ulp_distance(a_bits: np.ndarray, b_bits: np.ndarray) -> np.ndarray:
+    """Distance in representable bf16 values (sign-magnitude -> ordered integers)."""
+    def ordered(u):
+        u = u.astype(np.int32)
+        return np.where(u & 0x8000, -(u & 0x7FFF), u & 0x7FFF)
+    return np.abs(ordered(a_bits) - ordered(b_bits))
+
+
+def assert_close_f32(got: torch.Tensor, want: np.ndarray, what: str):
+    got = got.detach().float().cpu().numpy()
+    bad = ~(np.abs(got - want) <= ATOL + RTOL * np.abs(want))
+    assert not bad.any(), (
+        f"{what}: {bad.sum()} of {bad.size} elements outside rtol=atol=1e-2; "
+        f"worst abs err {np.abs(got - want)[bad].max():.4g} at {np.argwhere(bad)[0]}"
+    )
+
+
+def rel_l2(x: np.ndarray, y: np.ndarray) -> float:
+    return float(np.linalg.norm((x - y).ravel()) / max(np.linalg.norm(y.ravel()), 1e-30))
+
+
+def run_bf16(alpha, beta, dout, config=None):
+    a, b, do = alpha.to(DEV), beta.to(DEV), dout.to(DEV)
+    h = ext._forward(torch.bfloat16, a, b, config)
+    ga, gb = ext._backward(torch.bfloat16, a, h, do, config)
+    torch.cuda.synchronize()
+    return h, ga, gb
+
+
+def check_bf16(oracle, alpha, beta, dout, config=None, exact=False, max_ulp=2, what=""):
+    h, ga, gb = run_bf16(alpha, beta, dout, config)
+    a_bits, b_bits, d_bits = bits(alpha), bits(beta), bits(dout)
+    # grading bar
+    h32 = oracle.scan_fwd_bf16_f32out(a_bits, b_bits)
+    ga32, gb32 = oracle.scan_bwd_bf16_f32out(a_bits, h32, d_bits)
+    assert_close_f32(h, h32, f"{what} h")
+    assert_close_f32(gb, gb32, f"{what} grad_beta")
+    assert_close_f32(ga, ga32, f"{what} grad_alpha")
+    # tight bar: same rounding points as the kernel
+    h_or = oracle.scan_fwd_bf16(a_bits, b_bits, fused=True)
+    ga_or, gb_or = oracle.scan_bwd_bf16(a_bits, bits(h), d_bits, fused=True)
+    for name, got, want in (("h", bits(h), h_or), ("grad_beta", bits(gb), gb_or), ("grad_alpha", bits(ga), ga_or)):
+        if exact:
+            np.testing.assert_array_equal(got, want, err_msg=f"{what} {name}")
+        else:
+            finite = np.isfinite(oracle.bf16_bits_to_f32(want))
+            dist = ulp_distance(got[finite], want[finite])
+            # re-associated carries may move a value across a rounding boundary, or - where
+            # the result nearly cancels - by a few ulps of a much smaller number
+            close = np.abs(oracle.bf16_bits_to_f32(got[finite]) - oracle.bf16_bits_to_f32(want[finite])) <= 1e-3
+            assert ((dist <= max_ulp) | close).all(), f"{what} {name}: max ulp distance {dist.max()}"
+    return h, ga, gb
+
+
+# ------------------------------------------------------------------ small shapes
+
+
+@pytest.mark.parametrize("seq", [1, 2, 3, 7, 8])
+@pytest.mark.parametrize("d", [1, 2, 6, 64, 100, 136, 520])
+def test_bf16_one_wave_is_bit_exact(oracle, seq, d):
+    """seq <= steps with one wave: no re-association anywhere -> identical bits."""
+    alpha, beta, dout = make_inputs("normal", 3, seq, d, seed=seq * 1000 + d)
+    vec = 8 if d % 8 == 0 else 4 if d % 4 == 0 else 2 if d % 2 == 0 else 1
+    for v in {1, vec, min(vec, 2)}:
+        check_bf16(oracle, alpha, beta, dout, config=(v, 8, 1), exact=True, what=f"v{v}")
+    check_bf16(oracle, alpha, beta, dout, config=None, exact=True, what="default")
+
+
+@pytest.mark.parametrize("seq", [9, 31, 64, 65, 257, 1000])
+@pytest.mark.parametrize("d", [2, 24, 128, 192, 768])
+@pytest.mark.parametrize("recipe", ["normal", "sigmoid"])
+def test_bf16_default_config(oracle, recipe, seq, d):
+    alpha, beta, dout = make_inputs(recipe, 2, seq, d, seed=seq + d)
+    check_bf16(oracle, alpha, beta, dout, what=f"{recipe} {seq}x{d}")
+
+
+CONFIGS = [
+    (1, 8, 1), (1, 16, 3), (1, 32, 16),
+    (2, 8, 2), (2, 16, 8), (2, 32, 4), (2, 32, 16),
+    (4, 8, 5), (4, 16, 8), (4, 8, 16),
+    (8, 8, 1), (8, 8, 8),
+]
+
+
+@pytest.mark.parametrize("config", CONFIGS, ids=lambda c: "v%d_s%d_w%d" % c)
+def test_bf16_result_does_not_depend_on_chunking(oracle, config):
+    """Same inputs through every tiling: many chunks, ragged tails, partial column tiles."""
+    alpha, beta, dout = make_inputs("hawk", 2, 777, 328, seed=7)  # 328 = 8*41: partial tiles for every vec
+    check_bf16(oracle, alpha, beta, dout, config=config, what=str(config))
+
+
+@pytest.mark.parametrize("config", [(1, 8, 4), (2, 8, 16), (2, 16, 2), (4, 8, 8), (1, 32, 1)],
+                         ids=lambda c: "v%d_s%d_w%d" % c)
+def test_f32_chunking(oracle, config):
+    alpha, beta, dout = make_inputs("sigmoid", 3, 515, 204, dtype=torch.float32, seed=11)
+    a, b, do = alpha.to(DEV), beta.to(DEV), dout.to(DEV)
+    h = ext._forward(torch.float32, a, b, config)
+    ga, gb = ext._backward(torch.float32, a, h, do, config)
+    h_or = oracle.scan_fwd_f32(alpha.numpy(), beta.numpy(), fused=True)
+    ga_or, gb_or = oracle.scan_bwd_f32(alpha.numpy(), h.cpu().numpy(), dout.numpy(), fused=True)
+    assert rel_l2(h.cpu().numpy(), h_or) < 1e-6
+    assert rel_l2(gb.cpu().numpy(), gb_or) < 1e-6
+    assert rel_l2(ga.cpu().numpy(), ga_or) < 1e-6
+    np.testing.assert_allclose(h.cpu().numpy(), h_or, rtol=1e-4, atol=1e-5)
+    np.testing.assert_allclose(gb.cpu().numpy(), gb_or, rtol=1e-4, atol=1e-5)
+    np.testing.assert_allclose(ga.cpu().numpy(), ga_or, rtol=1e-4, atol=1e-5)
+
+
+def test_f32_one_wave_bit_exact(oracle):
+    alpha, beta, dout = make_inputs("normal", 2, 8, 100, dtype=torch.float32, seed=3)
+    a, b, do = alpha.to(DEV), beta.to(DEV), dout.to(DEV)
+    h = ext._forward(torch.float32, a, b, (1, 8, 1))
+    ga, gb = ext._backward(torch.float32, a, h, do, (1, 8, 1))
+    np.testing.assert_array_equal(h.cpu().numpy(), oracle.scan_fwd_f32(alpha.numpy(), beta.numpy(), fused=True))
+    ga_or, gb_or = oracle.scan_bwd_f32(alpha.numpy(), h.cpu().numpy(), dout.numpy(), fused=True)
+    np.testing.assert_array_equal(gb.cpu().numpy(), gb_or)
+    np.testing.assert_array_equal(ga.cpu().numpy(), ga_or)
+
+
+# ------------------------------------------------- the measured configurations
+
+
+@pytest.mark.parametrize("case", list(BASELINE_CASES), ids=list(BASELINE_CASES))
+def test_baseline_configs_full_size(oracle, case):
+    recipe, bs, seq, d = BASELINE_CASES[case]
+    alpha, beta, dout = make_inputs(recipe, bs, seq, d)
+    # N(0,1) alphas exceed 1 a third of the time: a product of a few of them can
+    # amplify the fp32 rounding of a re-associated carry, so allow more ulps there
+    check_bf16(oracle, alpha, beta, dout, max_ulp=2 if recipe != "normal" else 4, what=case)
+    ext.workspace_status()
+
+
+def test_closed_forms_at_headline_shape():
+    """Size-independent properties at the full headline size (bs 8, seq 4096, d 1024)."""
+    bs, seq, d = 8, 4096, 1024
+    beta = torch.randn(bs, seq, d, generator=torch.Generator().manual_seed(5)).to(torch.bfloat16).to(DEV)
+    zeros = torch.zeros_like(beta)
+    # alpha == 0 -> h == beta exactly
+    h = ext.scan_forward_half(zeros, beta)
+    assert torch.equal(h, beta)
+    # linearity in beta for fixed alpha: scan(a, 2b) == 2 scan(a, b) exactly (power of two)
+    alpha = torch.sigmoid(torch.randn(bs, seq, d, generator=torch.Generator().manual_seed(6))).to(torch.bfloat16).to(DEV)
+    h1 = ext.scan_forward_half(alpha, beta)
+    h2 = ext.scan_forward_half(alpha, beta * 2)
+    assert torch.equal(h2.float(), h1.float() * 2)
+    # alpha == 1, beta == 1/64: h[t] = (t+1)/64, exact in fp32, compare after bf16 rounding
+    ones = torch.ones_like(beta)
+    small = torch.full_like(beta, 1.0 / 64)
+    h = ext.scan_forward_half(ones, small)
+    expect = ((torch.arange(seq, device=DEV, dtype=torch.float32) + 1) / 64).to(torch.bfloat16)
+    assert torch.equal(h, expect[None, :, None].expand_as(h))
+    # backward with dout == 0 -> both grads exactly zero; with alpha == 0 -> grad_beta == dout
+    ga, gb = ext.scan_backward_half(alpha, h1, zeros)
+    assert not ga.any() and not gb.any()
+    ga, gb = ext.scan_backward_half(zeros, h1, beta)
+    assert torch.equal(gb, beta)
+    assert torch.equal(ga[:, 1:].float(), (beta[:, 1:].float() * h1[:, :-1].float()).to(torch.bfloat16).float())
+    assert not ga[:, 0].any()
+    ext.workspace_status()
+
+
+# -------------------------------------------------------------------- edge cases
+
+
+def test_alpha_row_zero_is_never_used(oracle):
+    alpha, beta, dout = make_inputs("sigmoid", 2, 300, 64, seed=21)
+    h0, ga0, gb0 = run_bf16(alpha, beta, dout)
+    alpha2 = alpha.clone()
+    alpha2[:, 0, :] = float("nan")
+    h1, ga1, gb1 = run_bf16(alpha2, beta, dout)
+    assert torch.equal(h0, h1) and torch.equal(gb0, gb1) and torch.equal(ga0, ga1)
+    assert not ga1[:, 0].any()
+
+
+def test_empty_tensors():
+    for shape in [(0, 5, 8), (2, 0, 8), (2, 5, 0)]:
+        a = torch.empty(shape, dtype=torch.bfloat16, device=DEV)
+        h = ext.scan_forward_half(a, a)
+        assert h.shape == a.shape
+        ga, gb = ext.scan_backward_half(a, h, a)
+        assert ga.shape == a.shape and gb.shape == a.shape
+
+
+def test_non_contiguous_and_offset_inputs(oracle):
+    alpha, beta, dout = make_inputs("sigmoid", 2, 130, 70, seed=31)
+    # time-major storage viewed as (bs, seq, d): not contiguous
+    a_nc = alpha.to(DEV).transpose(0, 1).contiguous().transpose(0, 1)
+    b_nc = beta.to(DEV).transpose(0, 1).contiguous().transpose(0, 1)
+    assert not a_nc.is_contiguous()
+    h = ext.scan_forward_half(a_nc, b_nc)
+    h_ref = ext.scan_forward_half(alpha.to(DEV), beta.to(DEV))
+    assert torch.equal(h, h_ref)
+    # a contiguous view that starts 2 bytes into its storage: only element alignment
+    flat = torch.empty(alpha.numel() + 1, dtype=torch.bfloat16, device=DEV)
+    a_off = flat[1:].view(alpha.shape)
+    a_off.copy_(alpha)
+    assert a_off.data_ptr() % 4 == 2
+    h_off = ext.scan_forward_half(a_off, beta.to(DEV))
+    assert torch.equal(h_off, h_ref)
+    ga, gb = ext.scan_backward_half(a_off, h_ref, dout.to(DEV))
+    ga_ref, gb_ref = ext.scan_backward_half(alpha.to(DEV), h_ref, dout.to(DEV))
+    assert torch.equal(ga, ga_ref) and torch.equal(gb, gb_ref)
+
+
+def test_non_default_stream_and_back_to_back_launches(oracle):
+    alpha, beta, dout = make_inputs("sigmoid", 4, 2000, 256, seed=41)
+    a, b, do = alpha.to(DEV), beta.to(DEV), dout.to(DEV)
+    h_ref, ga_ref, gb_ref = run_bf16(alpha, beta, dout)
+    s = torch.cuda.Stream()
+    s.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(s):
+        outs = []
+        for _ in range(20):  # back-to-back chained launches reuse one workspace
+            h = ext.scan_forward_half(a, b)
+            ga, gb = ext.scan_backward_half(a, h, do)
+            outs.append((h, ga, gb))
+        ext.workspace_status()
+    s.synchronize()
+    for h, ga, gb in outs:
+        assert torch.equal(h, h_ref) and torch.equal(ga, ga_ref) and torch.equal(gb, gb_ref)
+
+
+# ----------------------------------------------------- the public autograd API
+
+
+def test_scan_cu_autograd_matches_oracle(oracle):
+    alpha, beta, dout = make_inputs("sigmoid", 3, 600, 512, seed=51)
+    a = alpha.to(DEV).requires_grad_(True)
+    b = beta.to(DEV).requires_grad_(True)
+    out = scan_cu(a, b)
+    out.backward(dout.to(DEV), retain_graph=True)
+    h32 = oracle.scan_fwd_bf16_f32out(bits(alpha), bits(beta))
+    ga32, gb32 = oracle.scan_bwd_bf16_f32out(bits(alpha), h32, bits(dout))
+    assert_close_f32(out, h32, "h")
+    assert_close_f32(a.grad, ga32, "grad_alpha")
+    assert_close_f32(b.grad, gb32, "grad_beta")
+    # a second backward works: the forward output is not overwritten by the first
+    # (the reference aliases grad_beta onto it: csrc/sequential_scan_kernel.cu:197)
+    first = (a.grad.clone(), b.grad.clone())
+    a.grad = b.grad = None
+    out.backward(dout.to(DEV))
+    assert torch.equal(a.grad, first[0]) and torch.equal(b.grad, first[1])
+    assert_close_f32(out, h32, "h after two backwards")
+
+
+def test_scan_cu_under_autocast_casts_to_bf16(oracle):
+    alpha, beta, _ = make_inputs("sigmoid", 2, 100, 64, dtype=torch.float32, seed=61)
+    with torch.autocast("cuda", dtype=torch.bfloat16):
+        out = scan_cu(alpha.to(DEV), beta.to(DEV))
+    assert out.dtype == torch.bfloat16
+    want = oracle.scan_fwd_bf16(bits(alpha.to(torch.bfloat16)), bits(beta.to(torch.bfloat16)), fused=True)
+    assert (ulp_distance(bits(out), want) <= 2).all()
+    with pytest.raises(RuntimeError):  # outside autocast fp32 input is a dtype error, as in the reference
+        scan_cu(alpha.to(DEV), beta.to(DEV))
+
+
+@pytest.mark.parametrize("bs,sq,d", [(9, 128, 512), (2, 1024, 768), (12, 256, 1024)])
+def test_reference_test_matrix_fp32(oracle, bs, sq, d):
+    """The reference's own fp32 test (sequential_scan/test_scan_cuda.py:27-72): N(0,1)
+    inputs, relative L2 error below 1e-6 for the output and both gradients."""
+    g = torch.Generator().manual_seed(0)
+    alpha = torch.randn(bs, sq, d, generator=g)
+    beta = torch.randn(bs, sq, d, generator=g)
+    dy = torch.randn(bs, sq, d, generator=g)
+    a = alpha.to(DEV).requires_grad_(True)
+    b = beta.to(DEV).requires_grad_(True)
+    out = scan_cu_single(a, b)
+    out.backward(dy.to(DEV))
+    h = oracle.scan_fwd_f32(alpha.numpy(), beta.numpy())
+    ga, gb = oracle.scan_bwd_f32(alpha.numpy(), h, dy.numpy())
+    assert rel_l2(out.detach().cpu().numpy(), h) < 1e-6
+    assert rel_l2(a.grad.cpu().numpy(), ga) < 1e-6
+    assert rel_l2(b.grad.cpu().numpy(), gb) < 1e-6
+
+
+@pytest.mark.parametrize("bs,sq,d", [(5, 128, 512), (13, 512, 768), (3, 1024, 1024)])
+def test_reference_test_matrix_bf16(oracle, bs, sq, d):
+    """The reference's bf16 test (test_scan_cuda.py:80-124): relative L2 error below 0.1
+    against the scan evaluated in bf16 arithmetic; here against the fp32-accumulated one."""
+    alpha, beta, dy = make_inputs("normal", bs, sq, d, seed=71)
+    a = alpha.to(DEV).requires_grad_(True)
+    b = beta.to(DEV).requires_grad_(True)
+    out = scan_cu(a, b)
+    out.backward(dy.to(DEV))
+    h32 = oracle.scan_fwd_bf16_f32out(bits(alpha), bits(beta))
+    ga32, gb32 = oracle.scan_bwd_bf16_f32out(bits(alpha), h32, bits(dy))
+    assert rel_l2(out.detach().float().cpu().numpy(), h32) < 1e-2
+    assert rel_l2(a.grad.float().cpu().numpy(), ga32) < 1e-2
+    assert rel_l2(b.grad.float().cpu().numpy(), gb32) < 1e-2
+
+
+def test_c_abi_rejects_bad_arguments():
+    lib = _native.lib()
+    a = torch.zeros(2, 300, 64, dtype=torch.bfloat16, device=DEV)
+    s = torch.cuda.current_stream().cuda_stream
+    assert lib.fss_scan_fwd_bf16(None, a.data_ptr(), a.data_ptr(), 2, 300, 64, None, 0, s) == 1
+    assert lib.fss_scan_fwd_bf16(a.data_ptr(), a.data_ptr(), a.data_ptr(), -1, 300, 64, None, 0, s) == 2
+    # 300 steps need more than one chunk here -> a workspace is required
+    cfg = _native.FssConfig(2, 8, 2, 0)
+    import ctypes
+    assert lib.fss_scan_fwd_ex(0, a.data_ptr(), a.data_ptr(), a.data_ptr(), 2, 300, 64, None, 0, s, ctypes.byref(cfg)) == 4
+    bad = _native.FssConfig(3, 8, 2, 0)
+    assert lib.fss_scan_fwd_ex(0, a.data_ptr(), a.data_ptr(), a.data_ptr(), 2, 300, 64, None, 0, s, ctypes.byref(bad)) == 5
+    odd = _native.FssConfig(2, 8, 1, 0)  # vec 2 needs 4-byte alignment
+    assert lib.fss_scan_fwd_ex(0, a.data_ptr() + 2, a.data_ptr(), a.data_ptr(), 1, 8, 64, None, 0, s, ctypes.byref(odd)) == 3
+    torch.cuda.synchronize()
