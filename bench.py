@@ -1,0 +1,290 @@
+"""Benchmark of the bf16 scan, forward + backward, on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--case C3_4096] [--config V,S,W]
+
+One "step" is one forward scan plus one backward scan over one batch of
+synthetic input, launched through the C ABI on torch's current stream with all
+tensors already resident in HBM.  Prints ONE JSON line:
+
+  value            algorithmic GB/s of the whole step: 16 B per element (forward reads
+                   alpha, beta and writes h = 6 B; backward reads alpha, h, dout and
+                   writes grad_alpha, grad_beta = 10 B) divided by the wall time per step
+  roofline         the dominant kernel (the backward scan, 10 of the 16 B): its
+                   algorithmic bytes per launch over its mean duration, measured with
+                   HIP events recorded around every launch inside the timed region
+  cpu_baseline     the reference's PyTorch sequential loop (oracle/torch_loop.py) on the
+                   host cores, same inputs, fp32; also the parity check of this run
+"""
+from __future__ import annotations
+
+import argparse
+import ctypes
+import json
+import os
+import statistics
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBPS = 8000.0
+FWD_BYTES_PER_ELEM = 6
+BWD_BYTES_PER_ELEM = 10
+
+
+def parse_args():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=25)
+    ap.add_argument("--case", default="C3_4096", help="workload name from fast_sequential_scan_amd.workloads")
+    ap.add_argument("--config", default=None, help="explicit vec,steps,waves for both kernels (tuning)")
+    ap.add_argument("--fwd-config", default=None)
+    ap.add_argument("--bwd-config", default=None)
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline / parity leg")
+    ap.add_argument("--cpu-seconds", type=float, default=12.0, help="budget of the CPU baseline leg")
+    ap.add_argument("--flush-mb", type=int, default=1024, help="size of the cache-flush write for the cold timings")
+    return ap.parse_args()
+
+
+def main() -> int:
+    args = parse_args()
+    if args.gpus != 1:
+        print(
+            "bench.py measures one GPU: channels are independent, so more GPUs would each run this "
+            "same kernel on a slice of bs or d with no communication; run with --gpus 1",
+            file=sys.stderr,
+        )
+        return 2
+
+    import torch
+
+    from fast_sequential_scan_amd import _native, scan_cu
+    from fast_sequential_scan_amd import sequential_scan_cuda as ext
+    from fast_sequential_scan_amd.workloads import BASELINE_CASES, make_inputs
+
+    lib = _native.lib()  # no fallback: a missing HIP library is an error
+    if not torch.cuda.is_available():
+        print("bench.py needs a GPU", file=sys.stderr)
+        return 2
+    dev = torch.device("cuda", 0)
+    torch.cuda.set_device(dev)
+
+    recipe, bs, seq, d = BASELINE_CASES[args.case]
+    n_elem = bs * seq * d
+    alpha_c, beta_c, dout_c = make_inputs(recipe, bs, seq, d)
+    alpha, beta, dout = alpha_c.to(dev), beta_c.to(dev), dout_c.to(dev)
+    h = torch.empty_like(alpha)
+    galpha = torch.empty_like(alpha)
+    gbeta = torch.empty_like(alpha)
+
+    def cfg_of(text):
+        return tuple(int(x) for x in text.split(",")) if text else None
+
+    fwd_cfg = cfg_of(args.fwd_config or args.config)
+    bwd_cfg = cfg_of(args.bwd_config or args.config)
+    fwd_cfg_p, bwd_cfg_p = _native.make_config(fwd_cfg), _native.make_config(bwd_cfg)
+
+    stream = torch.cuda.current_stream()
+    sp = stream.cuda_stream
+    ws_bytes = max(
+        lib.fss_workspace_bytes(bs, seq, d, _native.FSS_BF16, _native.FSS_FWD, fwd_cfg_p),
+        lib.fss_workspace_bytes(bs, seq, d, _native.FSS_BF16, _native.FSS_BWD, bwd_cfg_p),
+    )
+    ws = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
+    _native.check(lib.fss_workspace_init(ws.data_ptr(), ws.numel(), sp))
+    pa, pb, pd, ph, pga, pgb, pws = (t.data_ptr() for t in (alpha, beta, dout, h, galpha, gbeta, ws))
+
+    def fwd():
+        rc = lib.fss_scan_fwd_ex(_native.FSS_BF16, pa, pb, ph, bs, seq, d, pws, ws_bytes, sp, fwd_cfg_p)
+        if rc:
+            _native.check(rc)
+
+    def bwd():
+        rc = lib.fss_scan_bwd_ex(_native.FSS_BF16, pa, ph, pd, pga, pgb, bs, seq, d, pws, ws_bytes, sp, bwd_cfg_p)
+        if rc:
+            _native.check(rc)
+
+    chosen = {}
+    for name, direction, user in (("fwd", _native.FSS_FWD, fwd_cfg), ("bwd", _native.FSS_BWD, bwd_cfg)):
+        c = _native.FssConfig()
+        lib.fss_choose_config(bs, seq, d, _native.FSS_BF16, direction, 16, ctypes.byref(c))
+        chosen[name] = list(user) if user else [c.vec, c.steps, c.waves]
+
+    # ---- warm-up, then the timed region: exactly K steps between two synchronisations ----
+    for _ in range(args.warmup):
+        fwd()
+        bwd()
+    K = args.steps
+    ev = [[torch.cuda.Event(enable_timing=True) for _ in range(3)] for _ in range(K)]
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for k in range(K):
+        ev[k][0].record(stream)
+        fwd()
+        ev[k][1].record(stream)
+        bwd()
+        ev[k][2].record(stream)
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    _native.check(lib.fss_workspace_status(pws, sp))
+
+    ms_per_step = wall * 1e3 / K
+    fwd_ms = [ev[k][0].elapsed_time(ev[k][1]) for k in range(K)]
+    bwd_ms = [ev[k][1].elapsed_time(ev[k][2]) for k in range(K)]
+    fwd_mean, bwd_mean = statistics.fmean(fwd_ms), statistics.fmean(bwd_ms)
+    step_bytes = (FWD_BYTES_PER_ELEM + BWD_BYTES_PER_ELEM) * n_elem
+    value = step_bytes / (ms_per_step * 1e-3) / 1e9
+    bwd_gbps = BWD_BYTES_PER_ELEM * n_elem / (bwd_mean * 1e-3) / 1e9
+    fwd_gbps = FWD_BYTES_PER_ELEM * n_elem / (fwd_mean * 1e-3) / 1e9
+
+    # ---- cold timings: reading a large buffer between launches evicts L2 and the memory-side
+    # cache and leaves them clean (a large write would leave dirty lines whose write-back is then
+    # charged to the kernel under test) ----
+    cold = {}
+    if args.flush_mb > 0:
+        junk = torch.zeros(args.flush_mb << 18, dtype=torch.int32, device=dev)
+        torch.cuda.synchronize()
+        e = [torch.cuda.Event(enable_timing=True) for _ in range(4)]
+        cf, cb = [], []
+        for _ in range(10):
+            junk.sum()
+            e[0].record(stream)
+            fwd()
+            e[1].record(stream)
+            junk.sum()
+            e[2].record(stream)
+            bwd()
+            e[3].record(stream)
+            torch.cuda.synchronize()
+            cf.append(e[0].elapsed_time(e[1]))
+            cb.append(e[2].elapsed_time(e[3]))
+        cold = {
+            "fwd_ms": round(statistics.median(cf), 5),
+            "bwd_ms": round(statistics.median(cb), 5),
+            "fwd_GBps": round(FWD_BYTES_PER_ELEM * n_elem / (statistics.median(cf) * 1e-3) / 1e9, 1),
+            "bwd_GBps": round(BWD_BYTES_PER_ELEM * n_elem / (statistics.median(cb) * 1e-3) / 1e9, 1),
+            "flush_MB": args.flush_mb,
+        }
+        del junk
+
+    # ---- the public autograd path (allocates its outputs, goes through torch.autograd) ----
+    a_req = alpha.detach().clone().requires_grad_(True)
+    b_req = beta.detach().clone().requires_grad_(True)
+    for _ in range(5):
+        scan_cu(a_req, b_req).backward(dout)
+        a_req.grad = b_req.grad = None
+    torch.cuda.synchronize()
+    n_auto = max(10, K // 4)
+    t0 = time.perf_counter()
+    for _ in range(n_auto):
+        scan_cu(a_req, b_req).backward(dout)
+        a_req.grad = b_req.grad = None
+    torch.cuda.synchronize()
+    autograd_ms = (time.perf_counter() - t0) * 1e3 / n_auto
+
+    # ---- CPU baseline + parity of this very run ----
+    cpu = None
+    parity = None
+    if not args.no_cpu:
+        from oracle.torch_loop import torch_loop_bwd, torch_loop_fwd
+
+        fwd()
+        bwd()
+        torch.cuda.synchronize()
+        h_gpu, ga_gpu, gb_gpu = h.float().cpu(), galpha.float().cpu(), gbeta.float().cpu()
+        reps, spent = 0, 0.0
+        f_times, b_times = [], []
+        while reps < 1 or (spent < args.cpu_seconds and reps < 20):
+            t0 = time.perf_counter()
+            h_ref = torch_loop_fwd(alpha_c, beta_c)
+            t1 = time.perf_counter()
+            ga_ref, gb_ref = torch_loop_bwd(alpha_c, h_ref, dout_c)
+            t2 = time.perf_counter()
+            f_times.append(t1 - t0)
+            b_times.append(t2 - t1)
+            spent += t2 - t0
+            reps += 1
+        cpu_step = statistics.median(f_times) + statistics.median(b_times)
+
+        def ok(got, want):
+            return bool(((got - want).abs() <= 1e-2 + 1e-2 * want.abs()).all())
+
+        parity = {
+            "h": ok(h_gpu, h_ref), "grad_alpha": ok(ga_gpu, ga_ref), "grad_beta": ok(gb_gpu, gb_ref),
+            "rtol": 1e-2, "atol": 1e-2, "against": "fp32 sequential loop on the CPU, same bf16 inputs",
+        }
+        cpu = {
+            "value": round(step_bytes / cpu_step / 1e9, 3),
+            "unit": "GB/s",
+            "cores": torch.get_num_threads(),
+            "kind": "port",
+            "sample": f"the full workload ({args.case}: bs{bs} seq{seq} d{d}), fwd+bwd, median of {reps} run(s)",
+            "ms_per_step": round(cpu_step * 1e3, 2),
+            "fwd_ms": round(statistics.median(f_times) * 1e3, 2),
+            "bwd_ms": round(statistics.median(b_times) * 1e3, 2),
+            "host_cpus": os.cpu_count(),
+            "impl": "oracle/torch_loop.py: PyTorch loop over seq on CPU tensors, fp32",
+        }
+
+    out = {
+        "metric": "fwd+bwd scan ms & achieved HBM GB/s (% peak), bf16 bs8 d1024 seq4096"
+        if args.case == "C3_4096" else f"fwd+bwd scan ms & achieved HBM GB/s (% peak), bf16 {args.case}",
+        "value": round(value, 1),
+        "unit": "GB/s",
+        "n_gpus": 1,
+        "steps": K,
+        "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 5),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "bf16",
+        "data": "synthetic",
+        "config": {
+            "workload": f"{args.case}: bs{bs} seq{seq} d{d}, recipe {recipe}, bf16 storage / fp32 carries, forward+backward",
+            "bs": bs, "seq": seq, "d_model": d,
+            "launch_config_fwd_vec_steps_waves": chosen["fwd"],
+            "launch_config_bwd_vec_steps_waves": chosen["bwd"],
+        },
+        "pct_of_hbm_peak": round(100.0 * value / HBM_PEAK_GBPS, 2),
+        "fwd_ms": round(fwd_mean, 5),
+        "bwd_ms": round(bwd_mean, 5),
+        "fwd_ms_median": round(statistics.median(fwd_ms), 5),
+        "bwd_ms_median": round(statistics.median(bwd_ms), 5),
+        "algorithmic_bytes_per_step": step_bytes,
+        "roofline": {
+            "bound": "hbm",
+            "kernel": "scan_kernel<BF16,...,BWD=true> (backward scan)",
+            "achieved": round(bwd_gbps, 1),
+            "peak": HBM_PEAK_GBPS,
+            "unit": "GB/s",
+            "frac": round(bwd_gbps / HBM_PEAK_GBPS, 4),
+            "traffic": None,
+            "bytes_per_launch": BWD_BYTES_PER_ELEM * n_elem,
+            "avg_launch_ms": round(bwd_mean, 5),
+        },
+        "roofline_fwd": {
+            "bound": "hbm",
+            "kernel": "scan_kernel<BF16,...,BWD=false> (forward scan)",
+            "achieved": round(fwd_gbps, 1),
+            "peak": HBM_PEAK_GBPS,
+            "unit": "GB/s",
+            "frac": round(fwd_gbps / HBM_PEAK_GBPS, 4),
+            "traffic": None,
+            "bytes_per_launch": FWD_BYTES_PER_ELEM * n_elem,
+            "avg_launch_ms": round(fwd_mean, 5),
+        },
+        "cold_cache": cold,
+        "autograd_path_ms_per_step": round(autograd_ms, 5),
+        "parity": parity,
+        "cpu_baseline": cpu,
+    }
+    print(json.dumps(out))
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

@@ -23,11 +23,13 @@
 //     1. every lane issues all its loads at once (STEPS rows x 2 or 3 tensors:
 //        the memory-level parallelism that fills HBM), then folds its slice into
 //        the affine map x -> A*x + B it applies to the incoming state;
-//     2. wave 0 composes the waves' maps through LDS, publishes the chunk's map,
-//        obtains the chunk's incoming state by looking back over earlier chunks
-//        of the same channels (decoupled look-back over (A,B) pairs in global
-//        memory), publishes the outgoing state, and hands every wave its own
-//        incoming state through LDS;
+//     2. wave 0 composes the waves' maps through LDS and publishes the chunk's map;
+//        at the same time up to 8 waves each fetch what one earlier chunk of the
+//        same channels offers (its outgoing state if it has one, else its map),
+//        so the look-back over the nearest chunks costs one memory round trip, not
+//        one per chunk (decoupled look-back over (A,B) pairs in global memory).
+//        Wave 0 folds what they found into the chunk's incoming state, publishes
+//        the outgoing state, and hands every wave its own incoming state via LDS;
 //     3. every lane re-runs the recurrence over its register-resident slice from
 //        its true incoming state, in sequential order, and stores the results.
 //   Because phase 3 restarts from the incoming state, only that state is
@@ -35,19 +37,21 @@
 //   exactly the sequential one.
 //
 // Chaining across workgroups
-//   Tiles take a ticket from an atomic counter and the ticket fixes the tile:
-//   chunk-major, so every tile a workgroup may wait for holds a smaller ticket
-//   and is therefore already resident or finished - the wait cannot deadlock
-//   whatever order the hardware dispatches workgroups in.  State handed between
-//   chunks travels as 64-bit words {tag, fp32} written and read with relaxed
-//   agent-scope atomics; value and validity arrive together, so no fence is
-//   needed.  The tag is a per-workspace launch counter ("epoch", never 0), so
-//   words never need clearing; the last workgroup to finish its look-back resets
-//   the ticket counter and advances the epoch for the next launch.  The counter
-//   wraps after 2^32-1 launches; a host that can get there re-initialises the
-//   workspace first.  Every wait is
-//   bounded: a lane that exhausts its budget records an error in the workspace
-//   header and carries on with a zero state, so the grid always drains.
+//   The grid is persistent: it holds no more workgroups than the device keeps
+//   resident at once, and each walks tiles blockIdx, blockIdx+gridDim, ... in
+//   chunk-major order.  A tile only waits for lower-numbered tiles, each owned by
+//   a resident workgroup that reaches it no later than the waiter reaches its
+//   own, so the waits cannot deadlock - and no atomic ticket serialises the
+//   start of the workgroups.  State handed between chunks travels as 64-bit
+//   words {tag, fp32} written and read with relaxed agent-scope atomics; value
+//   and validity arrive together, so no fence is needed.  The tag is a
+//   per-workspace launch counter ("epoch", never 0), so words never need
+//   clearing; workgroups count themselves out at the end (two-level counter) and
+//   the last one advances the epoch for the next launch.  The counter wraps
+//   after 2^32-1 launches; a host that can get there re-initialises the
+//   workspace first.  Every wait is bounded: a wave that exhausts its budget
+//   records an error in the workspace header and carries on with a zero state,
+//   so the grid always drains.
 //
 // The backward runs the same machine over reversed time r = seq-1-t with
 // a'[r] = alpha[t+1], b'[r] = dout[t], plus the elementwise g[t]*h[t-1].
@@ -75,6 +79,17 @@ struct F32 {
 
 __device__ __forceinline__ float as_f32(uint32_t u) { return __builtin_bit_cast(float, u); }
 __device__ __forceinline__ uint32_t as_u32(float f) { return __builtin_bit_cast(uint32_t, f); }
+
+// Pins a wave-uniform pointer into scalar registers, so that `p + lane_offset`
+// becomes the scalar-base + 32-bit-vector-offset form of a global access and
+// costs no vector registers or 64-bit vector adds per row.
+template <typename P>
+__device__ __forceinline__ P *uniform_ptr(P *ptr) {
+  const uint64_t u = reinterpret_cast<uint64_t>(ptr);
+  const uint32_t lo = __builtin_amdgcn_readfirstlane(static_cast<uint32_t>(u));
+  const uint32_t hi = __builtin_amdgcn_readfirstlane(static_cast<uint32_t>(u >> 32));
+  return reinterpret_cast<P *>((static_cast<uint64_t>(hi) << 32) | lo);
+}
 
 // Loads/stores of N dwords per lane.
 template <int N>
@@ -184,19 +199,40 @@ struct Row<F32, VEC> {
   }
 };
 
-// ---- workspace ----------------------------------------------------------------
+// Makes the compiler forget what it derived from a packed row: the rows stay
+// packed in registers across the chaining phase and are unpacked again after
+// it, instead of keeping an fp32 copy of every element alive next to them.
+template <typename RowT>
+__device__ __forceinline__ void keep_packed(RowT &r) {
+#pragma unroll
+  for (int i = 0; i < RowT::kDwords; ++i) asm volatile("" : "+v"(r.dw[i]));
+}
 
-enum : int { HDR_TICKET = 0, HDR_DONE = 1, HDR_EPOCH = 2, HDR_ERROR = 3 };
-constexpr size_t kHeaderBytes = 256;
-// Polls a lane makes before it gives up on a predecessor (each poll is a memory
+// ---- workspace ----------------------------------------------------------------
+//
+// Header (kHeaderBytes): word 1 = top-level completion counter, word 2 = epoch,
+// word 3 = sticky error flag, words 64+32*i (i < 16, one 128-byte line each) =
+// first-level completion counters.  Then the tagged words,
+// [chunk][column tile][kind: map A, map B, outgoing state][VEC][64 lanes].
+
+enum : int { HDR_DONE = 1, HDR_EPOCH = 2, HDR_ERROR = 3, HDR_SLOT0 = 64, HDR_SLOT_STRIDE = 32 };
+constexpr int kDoneSlots = 16;
+constexpr size_t kHeaderBytes = 4096;
+// Polls a wave makes before it gives up on an earlier chunk (each poll is a memory
 // round trip plus a sleep: seconds in total, far beyond any healthy wait).
 constexpr uint32_t kSpinLimit = 1u << 20;
+// Most waves of a workgroup that look back in parallel, one earlier chunk each.
+constexpr int kMaxLookWaves = 16;
+enum : uint32_t { kPredNone = 0, kPredMap = 1, kPredState = 2 };
 
 __device__ __forceinline__ uint32_t ld_u32(const uint32_t *p) {
   return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 __device__ __forceinline__ void st_u32(uint32_t *p, uint32_t v) {
   __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ uint32_t add_u32(uint32_t *p, uint32_t v) {
+  return __hip_atomic_fetch_add(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 __device__ __forceinline__ uint64_t ld_word(const uint64_t *p) {
   return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -219,8 +255,10 @@ struct ScanArgs {
   int32_t tiles_per_row;  // ceil(d / (64*VEC))
   int32_t n_ctiles;       // bs * tiles_per_row
   int32_t n_chunks;       // ceil(seq / (WAVES*STEPS))
-  uint32_t *hdr;          // workspace header (4 words used)
-  uint64_t *words;        // [chunk][ctile][3][VEC][64] tagged words: A, B, outgoing state
+  int32_t n_tiles;        // n_ctiles * n_chunks
+  int32_t look_waves;     // waves that look back in parallel (1..min(WAVES, kMaxLookWaves))
+  uint32_t *hdr;          // workspace header
+  uint64_t *words;        // tagged words
 };
 
 // ---- the kernel ----------------------------------------------------------------
@@ -232,279 +270,340 @@ __global__ __launch_bounds__(1024) void scan_kernel(const ScanArgs p) {
   constexpr int kLaneSlots = 64 * VEC;  // channels per tile
 
   extern __shared__ float lds[];
-  __shared__ uint32_t s_ticket, s_epoch;
+  __shared__ uint32_t s_kind[kMaxLookWaves];
+  __shared__ uint32_t s_resolved;
 
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int n_waves = blockDim.x >> 6;
-  float2 *lds_map = reinterpret_cast<float2 *>(lds);        // [wave][v][lane] = (A, B)
-  float *lds_in = lds + 2 * n_waves * kLaneSlots;           // [wave][v][lane] incoming state
+  const int look = p.look_waves;
+  float2 *lds_map = reinterpret_cast<float2 *>(lds);   // [wave][v][lane] = (A, B), later .x = incoming state
+  float2 *lds_pred = lds_map + n_waves * kLaneSlots;   // [look wave][v][lane] = what an earlier chunk offers
 
-  const bool chained = p.n_chunks > 1;
-  uint32_t tile = blockIdx.x;
-  uint32_t epoch = 0;
-  if (chained) {
-    if (threadIdx.x == 0) {
-      s_ticket = __hip_atomic_fetch_add(p.hdr + HDR_TICKET, 1u, __ATOMIC_RELAXED,
-                                        __HIP_MEMORY_SCOPE_AGENT);
-      s_epoch = ld_u32(p.hdr + HDR_EPOCH);
-    }
-    __syncthreads();
-    tile = s_ticket;
-    epoch = s_epoch;
+#ifdef FSS_RESIDENCY_PROBE
+  // debug build only: header words 8/9 = workgroups resident now / the most ever seen
+  if (threadIdx.x == 0 && p.hdr) {
+    const uint32_t now = add_u32(p.hdr + 8, 1u) + 1u;
+    __hip_atomic_fetch_max(p.hdr + 9, now, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   }
-  tile = __builtin_amdgcn_readfirstlane(tile);
-  const int chunk = tile / static_cast<uint32_t>(p.n_ctiles);
-  const int ctile = tile - chunk * p.n_ctiles;
-  const int batch = ctile / p.tiles_per_row;
-  const int coltile = ctile - batch * p.tiles_per_row;
+#endif
+  const bool chained = p.n_chunks > 1;
+  // every workgroup of a launch reads the same value: it only changes when all are done
+  const uint32_t tag = chained ? __builtin_amdgcn_readfirstlane(ld_u32(p.hdr + HDR_EPOCH)) : 0u;
 
   const int64_t seq = p.seq;
   const int64_t row_bytes = p.d * E::kBytes;
-  const int64_t col0 = static_cast<int64_t>(coltile) * kLaneSlots;  // first channel of the tile
-  const bool col_ok = col0 + lane * VEC < p.d;                       // d % VEC == 0 (host)
   const uint32_t lane_off = static_cast<uint32_t>(lane * kRowBytes);
-  // byte offset of (batch, row 0, col0); uniform over the wave
-  const int64_t tile_base = (static_cast<int64_t>(batch) * seq * p.d + col0) * E::kBytes;
-  // first scan-order index of this wave's slice (forward: r = t, backward: r = seq-1-t)
-  const int64_t r0 = (static_cast<int64_t>(chunk) * n_waves + wave) * STEPS;
 
-  // Fast path: every row this wave touches exists, is interior, and every lane
-  // has channels.  Forward touches rows r0..r0+STEPS-1 and must not be at r = 0;
-  // backward additionally reads row t+1 and t-1.
-  const bool full = (col0 + kLaneSlots <= p.d) && (r0 >= 1) &&
-                    (BWD ? (r0 + STEPS <= seq - 1) : (r0 + STEPS <= seq));
+  // The grid is sized to be resident all at once; each workgroup walks tiles
+  // blockIdx, blockIdx + gridDim, ...  Tiles are numbered chunk-major, so a tile
+  // only ever waits for tiles with smaller numbers: those belong to a resident
+  // workgroup that reaches them no later than this one reaches its own.
+  for (uint32_t tile = blockIdx.x; tile < static_cast<uint32_t>(p.n_tiles); tile += gridDim.x) {
+    // unsigned, wave-uniform arithmetic: stays on the scalar unit
+    const uint32_t uchunk = tile / static_cast<uint32_t>(p.n_ctiles);
+    const uint32_t uctile = tile - uchunk * static_cast<uint32_t>(p.n_ctiles);
+    const uint32_t batch = uctile / static_cast<uint32_t>(p.tiles_per_row);
+    const uint32_t coltile = uctile - batch * static_cast<uint32_t>(p.tiles_per_row);
+    const int chunk = static_cast<int>(uchunk);
+    const int ctile = static_cast<int>(uctile);
 
-  RowT a[STEPS], b[STEPS];
-  RowT hp[BWD ? STEPS : 1];
+    const int64_t col0 = static_cast<int64_t>(coltile) * kLaneSlots;  // first channel of the tile
+    const bool col_ok = col0 + lane * VEC < p.d;                       // d % VEC == 0 (host)
+    // byte offset of (batch, row 0, col0); uniform over the wave
+    const int64_t tile_base = (static_cast<int64_t>(batch) * seq * p.d + col0) * E::kBytes;
+    // first scan-order index of this wave's slice (forward: r = t, backward: r = seq-1-t)
+    const int64_t r0 = (static_cast<int64_t>(chunk) * n_waves + wave) * STEPS;
 
-  // ---- phase 1a: issue every load of the slice ----------------------------------
-  if (full) {
-    if (!BWD) {
-      const char *pa = p.in_a + tile_base + r0 * row_bytes;
-      const char *pb = p.in_b + tile_base + r0 * row_bytes;
+    // Fast path: every row this wave touches exists, is interior, and every lane
+    // has channels.  Forward touches rows r0..r0+STEPS-1 and must not be at r = 0;
+    // backward additionally reads row t+1 and t-1.
+    const bool full = (col0 + kLaneSlots <= p.d) && (r0 >= 1) &&
+                      (BWD ? (r0 + STEPS <= seq - 1) : (r0 + STEPS <= seq));
+
+    RowT a[STEPS], b[STEPS];
+    RowT hp[BWD ? STEPS : 1];
+
+    // ---- phase 1a: issue every load of the slice ----------------------------------
+    if (full) {
+      if (!BWD) {
+        const char *pa = p.in_a + tile_base + r0 * row_bytes;
+        const char *pb = p.in_b + tile_base + r0 * row_bytes;
 #pragma unroll
-      for (int s = 0; s < STEPS; ++s) {
-        a[s].load(pa + s * row_bytes + lane_off);
-        b[s].load(pb + s * row_bytes + lane_off);
+        for (int s = 0; s < STEPS; ++s) {
+          a[s].load(uniform_ptr(pa + s * row_bytes) + lane_off);
+          b[s].load(uniform_ptr(pb + s * row_bytes) + lane_off);
+        }
+      } else {
+        // t = seq-1-r: alpha row t+1, dout row t, h row t-1
+        const int64_t t0 = seq - 1 - r0;
+        const char *pa = p.in_a + tile_base + (t0 + 1) * row_bytes;
+        const char *pb = p.in_b + tile_base + t0 * row_bytes;
+        const char *ph = p.in_h + tile_base + (t0 - 1) * row_bytes;
+#pragma unroll
+        for (int s = 0; s < STEPS; ++s) {
+          a[s].load(uniform_ptr(pa - s * row_bytes) + lane_off);
+          b[s].load(uniform_ptr(pb - s * row_bytes) + lane_off);
+        }
+#pragma unroll
+        for (int s = 0; s < STEPS; ++s) hp[s].load(uniform_ptr(ph - s * row_bytes) + lane_off);
       }
     } else {
-      // t = seq-1-r: alpha row t+1, dout row t, h row t-1
-      const int64_t t0 = seq - 1 - r0;
-      const char *pa = p.in_a + tile_base + (t0 + 1) * row_bytes;
-      const char *pb = p.in_b + tile_base + t0 * row_bytes;
-      const char *ph = p.in_h + tile_base + (t0 - 1) * row_bytes;
 #pragma unroll
       for (int s = 0; s < STEPS; ++s) {
-        a[s].load(pa - s * row_bytes + lane_off);
-        b[s].load(pb - s * row_bytes + lane_off);
-      }
-#pragma unroll
-      for (int s = 0; s < STEPS; ++s) hp[s].load(ph - s * row_bytes + lane_off);
-    }
-  } else {
-#pragma unroll
-    for (int s = 0; s < STEPS; ++s) {
-      const int64_t r = r0 + s;
-      const int64_t t = BWD ? seq - 1 - r : r;
-      // Outside the sequence the step is the identity map (a=1, b=0); the first
-      // step of the scan has no predecessor (a=0), whatever alpha holds there.
-      a[s].fill(r >= seq ? 1.0f : 0.0f);
-      b[s].fill(0.0f);
-      if (BWD) hp[s].fill(0.0f);
-      if (col_ok && r < seq) {
-        if (r >= 1) a[s].load(p.in_a + tile_base + (BWD ? t + 1 : t) * row_bytes + lane_off);
-        b[s].load(p.in_b + tile_base + t * row_bytes + lane_off);
-        if (BWD && t >= 1) hp[s].load(p.in_h + tile_base + (t - 1) * row_bytes + lane_off);
-      }
-    }
-  }
-
-  float state[VEC];
-  const bool solo = !chained && n_waves == 1;  // the slice is the whole sequence: state starts at 0
-  if (solo) {
-#pragma unroll
-    for (int v = 0; v < VEC; ++v) state[v] = 0.0f;
-  } else {
-    // ---- phase 1b: the slice as an affine map --------------------------------------
-    float mA[VEC], mB[VEC];
-#pragma unroll
-    for (int v = 0; v < VEC; ++v) {
-      mA[v] = 1.0f;
-      mB[v] = 0.0f;
-    }
-#pragma unroll
-    for (int s = 0; s < STEPS; ++s) {
-#pragma unroll
-      for (int v = 0; v < VEC; ++v) {
-        const float av = a[s].get(v);
-        mB[v] = __builtin_fmaf(av, mB[v], b[s].get(v));
-        mA[v] *= av;
-      }
-    }
-#pragma unroll
-    for (int v = 0; v < VEC; ++v)
-      lds_map[(wave * VEC + v) * 64 + lane] = make_float2(mA[v], mB[v]);
-    __syncthreads();
-
-    // ---- phase 2: wave 0 composes the waves and chains the chunks -------------------
-    if (wave == 0) {
-      float cA[VEC], cB[VEC], hin[VEC];
-#pragma unroll
-      for (int v = 0; v < VEC; ++v) {
-        cA[v] = 1.0f;
-        cB[v] = 0.0f;
-        hin[v] = 0.0f;
-      }
-      for (int w = 0; w < n_waves; ++w) {
-#pragma unroll
-        for (int v = 0; v < VEC; ++v) {
-          const float2 m = lds_map[(w * VEC + v) * 64 + lane];
-          cB[v] = __builtin_fmaf(m.x, cB[v], m.y);
-          cA[v] *= m.x;
+        const int64_t r = r0 + s;
+        const int64_t t = BWD ? seq - 1 - r : r;
+        // Outside the sequence the step is the identity map (a=1, b=0); the first
+        // step of the scan has no predecessor (a=0), whatever alpha holds there.
+        a[s].fill(r >= seq ? 1.0f : 0.0f);
+        b[s].fill(0.0f);
+        if (BWD) hp[s].fill(0.0f);
+        if (col_ok && r < seq) {
+          if (r >= 1) a[s].load(uniform_ptr(p.in_a + tile_base + (BWD ? t + 1 : t) * row_bytes) + lane_off);
+          b[s].load(uniform_ptr(p.in_b + tile_base + t * row_bytes) + lane_off);
+          if (BWD && t >= 1) hp[s].load(uniform_ptr(p.in_h + tile_base + (t - 1) * row_bytes) + lane_off);
         }
       }
-      if (chained) {
-        const bool last = chunk == p.n_chunks - 1;
-        uint64_t *mine = p.words + (static_cast<size_t>(chunk) * p.n_ctiles + ctile) * 3 * kLaneSlots + lane;
-        if (chunk > 0) {
-          if (!last) {
+    }
+
+    float state[VEC];
+    const bool solo = !chained && n_waves == 1;  // the slice is the whole sequence: state starts at 0
+    if (solo) {
 #pragma unroll
-            for (int v = 0; v < VEC; ++v) {
-              st_word(mine + (0 * VEC + v) * 64, epoch, cA[v]);
-              st_word(mine + (1 * VEC + v) * 64, epoch, cB[v]);
-            }
-          }
-          // Look back: compose maps of earlier chunks until one offers its outgoing state.
-          float accA[VEC], accB[VEC];
+      for (int v = 0; v < VEC; ++v) state[v] = 0.0f;
+    } else {
+      // ---- phase 1b: the slice as an affine map --------------------------------------
+      float mA[VEC], mB[VEC];
+#pragma unroll
+      for (int v = 0; v < VEC; ++v) {
+        mA[v] = 1.0f;
+        mB[v] = 0.0f;
+      }
+#pragma unroll
+      for (int s = 0; s < STEPS; ++s) {
+#pragma unroll
+        for (int v = 0; v < VEC; ++v) {
+          const float av = a[s].get(v);
+          mB[v] = __builtin_fmaf(av, mB[v], b[s].get(v));
+          mA[v] *= av;
+        }
+      }
+#pragma unroll
+      for (int v = 0; v < VEC; ++v)
+        lds_map[(wave * VEC + v) * 64 + lane] = make_float2(mA[v], mB[v]);
+      __syncthreads();
+
+      // ---- phase 2: compose the waves, chain the chunks --------------------------------
+      // Wave 0 folds the waves' maps into the chunk's map and publishes it.  Meanwhile
+      // wave w (w < look) fetches what chunk-1-w offers - its outgoing state if it has
+      // one, else its map - so a look-back over `look` chunks costs one memory round
+      // trip instead of one per chunk.  Chains longer than that repeat the step.
+      const bool last = chunk == p.n_chunks - 1;
+      uint64_t *mine = nullptr;
+      float cA[VEC], cB[VEC], hin[VEC], accA[VEC], accB[VEC];
+#pragma unroll
+      for (int v = 0; v < VEC; ++v) {
+        cA[v] = accA[v] = 1.0f;
+        cB[v] = accB[v] = hin[v] = 0.0f;
+      }
+      if (wave == 0) {
+        for (int w = 0; w < n_waves; ++w) {
 #pragma unroll
           for (int v = 0; v < VEC; ++v) {
-            accA[v] = 1.0f;
-            accB[v] = 0.0f;
+            const float2 m = lds_map[(w * VEC + v) * 64 + lane];
+            cB[v] = __builtin_fmaf(m.x, cB[v], m.y);
+            cA[v] *= m.x;
           }
-          int j = chunk - 1;
-          uint32_t polls = 0;
-          bool resolved = false;
-          while (!resolved) {
+        }
+        if (chained) {
+          mine = p.words + (static_cast<size_t>(chunk) * p.n_ctiles + ctile) * 3 * kLaneSlots + lane;
+          if (chunk > 0 && !last) {
+#pragma unroll
+            for (int v = 0; v < VEC; ++v) {
+              st_word(mine + (0 * VEC + v) * 64, tag, cA[v]);
+              st_word(mine + (1 * VEC + v) * 64, tag, cB[v]);
+            }
+          }
+        }
+      }
+      if (chained && chunk > 0) {
+        int nearest = chunk - 1;  // nearest earlier chunk not folded yet
+        for (;;) {
+          const int j = nearest - wave;
+          if (wave < look && j >= 0) {
             const uint64_t *theirs =
                 p.words + (static_cast<size_t>(j) * p.n_ctiles + ctile) * 3 * kLaneSlots + lane;
-            uint64_t wa[VEC], wb[VEC], ws[VEC];
-#pragma unroll
-            for (int v = 0; v < VEC; ++v) {
-              ws[v] = ld_word(theirs + (2 * VEC + v) * 64);
-              wa[v] = ld_word(theirs + (0 * VEC + v) * 64);
-              wb[v] = ld_word(theirs + (1 * VEC + v) * 64);
-            }
-            bool have_state = true, have_map = true;
-#pragma unroll
-            for (int v = 0; v < VEC; ++v) {
-              have_state = have_state && word_tag(ws[v]) == epoch;
-              have_map = have_map && word_tag(wa[v]) == epoch && word_tag(wb[v]) == epoch;
-            }
-            if (have_state) {
-#pragma unroll
-              for (int v = 0; v < VEC; ++v) hin[v] = __builtin_fmaf(accA[v], word_val(ws[v]), accB[v]);
-              resolved = true;
-            } else if (have_map && j > 0) {
+            float pA[VEC], pB[VEC];
+            uint32_t kind = kPredNone;
+            uint32_t polls = 0;
+            while (kind == kPredNone) {
+              uint64_t wa[VEC], wb[VEC], ws[VEC];
 #pragma unroll
               for (int v = 0; v < VEC; ++v) {
-                accB[v] = __builtin_fmaf(accA[v], word_val(wb[v]), accB[v]);
-                accA[v] *= word_val(wa[v]);
+                ws[v] = ld_word(theirs + (2 * VEC + v) * 64);
+                wa[v] = ld_word(theirs + (0 * VEC + v) * 64);
+                wb[v] = ld_word(theirs + (1 * VEC + v) * 64);
               }
-              --j;
-            } else {
-              if (++polls > kSpinLimit) {
-                st_u32(p.hdr + HDR_ERROR, 1u);
-                resolved = true;  // give up: zero incoming state, the grid still drains
+              bool have_state = true, have_map = true;
+#pragma unroll
+              for (int v = 0; v < VEC; ++v) {
+                have_state = have_state && word_tag(ws[v]) == tag;
+                have_map = have_map && word_tag(wa[v]) == tag && word_tag(wb[v]) == tag;
               }
-              __builtin_amdgcn_s_sleep(2);
+              // decide for the whole wave, so that one word per wave describes the slot
+              if (__builtin_amdgcn_ballot_w64(have_state) == ~0ull) {
+                kind = kPredState;
+#pragma unroll
+                for (int v = 0; v < VEC; ++v) {
+                  pA[v] = 0.0f;
+                  pB[v] = word_val(ws[v]);
+                }
+              } else if (j > 0 && __builtin_amdgcn_ballot_w64(have_map) == ~0ull) {
+                kind = kPredMap;
+#pragma unroll
+                for (int v = 0; v < VEC; ++v) {
+                  pA[v] = word_val(wa[v]);
+                  pB[v] = word_val(wb[v]);
+                }
+              } else if (++polls > kSpinLimit) {
+                if (lane == 0) st_u32(p.hdr + HDR_ERROR, 1u);
+                kind = kPredState;  // give up: zero state, so that the grid still drains
+#pragma unroll
+                for (int v = 0; v < VEC; ++v) pA[v] = pB[v] = 0.0f;
+              } else {
+                __builtin_amdgcn_s_sleep(2);
+              }
             }
+#pragma unroll
+            for (int v = 0; v < VEC; ++v)
+              lds_pred[(wave * VEC + v) * 64 + lane] = make_float2(pA[v], pB[v]);
+            if (lane == 0) s_kind[wave] = kind;
           }
+          __syncthreads();
+          if (wave == 0) {
+            bool resolved = false;
+            for (int w = 0; w < look && nearest - w >= 0 && !resolved; ++w) {
+              const bool is_state = s_kind[w] == kPredState;
+#pragma unroll
+              for (int v = 0; v < VEC; ++v) {
+                const float2 m = lds_pred[(w * VEC + v) * 64 + lane];
+                if (is_state) {
+                  hin[v] = __builtin_fmaf(accA[v], m.y, accB[v]);
+                } else {
+                  accB[v] = __builtin_fmaf(accA[v], m.y, accB[v]);
+                  accA[v] *= m.x;
+                }
+              }
+              resolved = is_state;
+            }
+            if (lane == 0) s_resolved = resolved ? 1u : 0u;
+          }
+          __syncthreads();
+          if (s_resolved != 0u) break;  // chunk 0 always offers a state, so this is reached
+          nearest -= look;
         }
-        if (!last) {
+      }
+
+      if (wave == 0) {
+        if (chained && !last) {
 #pragma unroll
           for (int v = 0; v < VEC; ++v)
-            st_word(mine + (2 * VEC + v) * 64, epoch, __builtin_fmaf(cA[v], hin[v], cB[v]));
+            st_word(mine + (2 * VEC + v) * 64, tag, __builtin_fmaf(cA[v], hin[v], cB[v]));
         }
-        // Nothing below reads the workspace.  The workgroup that counts last knows
-        // every tile is past its look-back and rearms the header for the next launch.
-        if (lane == 0) {
-          const uint32_t old = __hip_atomic_fetch_add(p.hdr + HDR_DONE, 1u, __ATOMIC_RELAXED,
-                                                      __HIP_MEMORY_SCOPE_AGENT);
-          if (old == gridDim.x - 1) {
-            st_u32(p.hdr + HDR_TICKET, 0u);
-            st_u32(p.hdr + HDR_DONE, 0u);
-            // 0 is the tag of never-written words: skip it when the counter wraps
-            st_u32(p.hdr + HDR_EPOCH, epoch + 1u == 0u ? 1u : epoch + 1u);
+        // incoming state of every wave of this tile, left where the wave's map was
+        for (int w = 0; w < n_waves; ++w) {
+#pragma unroll
+          for (int v = 0; v < VEC; ++v) {
+            const float2 m = lds_map[(w * VEC + v) * 64 + lane];
+            lds_map[(w * VEC + v) * 64 + lane].x = hin[v];
+            hin[v] = __builtin_fmaf(m.x, hin[v], m.y);
           }
         }
       }
-      // incoming state of every wave of this tile
-      for (int w = 0; w < n_waves; ++w) {
+      __syncthreads();
 #pragma unroll
-        for (int v = 0; v < VEC; ++v) {
-          lds_in[(w * VEC + v) * 64 + lane] = hin[v];
-          const float2 m = lds_map[(w * VEC + v) * 64 + lane];
-          hin[v] = __builtin_fmaf(m.x, hin[v], m.y);
+      for (int v = 0; v < VEC; ++v) state[v] = lds_map[(wave * VEC + v) * 64 + lane].x;
+    }
+
+    // ---- phase 3: the recurrence from the true incoming state, in order -------------
+#pragma unroll
+    for (int s = 0; s < STEPS; ++s) {
+      keep_packed(a[s]);
+      keep_packed(b[s]);
+      if (BWD) keep_packed(hp[s]);
+    }
+    if (full) {
+      if (!BWD) {
+        char *po = p.out0 + tile_base + r0 * row_bytes;
+#pragma unroll
+        for (int s = 0; s < STEPS; ++s) {
+#pragma unroll
+          for (int v = 0; v < VEC; ++v) state[v] = __builtin_fmaf(a[s].get(v), state[v], b[s].get(v));
+          RowT o;
+          o.pack(state);
+          o.store(uniform_ptr(po + s * row_bytes) + lane_off);
+        }
+      } else {
+        const int64_t t0 = seq - 1 - r0;
+        char *pgb = p.out0 + tile_base + t0 * row_bytes;
+        char *pga = p.out1 + tile_base + t0 * row_bytes;
+#pragma unroll
+        for (int s = 0; s < STEPS; ++s) {
+          float ga[VEC];
+#pragma unroll
+          for (int v = 0; v < VEC; ++v) {
+            state[v] = __builtin_fmaf(a[s].get(v), state[v], b[s].get(v));
+            ga[v] = state[v] * hp[s].get(v);
+          }
+          RowT ob, oa;
+          ob.pack(state);
+          oa.pack(ga);
+          ob.store(uniform_ptr(pgb - s * row_bytes) + lane_off);
+          oa.store(uniform_ptr(pga - s * row_bytes) + lane_off);
         }
       }
-    }
-    __syncthreads();
-#pragma unroll
-    for (int v = 0; v < VEC; ++v) state[v] = lds_in[(wave * VEC + v) * 64 + lane];
-  }
-
-  // ---- phase 3: the recurrence from the true incoming state, in order -------------
-  if (full) {
-    if (!BWD) {
-      char *po = p.out0 + tile_base + r0 * row_bytes;
-#pragma unroll
-      for (int s = 0; s < STEPS; ++s) {
-#pragma unroll
-        for (int v = 0; v < VEC; ++v) state[v] = __builtin_fmaf(a[s].get(v), state[v], b[s].get(v));
-        RowT o;
-        o.pack(state);
-        o.store(po + s * row_bytes + lane_off);
-      }
     } else {
-      const int64_t t0 = seq - 1 - r0;
-      char *pgb = p.out0 + tile_base + t0 * row_bytes;
-      char *pga = p.out1 + tile_base + t0 * row_bytes;
 #pragma unroll
       for (int s = 0; s < STEPS; ++s) {
+        const int64_t r = r0 + s;
+        const int64_t t = BWD ? seq - 1 - r : r;
         float ga[VEC];
 #pragma unroll
         for (int v = 0; v < VEC; ++v) {
           state[v] = __builtin_fmaf(a[s].get(v), state[v], b[s].get(v));
-          ga[v] = state[v] * hp[s].get(v);
+          if (BWD) ga[v] = (t >= 1) ? state[v] * hp[s].get(v) : 0.0f;  // grad_alpha[0] = 0
         }
-        RowT ob, oa;
-        ob.pack(state);
-        oa.pack(ga);
-        ob.store(pgb - s * row_bytes + lane_off);
-        oa.store(pga - s * row_bytes + lane_off);
+        if (col_ok && r < seq) {
+          RowT o;
+          o.pack(state);
+          o.store(uniform_ptr(p.out0 + tile_base + t * row_bytes) + lane_off);
+          if (BWD) {
+            RowT oa;
+            oa.pack(ga);
+            oa.store(uniform_ptr(p.out1 + tile_base + t * row_bytes) + lane_off);
+          }
+        }
       }
     }
-  } else {
-#pragma unroll
-    for (int s = 0; s < STEPS; ++s) {
-      const int64_t r = r0 + s;
-      const int64_t t = BWD ? seq - 1 - r : r;
-      float ga[VEC];
-#pragma unroll
-      for (int v = 0; v < VEC; ++v) {
-        state[v] = __builtin_fmaf(a[s].get(v), state[v], b[s].get(v));
-        if (BWD) ga[v] = (t >= 1) ? state[v] * hp[s].get(v) : 0.0f;  // grad_alpha[0] = 0
-      }
-      if (col_ok && r < seq) {
-        RowT o;
-        o.pack(state);
-        o.store(p.out0 + tile_base + t * row_bytes + lane_off);
-        if (BWD) {
-          RowT oa;
-          oa.pack(ga);
-          oa.store(p.out1 + tile_base + t * row_bytes + lane_off);
-        }
+  }
+
+#ifdef FSS_RESIDENCY_PROBE
+  if (threadIdx.x == 0 && p.hdr) __hip_atomic_fetch_sub(p.hdr + 8, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+#endif
+  // Two-level completion count (16 first-level counters on separate lines keep the
+  // atomics off one hot address).  Whoever counts last knows that no workgroup will
+  // read the workspace again and advances the epoch for the next launch.
+  if (chained && threadIdx.x == 0) {
+    const uint32_t slot = blockIdx.x % kDoneSlots;
+    const uint32_t in_slot = (gridDim.x - slot + kDoneSlots - 1) / kDoneSlots;
+    uint32_t *counter = p.hdr + HDR_SLOT0 + slot * HDR_SLOT_STRIDE;
+    if (add_u32(counter, 1u) == in_slot - 1) {
+      st_u32(counter, 0u);
+      const uint32_t slots_used = gridDim.x < kDoneSlots ? gridDim.x : kDoneSlots;
+      if (add_u32(p.hdr + HDR_DONE, 1u) == slots_used - 1) {
+        st_u32(p.hdr + HDR_DONE, 0u);
+        // 0 is the tag of never-written words: skip it when the counter wraps
+        st_u32(p.hdr + HDR_EPOCH, tag + 1u == 0u ? 1u : tag + 1u);
       }
     }
   }
@@ -532,6 +631,18 @@ inline int64_t ceil_div(int64_t a, int64_t b) { return (a + b - 1) / b; }
 // Register budget: packed dwords a lane may hold per input tensor.
 inline int max_vec_steps(int dtype) { return dtype == FSS_BF16 ? 64 : 32; }  // vec*steps
 
+// LDS: one (A,B) slot per lane and vector element for every wave, plus the same
+// for every wave that looks back.
+constexpr size_t kLdsBudget = 60 * 1024;
+inline int look_waves(int waves, int vec) {
+  int look = waves < kMaxLookWaves ? waves : kMaxLookWaves;
+  while (look > 1 && static_cast<size_t>(waves + look) * vec * 512 > kLdsBudget) --look;
+  return look;
+}
+inline size_t lds_bytes(int waves, int vec) {
+  return static_cast<size_t>(waves + look_waves(waves, vec)) * vec * 512;
+}
+
 inline bool config_valid(const fss_config &c, int dtype) {
   const bool vec_ok = dtype == FSS_BF16 ? (c.vec == 1 || c.vec == 2 || c.vec == 4 || c.vec == 8)
                                         : (c.vec == 1 || c.vec == 2 || c.vec == 4);
@@ -540,8 +651,7 @@ inline bool config_valid(const fss_config &c, int dtype) {
   if (c.vec * c.steps > max_vec_steps(dtype)) return false;
   if (dtype == FSS_BF16 && c.vec == 1 && c.steps > 32) return false;
   if (c.waves < 1 || c.waves > 16) return false;
-  // LDS: waves * vec * 64 * 12 bytes
-  if (static_cast<size_t>(c.waves) * c.vec * 64 * 12 > 64 * 1024) return false;
+  if (lds_bytes(c.waves, c.vec) > kLdsBudget) return false;
   return true;
 }
 
@@ -549,30 +659,42 @@ inline bool config_valid(const fss_config &c, int dtype) {
 // tensors of the call.
 void complete_config(fss_config &c, int64_t bs, int64_t seq, int64_t d, int dtype, int dir,
                      size_t align) {
+  // Choices below come from sweeps on MI355X over the five measured workloads
+  // (bs8 d1024 seq512..8192, bs16 d512 seq2048, bs4 d2048 seq8192, bs2 d768
+  // seq1024, bs1 d256 seq65521).  What they showed: 4 bytes per lane per load
+  // (bf16 x2) with as many timesteps in registers as fit beats wider vectors;
+  // 8 waves per workgroup (two workgroups per CU, one loading while the other
+  // chains and stores) beats 16 unless the chain of chunks is long; with few
+  // channels, one channel per lane (twice the column tiles) and shorter slices
+  // put more waves in flight.
   const int esize = dtype == FSS_BF16 ? 2 : 4;
+  const int64_t channels = bs * d;
   if (c.vec == 0) {
-    const int vmax = dtype == FSS_BF16 ? 4 : 2;
-    int v = vmax;
-    while (v > 1 && (d % v != 0 || align % (static_cast<size_t>(v) * esize) != 0)) v >>= 1;
-    // do not let a wide vector leave most of the last column tile empty
-    while (v > 1 && ceil_div(d, 64 * v) * 64 * v > d + d / 4 && d % (64 * (v / 2)) == 0) v >>= 1;
+    const bool can2 = d % 2 == 0 && align % (2 * static_cast<size_t>(esize)) == 0;
+    int v = can2 ? 2 : 1;
+    // few channels: more, narrower column tiles; also never pad a row to twice its width
+    if (v == 2 && (channels < 8192 || ceil_div(d, 128) * 128 >= 2 * ceil_div(d, 64) * 64)) v = 1;
     c.vec = v;
   }
+  // packed dwords one lane holds per timestep and tensor
+  const int dwords = dtype == FSS_BF16 ? (c.vec + 1) / 2 : c.vec;
   if (c.steps == 0) {
-    int budget = (dir == FSS_BWD ? 32 : 64);
-    if (dtype == FSS_F32) budget /= 2;
-    int s = budget / c.vec;
+    int s = (dir == FSS_BWD ? 16 : 32) / dwords;  // 2 (forward) or 3 (backward) tensors stay in registers
     if (s > 32) s = 32;
     if (s < 8) s = 8;
-    // keep enough waves in flight to cover the machine (256 CUs x 16 waves)
+    // small problems: shorter slices until the machine has a few waves per SIMD
     const int64_t ctiles = bs * ceil_div(d, 64 * c.vec);
-    while (s > 8 && ctiles * ceil_div(seq, s) < 4096) s >>= 1;
+    while (s > 8 && ctiles * ceil_div(seq, s) < 1024) s >>= 1;
+    // never longer than the sequence needs
+    while (s > 8 && seq <= s / 2) s >>= 1;
     c.steps = s;
   }
   if (c.waves == 0) {
     int64_t w = ceil_div(seq, c.steps);
-    if (w > 8) w = 8;
-    while (w > 1 && static_cast<size_t>(w) * c.vec * 64 * 12 > 64 * 1024) --w;
+    // long chains of chunks (few channels, long sequence): the largest tile
+    const int64_t cap = ceil_div(seq, static_cast<int64_t>(8) * c.steps) > 64 ? 16 : 8;
+    if (w > cap) w = cap;
+    while (w > 1 && lds_bytes(static_cast<int>(w), c.vec) > kLdsBudget) --w;
     c.waves = static_cast<int32_t>(w);
   }
 }
@@ -596,7 +718,7 @@ int make_plan(Plan &pl, int64_t bs, int64_t seq, int64_t d, int dtype, int dir, 
   }
   fss_config c = {0, 0, 0, 0};
   if (user) c = *user;
-  c.reserved = 0;
+  if (c.max_groups < 0) return FSS_ERR_BAD_CONFIG;
   const int64_t dd = d > 0 ? d : 1, ss = seq > 0 ? seq : 1, bb = bs > 0 ? bs : 1;
   complete_config(c, bb, ss, dd, dtype, dir, align);
   if (!config_valid(c, dtype)) return FSS_ERR_BAD_CONFIG;
@@ -639,12 +761,63 @@ int check_device() {
   return state == 1 ? FSS_OK : FSS_ERR_UNSUPPORTED_DEVICE;
 }
 
+// Workgroups of `kernel` that are certainly resident together on the device (0 on
+// error).  Deliberately not the runtime's occupancy query: the kernel's waits
+// need a lower bound, and that query bounds by vector registers and LDS only.
+// These kernels hold many scalar registers as well (a row pointer per load); a
+// wave may be allocated 128 of the 800 a SIMD has, which caps a SIMD at 6 waves -
+// the residency measured on MI355X for the scalar-heaviest variants.
+template <typename Kernel>
+int resident_workgroups(Kernel kernel, int waves, size_t lds) {
+  static int cu_count = 0;
+  if (cu_count == 0) {
+    int dev = 0, n = 0;
+    if (hipGetDevice(&dev) != hipSuccess ||
+        hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0)
+      return 0;
+    cu_count = n;
+  }
+  hipFuncAttributes attr;
+  const hipError_t e = hipFuncGetAttributes(&attr, reinterpret_cast<const void *>(kernel));
+  if (e != hipSuccess) {
+    tls_hip_error = static_cast<int>(e);
+    return 0;
+  }
+  int vgprs = attr.numRegs > 0 ? attr.numRegs : 128;
+  vgprs = (vgprs + 7) / 8 * 8;                    // allocation granule
+  int per_simd = 512 / vgprs;                      // 512 vector registers per lane per SIMD
+  if (per_simd > 6) per_simd = 6;                  // scalar-register bound, see above
+  if (per_simd < 1) return 0;
+  int per_cu;
+  if (waves >= 4)
+    per_cu = per_simd / ((waves + 3) / 4);         // a workgroup puts ceil(waves/4) waves on a SIMD
+  else
+    per_cu = per_simd * (waves == 1 ? 4 : waves == 2 ? 2 : 1);
+  const size_t lds_alloc = (lds + attr.sharedSizeBytes + 1023) / 1024 * 1024;
+  const int by_lds = static_cast<int>((160 * 1024) / (lds_alloc ? lds_alloc : 1024));
+  if (per_cu > by_lds) per_cu = by_lds;
+  if (per_cu > 32) per_cu = 32;
+  return per_cu * cu_count;
+}
+
 template <typename E, int VEC, int STEPS, bool BWD>
 int launch_one(const ScanArgs &args, const Plan &pl, hipStream_t stream) {
-  const dim3 grid(static_cast<uint32_t>(pl.n_tiles));
-  const dim3 block(static_cast<uint32_t>(pl.cfg.waves) * 64);
-  const size_t lds_bytes = static_cast<size_t>(pl.cfg.waves) * VEC * 64 * 12;
-  hipLaunchKernelGGL((scan_kernel<E, VEC, STEPS, BWD>), grid, block, lds_bytes, stream, args);
+  // The kernel's waits are only safe if every workgroup of the grid is resident,
+  // so the grid never exceeds what the device holds at once; workgroups loop.
+  static int resident[17] = {0};  // by waves per workgroup; same answer on every call
+  const int waves = pl.cfg.waves;
+  const size_t lds = lds_bytes(waves, VEC);
+  int fit = __atomic_load_n(&resident[waves], __ATOMIC_RELAXED);
+  if (fit == 0) {
+    fit = resident_workgroups(scan_kernel<E, VEC, STEPS, BWD>, waves, lds);
+    if (fit <= 0) return FSS_ERR_LAUNCH;
+    __atomic_store_n(&resident[waves], fit, __ATOMIC_RELAXED);
+  }
+  int64_t n_groups = pl.n_tiles < fit ? pl.n_tiles : fit;
+  if (pl.cfg.max_groups > 0 && pl.cfg.max_groups < n_groups) n_groups = pl.cfg.max_groups;
+  const dim3 grid(static_cast<uint32_t>(n_groups));
+  const dim3 block(static_cast<uint32_t>(waves) * 64);
+  hipLaunchKernelGGL((scan_kernel<E, VEC, STEPS, BWD>), grid, block, lds, stream, args);
   const hipError_t e = hipGetLastError();
   if (e != hipSuccess) {
     tls_hip_error = static_cast<int>(e);
@@ -716,6 +889,8 @@ int run_scan(int dtype, int dir, const void *alpha, const void *in_b, const void
   args.tiles_per_row = static_cast<int32_t>(pl.tiles_per_row);
   args.n_ctiles = static_cast<int32_t>(pl.n_ctiles);
   args.n_chunks = static_cast<int32_t>(pl.n_chunks);
+  args.n_tiles = static_cast<int32_t>(pl.n_tiles);
+  args.look_waves = look_waves(pl.cfg.waves, pl.cfg.vec);
   args.hdr = static_cast<uint32_t *>(workspace);
   args.words = workspace ? reinterpret_cast<uint64_t *>(static_cast<char *>(workspace) + kHeaderBytes) : nullptr;
   hipStream_t s = static_cast<hipStream_t>(stream);

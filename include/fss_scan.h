@@ -75,7 +75,10 @@ typedef enum fss_dir { FSS_FWD = 0, FSS_BWD = 1 } fss_dir;
  *   steps  timesteps each lane keeps in registers (8, 16 or 32; vec*steps bounded
  *          by the register budget of the direction)
  *   waves  wavefronts per workgroup (1..16); one workgroup scans waves*steps
- *          consecutive timesteps of 64*vec channels
+ *          consecutive timesteps of 64*vec channels at a time
+ *   max_groups  upper bound on the workgroups launched; 0 = as many as the device
+ *          holds resident at once (the grid is persistent: workgroups loop over
+ *          tiles, and never more are launched than are resident together)
  * Results do not depend on the configuration beyond fp32 rounding of the
  * carries handed between chunks.
  */
@@ -83,7 +86,7 @@ typedef struct fss_config {
   int32_t vec;
   int32_t steps;
   int32_t waves;
-  int32_t reserved;
+  int32_t max_groups;
 } fss_config;
 
 int fss_abi_version(void);

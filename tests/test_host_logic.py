@@ -37,20 +37,20 @@ def test_workspace_sizing_and_config_choice():
                 assert lib.fss_choose_config(bs, seq, d, dtype, direction, 16, ctypes.byref(cfg)) == 0
                 assert d % cfg.vec == 0 and cfg.steps in (8, 16, 32) and 1 <= cfg.waves <= 16
                 need = lib.fss_workspace_bytes(bs, seq, d, dtype, direction, None)
-                assert need >= 256 and need % 256 == 0
+                assert need >= 4096 and need % 256 == 0
                 assert need <= lib.fss_workspace_bytes_max(bs, seq, d)
                 chunks = -(-seq // (cfg.steps * cfg.waves))
                 tiles = bs * -(-d // (64 * cfg.vec)) * chunks
-                expect = 256 + (tiles * 3 * 64 * cfg.vec * 8 if chunks > 1 else 0)
+                expect = 4096 + (tiles * 3 * 64 * cfg.vec * 8 if chunks > 1 else 0)
                 assert need == expect
     # odd d forces the scalar path; 2-byte alignment too
     assert lib.fss_choose_config(2, 100, 77, 0, 0, 16, ctypes.byref(cfg)) == 0 and cfg.vec == 1
     assert lib.fss_choose_config(2, 100, 64, 0, 0, 2, ctypes.byref(cfg)) == 0 and cfg.vec == 1
     # explicit configurations: bad ones are refused, good ones size the workspace
     bad = _native.FssConfig(3, 8, 1, 0)
-    assert lib.fss_workspace_bytes(2, 100, 64, 0, 0, ctypes.byref(bad)) == 256
+    assert lib.fss_workspace_bytes(2, 100, 64, 0, 0, ctypes.byref(bad)) == 4096
     good = _native.FssConfig(2, 8, 2, 0)
-    assert lib.fss_workspace_bytes(2, 100, 64, 0, 0, ctypes.byref(good)) == 256 + 2 * 1 * 7 * 3 * 128 * 8
+    assert lib.fss_workspace_bytes(2, 100, 64, 0, 0, ctypes.byref(good)) == 4096 + 2 * 1 * 7 * 3 * 128 * 8
     assert lib.fss_choose_config(-1, 4, 4, 0, 0, 16, ctypes.byref(cfg)) == 2
 
 

@@ -251,3 +251,22 @@ def test_against_compiled_reference_header(oracle):
         ga, gb = oracle.scan_bwd_f32(alpha, h, dout)
         np.testing.assert_array_equal(gb, gb_ref, err_msg=str(shape))
         np.testing.assert_array_equal(ga, ga_ref, err_msg=str(shape))
+
+
+def test_torch_loop_baseline_equals_c_oracle(oracle):
+    """The CPU baseline timed by the bench (oracle/torch_loop.py) computes what the C oracle computes."""
+    from oracle.torch_loop import torch_loop_bwd, torch_loop_fwd
+
+    g = torch.Generator().manual_seed(12)
+    for shape in [(1, 1, 3), (2, 2, 4), (3, 40, 9)]:
+        alpha = torch.randn(shape, generator=g).to(torch.bfloat16)
+        beta = torch.randn(shape, generator=g).to(torch.bfloat16)
+        dout = torch.randn(shape, generator=g).to(torch.bfloat16)
+        bits = oracle.torch_bf16_to_bits
+        h = torch_loop_fwd(alpha, beta)
+        h_c = oracle.scan_fwd_bf16_f32out(bits(alpha), bits(beta))
+        np.testing.assert_array_equal(h.numpy(), h_c)
+        ga, gb = torch_loop_bwd(alpha, h, dout)
+        ga_c, gb_c = oracle.scan_bwd_bf16_f32out(bits(alpha), h_c, bits(dout))
+        np.testing.assert_array_equal(gb.numpy(), gb_c)
+        np.testing.assert_array_equal(ga.numpy(), ga_c)

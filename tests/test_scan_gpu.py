@@ -108,7 +108,7 @@ CONFIGS = [
     (1, 8, 1), (1, 16, 3), (1, 32, 16),
     (2, 8, 2), (2, 16, 8), (2, 32, 4), (2, 32, 16),
     (4, 8, 5), (4, 16, 8), (4, 8, 16),
-    (8, 8, 1), (8, 8, 8),
+    (8, 8, 1), (8, 8, 7),
 ]
 
 
@@ -117,6 +117,34 @@ def test_bf16_result_does_not_depend_on_chunking(oracle, config):
     """Same inputs through every tiling: many chunks, ragged tails, partial column tiles."""
     alpha, beta, dout = make_inputs("hawk", 2, 777, 328, seed=7)  # 328 = 8*41: partial tiles for every vec
     check_bf16(oracle, alpha, beta, dout, config=config, what=str(config))
+
+
+@pytest.mark.parametrize("groups", [1, 3, 7, 64])
+@pytest.mark.parametrize("config", [(1, 8, 1), (2, 8, 3), (2, 16, 8), (2, 32, 2), (4, 8, 16)],
+                         ids=lambda c: "v%d_s%d_w%d" % c)
+def test_bf16_few_workgroups_walk_many_tiles(oracle, config, groups):
+    """The grid is persistent: cap it far below the tile count, so that every workgroup
+    loops over many tiles and chunks wait on tiles of the same workgroup's earlier rounds."""
+    alpha, beta, dout = make_inputs("sigmoid", 2, 1531, 200, seed=13)
+    check_bf16(oracle, alpha, beta, dout, config=config + (groups,), what=f"{config} groups={groups}")
+    ext.workspace_status()
+
+
+@pytest.mark.parametrize("config", [(1, 8, 1), (1, 8, 2), (1, 8, 4), (2, 8, 2), (1, 16, 1), (2, 8, 8)],
+                         ids=lambda c: "v%d_s%d_w%d" % c)
+def test_bf16_full_grid_is_resident(oracle, config):
+    """Small workgroups at a size where the uncapped grid fills the device: every wait
+    must be served (no chain timeout), i.e. the grid really is resident all at once."""
+    alpha, beta, dout = make_inputs("sigmoid", 8, 4096, 1024, seed=17)
+    a, b, do = alpha.to(DEV), beta.to(DEV), dout.to(DEV)
+    h = ext._forward(torch.bfloat16, a, b, config)
+    ga, gb = ext._backward(torch.bfloat16, a, h, do, config)
+    ext.workspace_status()  # raises on a chain timeout
+    h_ref = ext._forward(torch.bfloat16, a, b, (2, 32, 16))
+    ga_ref, gb_ref = ext._backward(torch.bfloat16, a, h_ref, do, (2, 16, 16))
+    for got, want in ((h, h_ref), (ga, ga_ref), (gb, gb_ref)):
+        close = (got.float() - want.float()).abs().cpu().numpy() <= 1e-3
+        assert ((ulp_distance(bits(got), bits(want)) <= 2) | close).all()
 
 
 @pytest.mark.parametrize("config", [(1, 8, 4), (2, 8, 16), (2, 16, 2), (4, 8, 8), (1, 32, 1)],
