@@ -11,7 +11,8 @@ tensors already resident in HBM.  Prints ONE JSON line:
                    writes grad_alpha, grad_beta = 10 B) divided by the wall time per step
   roofline         the dominant kernel (the backward scan, 10 of the 16 B): its
                    algorithmic bytes per launch over its mean duration, measured with
-                   HIP events recorded around every launch inside the timed region
+                   HIP events recorded around the launches of every 8th step of the
+                   timed region
   cpu_baseline     the reference's PyTorch sequential loop (oracle/torch_loop.py) on the
                    host cores, same inputs, fp32; also the parity check of this run
 """
@@ -43,9 +44,14 @@ def parse_args():
     ap.add_argument("--config", default=None, help="explicit vec,steps,waves for both kernels (tuning)")
     ap.add_argument("--fwd-config", default=None)
     ap.add_argument("--bwd-config", default=None)
+    ap.add_argument("--event-stride", type=int, default=8,
+                    help="record HIP events around the two launches of every N-th timed step")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline / parity leg")
     ap.add_argument("--cpu-seconds", type=float, default=12.0, help="budget of the CPU baseline leg")
-    ap.add_argument("--flush-mb", type=int, default=1024, help="size of the cache-flush write for the cold timings")
+    ap.add_argument("--flush-mb", type=int, default=1024, help="size of the cache-flush read for the cold timings")
+    ap.add_argument("--copy-mb", type=int, default=0,
+                    help="run only the library's plain copy kernel on this many MiB, --steps times "
+                         "(hardware counters of the scan kernels are scaled by what they read for it)")
     return ap.parse_args()
 
 
@@ -71,6 +77,26 @@ def main() -> int:
         return 2
     dev = torch.device("cuda", 0)
     torch.cuda.set_device(dev)
+
+    if args.copy_mb > 0:
+        n = args.copy_mb << 20
+        src = torch.ones(n, dtype=torch.uint8, device=dev)
+        dst = torch.empty_like(src)
+        sp = torch.cuda.current_stream().cuda_stream
+        for _ in range(args.warmup):
+            _native.check(lib.fss_copy_bytes(src.data_ptr(), dst.data_ptr(), n, sp))
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        torch.cuda.synchronize()
+        e0.record()
+        for _ in range(args.steps):
+            _native.check(lib.fss_copy_bytes(src.data_ptr(), dst.data_ptr(), n, sp))
+        e1.record()
+        torch.cuda.synchronize()
+        ms = e0.elapsed_time(e1) / args.steps
+        print(json.dumps({"metric": "plain copy kernel", "read_bytes": n, "written_bytes": n, "steps": args.steps,
+                          "ms_per_launch": round(ms, 5), "value": round(2 * n / (ms * 1e-3) / 1e9, 1),
+                          "unit": "GB/s (read+write)"}))
+        return 0
 
     recipe, bs, seq, d = BASELINE_CASES[args.case]
     n_elem = bs * seq * d
@@ -118,22 +144,31 @@ def main() -> int:
         fwd()
         bwd()
     K = args.steps
-    ev = [[torch.cuda.Event(enable_timing=True) for _ in range(3)] for _ in range(K)]
+    # HIP events around the launches of every `stride`-th step of the timed region (an event
+    # between two kernels costs a few microseconds of GPU time, so not around every one)
+    stride = max(1, args.event_stride)
+    sampled = list(range(0, K, stride))
+    ev = {k: [torch.cuda.Event(enable_timing=True) for _ in range(3)] for k in sampled}
     torch.cuda.synchronize()
     t0 = time.perf_counter()
     for k in range(K):
-        ev[k][0].record(stream)
-        fwd()
-        ev[k][1].record(stream)
-        bwd()
-        ev[k][2].record(stream)
+        e = ev.get(k)
+        if e is None:
+            fwd()
+            bwd()
+        else:
+            e[0].record(stream)
+            fwd()
+            e[1].record(stream)
+            bwd()
+            e[2].record(stream)
     torch.cuda.synchronize()
     wall = time.perf_counter() - t0
     _native.check(lib.fss_workspace_status(pws, sp))
 
     ms_per_step = wall * 1e3 / K
-    fwd_ms = [ev[k][0].elapsed_time(ev[k][1]) for k in range(K)]
-    bwd_ms = [ev[k][1].elapsed_time(ev[k][2]) for k in range(K)]
+    fwd_ms = [ev[k][0].elapsed_time(ev[k][1]) for k in sampled]
+    bwd_ms = [ev[k][1].elapsed_time(ev[k][2]) for k in sampled]
     fwd_mean, bwd_mean = statistics.fmean(fwd_ms), statistics.fmean(bwd_ms)
     step_bytes = (FWD_BYTES_PER_ELEM + BWD_BYTES_PER_ELEM) * n_elem
     value = step_bytes / (ms_per_step * 1e-3) / 1e9
@@ -255,6 +290,7 @@ def main() -> int:
         "fwd_ms_median": round(statistics.median(fwd_ms), 5),
         "bwd_ms_median": round(statistics.median(bwd_ms), 5),
         "algorithmic_bytes_per_step": step_bytes,
+        "event_sampled_steps": len(sampled),
         "roofline": {
             "bound": "hbm",
             "kernel": "scan_kernel<BF16,...,BWD=true> (backward scan)",

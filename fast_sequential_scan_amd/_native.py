@@ -11,7 +11,8 @@ import threading
 from typing import Optional, Tuple
 
 PKG_DIR = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(PKG_DIR, "_lib", "libfss_scan.so")
+# FSS_SCAN_LIBRARY points at an alternative build of the same library (tuning experiments)
+LIB_PATH = os.environ.get("FSS_SCAN_LIBRARY") or os.path.join(PKG_DIR, "_lib", "libfss_scan.so")
 
 FSS_BF16, FSS_F32 = 0, 1
 FSS_FWD, FSS_BWD = 0, 1

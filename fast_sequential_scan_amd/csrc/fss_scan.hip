@@ -65,6 +65,12 @@
 
 namespace fss {
 
+// Device pointers are kept in the global address space explicitly: the generic
+// ("flat") form costs a 64-bit vector address per access and a slower instruction.
+#define FSS_GLOBAL __attribute__((address_space(1)))
+typedef const FSS_GLOBAL char *gcptr_t;
+typedef FSS_GLOBAL char *gptr_t;
+
 typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 typedef float f32x2 __attribute__((ext_vector_type(2)));
@@ -83,50 +89,66 @@ __device__ __forceinline__ uint32_t as_u32(float f) { return __builtin_bit_cast(
 // Pins a wave-uniform pointer into scalar registers, so that `p + lane_offset`
 // becomes the scalar-base + 32-bit-vector-offset form of a global access and
 // costs no vector registers or 64-bit vector adds per row.
-template <typename P>
-__device__ __forceinline__ P *uniform_ptr(P *ptr) {
+template <typename Ptr>
+__device__ __forceinline__ Ptr uniform_ptr(Ptr ptr) {
   const uint64_t u = reinterpret_cast<uint64_t>(ptr);
   const uint32_t lo = __builtin_amdgcn_readfirstlane(static_cast<uint32_t>(u));
   const uint32_t hi = __builtin_amdgcn_readfirstlane(static_cast<uint32_t>(u >> 32));
-  return reinterpret_cast<P *>((static_cast<uint64_t>(hi) << 32) | lo);
+  return reinterpret_cast<Ptr>((static_cast<uint64_t>(hi) << 32) | lo);
 }
 
-// Loads/stores of N dwords per lane.
-template <int N>
+// Loads/stores of N dwords per lane.  NT marks the access non-temporal: the data
+// is touched once, so the caches should not keep it in preference to other lines.
+template <int N, bool NT>
 struct DwordIO;
-template <>
-struct DwordIO<1> {
-  static __device__ __forceinline__ void load(uint32_t *dst, const char *p) {
-    dst[0] = *reinterpret_cast<const uint32_t *>(p);
+template <bool NT>
+struct DwordIO<1, NT> {
+  static __device__ __forceinline__ void load(uint32_t *dst, gcptr_t p) {
+    const FSS_GLOBAL uint32_t *q = reinterpret_cast<const FSS_GLOBAL uint32_t *>(p);
+    dst[0] = NT ? __builtin_nontemporal_load(q) : *q;
   }
-  static __device__ __forceinline__ void store(char *p, const uint32_t *src) {
-    *reinterpret_cast<uint32_t *>(p) = src[0];
+  static __device__ __forceinline__ void store(gptr_t p, const uint32_t *src) {
+    FSS_GLOBAL uint32_t *q = reinterpret_cast<FSS_GLOBAL uint32_t *>(p);
+    if (NT)
+      __builtin_nontemporal_store(src[0], q);
+    else
+      *q = src[0];
   }
 };
-template <>
-struct DwordIO<2> {
-  static __device__ __forceinline__ void load(uint32_t *dst, const char *p) {
-    u32x2 v = *reinterpret_cast<const u32x2 *>(p);
+template <bool NT>
+struct DwordIO<2, NT> {
+  static __device__ __forceinline__ void load(uint32_t *dst, gcptr_t p) {
+    const FSS_GLOBAL u32x2 *q = reinterpret_cast<const FSS_GLOBAL u32x2 *>(p);
+    const u32x2 v = NT ? __builtin_nontemporal_load(q) : *q;
     dst[0] = v.x;
     dst[1] = v.y;
   }
-  static __device__ __forceinline__ void store(char *p, const uint32_t *src) {
-    u32x2 v = {src[0], src[1]};
-    *reinterpret_cast<u32x2 *>(p) = v;
+  static __device__ __forceinline__ void store(gptr_t p, const uint32_t *src) {
+    const u32x2 v = {src[0], src[1]};
+    FSS_GLOBAL u32x2 *q = reinterpret_cast<FSS_GLOBAL u32x2 *>(p);
+    if (NT)
+      __builtin_nontemporal_store(v, q);
+    else
+      *q = v;
   }
 };
-template <>
-struct DwordIO<4> {
-  static __device__ __forceinline__ void load(uint32_t *dst, const char *p) {
-    u32x4 v = *reinterpret_cast<const u32x4 *>(p);
+template <bool NT>
+struct DwordIO<4, NT> {
+  static __device__ __forceinline__ void load(uint32_t *dst, gcptr_t p) {
+    const FSS_GLOBAL u32x4 *q = reinterpret_cast<const FSS_GLOBAL u32x4 *>(p);
+    const u32x4 v = NT ? __builtin_nontemporal_load(q) : *q;
     dst[0] = v.x;
     dst[1] = v.y;
     dst[2] = v.z;
     dst[3] = v.w;
   }
-  static __device__ __forceinline__ void store(char *p, const uint32_t *src) {
-    u32x4 v = {src[0], src[1], src[2], src[3]};
-    *reinterpret_cast<u32x4 *>(p) = v;
+  static __device__ __forceinline__ void store(gptr_t p, const uint32_t *src) {
+    const u32x4 v = {src[0], src[1], src[2], src[3]};
+    FSS_GLOBAL u32x4 *q = reinterpret_cast<FSS_GLOBAL u32x4 *>(p);
+    if (NT)
+      __builtin_nontemporal_store(v, q);
+    else
+      *q = v;
   }
 };
 
@@ -140,8 +162,14 @@ struct Row<BF16, VEC> {
   static constexpr int kDwords = VEC / 2;
   static constexpr int kBytes = VEC * 2;
   uint32_t dw[kDwords];
-  __device__ __forceinline__ void load(const char *p) { DwordIO<kDwords>::load(dw, p); }
-  __device__ __forceinline__ void store(char *p) const { DwordIO<kDwords>::store(p, dw); }
+  template <bool NT = false>
+  __device__ __forceinline__ void load(gcptr_t p) {
+    DwordIO<kDwords, NT>::load(dw, p);
+  }
+  template <bool NT = false>
+  __device__ __forceinline__ void store(gptr_t p) const {
+    DwordIO<kDwords, NT>::store(p, dw);
+  }
   __device__ __forceinline__ float get(int i) const {
     const uint32_t w = dw[i >> 1];
     return (i & 1) ? as_f32(w & 0xffff0000u) : as_f32(w << 16);
@@ -166,11 +194,18 @@ struct Row<BF16, 1> {
   static constexpr int kDwords = 1;
   static constexpr int kBytes = 2;
   uint32_t dw[1];
-  __device__ __forceinline__ void load(const char *p) {
-    dw[0] = *reinterpret_cast<const uint16_t *>(p);
+  template <bool NT = false>
+  __device__ __forceinline__ void load(gcptr_t p) {
+    const FSS_GLOBAL uint16_t *q = reinterpret_cast<const FSS_GLOBAL uint16_t *>(p);
+    dw[0] = NT ? __builtin_nontemporal_load(q) : *q;
   }
-  __device__ __forceinline__ void store(char *p) const {
-    *reinterpret_cast<uint16_t *>(p) = static_cast<uint16_t>(dw[0]);
+  template <bool NT = false>
+  __device__ __forceinline__ void store(gptr_t p) const {
+    FSS_GLOBAL uint16_t *q = reinterpret_cast<FSS_GLOBAL uint16_t *>(p);
+    if (NT)
+      __builtin_nontemporal_store(static_cast<uint16_t>(dw[0]), q);
+    else
+      *q = static_cast<uint16_t>(dw[0]);
   }
   __device__ __forceinline__ float get(int) const { return as_f32(dw[0] << 16); }
   __device__ __forceinline__ void fill(float x) { dw[0] = as_u32(x) >> 16; }
@@ -186,8 +221,14 @@ struct Row<F32, VEC> {
   static constexpr int kDwords = VEC;
   static constexpr int kBytes = VEC * 4;
   uint32_t dw[kDwords];
-  __device__ __forceinline__ void load(const char *p) { DwordIO<kDwords>::load(dw, p); }
-  __device__ __forceinline__ void store(char *p) const { DwordIO<kDwords>::store(p, dw); }
+  template <bool NT = false>
+  __device__ __forceinline__ void load(gcptr_t p) {
+    DwordIO<kDwords, NT>::load(dw, p);
+  }
+  template <bool NT = false>
+  __device__ __forceinline__ void store(gptr_t p) const {
+    DwordIO<kDwords, NT>::store(p, dw);
+  }
   __device__ __forceinline__ float get(int i) const { return as_f32(dw[i]); }
   __device__ __forceinline__ void fill(float x) {
 #pragma unroll
@@ -226,19 +267,19 @@ constexpr int kMaxLookWaves = 16;
 enum : uint32_t { kPredNone = 0, kPredMap = 1, kPredState = 2 };
 
 __device__ __forceinline__ uint32_t ld_u32(const uint32_t *p) {
-  return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  return __hip_atomic_load((const FSS_GLOBAL uint32_t *)p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 __device__ __forceinline__ void st_u32(uint32_t *p, uint32_t v) {
-  __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  __hip_atomic_store((FSS_GLOBAL uint32_t *)p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 __device__ __forceinline__ uint32_t add_u32(uint32_t *p, uint32_t v) {
-  return __hip_atomic_fetch_add(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  return __hip_atomic_fetch_add((FSS_GLOBAL uint32_t *)p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 __device__ __forceinline__ uint64_t ld_word(const uint64_t *p) {
-  return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  return __hip_atomic_load((const FSS_GLOBAL uint64_t *)p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 __device__ __forceinline__ void st_word(uint64_t *p, uint32_t tag, float v) {
-  __hip_atomic_store(p, (static_cast<uint64_t>(tag) << 32) | as_u32(v), __ATOMIC_RELAXED,
+  __hip_atomic_store((FSS_GLOBAL uint64_t *)p, (static_cast<uint64_t>(tag) << 32) | as_u32(v), __ATOMIC_RELAXED,
                      __HIP_MEMORY_SCOPE_AGENT);
 }
 __device__ __forceinline__ uint32_t word_tag(uint64_t w) { return static_cast<uint32_t>(w >> 32); }
@@ -259,26 +300,419 @@ struct ScanArgs {
   int32_t look_waves;     // waves that look back in parallel (1..min(WAVES, kMaxLookWaves))
   uint32_t *hdr;          // workspace header
   uint64_t *words;        // tagged words
+#ifdef FSS_TRACE
+  uint64_t *trace;        // debug build: 8 timestamps per tile, written by lane 0 of every wave 0
+#endif
 };
 
 // ---- the kernel ----------------------------------------------------------------
 
+// Which streams are accessed non-temporally (bit 0: alpha, 1: beta/dout, 2: saved h,
+// 3: h output of the forward, 4: gradient outputs of the backward).  Measured on
+// MI355X at bs8 seq4096 d1024, forward and backward alternating: marking the
+// three output streams and the backward's reads of h non-temporal takes the step
+// from 134 us to 113 us; marking the reads of alpha, beta or dout as well is slower.
+#ifndef FSS_NT_MASK
+#define FSS_NT_MASK 28
+#endif
+constexpr bool kNtA = (FSS_NT_MASK & 1) != 0;
+constexpr bool kNtB = (FSS_NT_MASK & 2) != 0;
+constexpr bool kNtH = (FSS_NT_MASK & 4) != 0;
+constexpr bool kNtOutFwd = (FSS_NT_MASK & 8) != 0;
+constexpr bool kNtOutBwd = (FSS_NT_MASK & 16) != 0;
+
+#ifdef FSS_TRACE
+#define FSS_STAMP(c, p, slot)                                                                   \
+  do {                                                                                          \
+    if ((p).trace && (c).lane == 0 && (c).wave == (c).trace_wave)                                \
+      (p).trace[(static_cast<size_t>((c).chunk) * (p).n_ctiles + (c).ctile) * 8 + (slot)] =       \
+          __builtin_amdgcn_s_memrealtime();                                                         \
+  } while (0)
+#else
+#define FSS_STAMP(c, p, slot) \
+  do {                        \
+  } while (0)
+#endif
+
+// What is fixed for a wave while it works on one tile.
+struct TileCtx {
+  int lane, wave, n_waves, look;
+  int chunk, ctile;      // position of the tile: chunk of the sequence, column tile
+  bool chained, last;    // more than one chunk in the sequence; this is the last one
+  uint32_t tag;          // epoch of this launch
+  int64_t tile_base;     // byte offset of (batch, row 0, first channel of the tile)
+  int64_t r0;            // first scan-order index of this wave's slice
+  int64_t seq, row_bytes;
+  uint32_t lane_off;     // byte offset of the lane's channels inside the tile's row segment
+  bool col_ok;           // the lane's channels exist (d % VEC == 0, so all or none)
+  float2 *lds_map;       // [wave][v][lane] = (A, B) of this tile
+  float2 *lds_pred;      // [look wave][v][lane] = what an earlier chunk offers
+  float *lds_hin;        // [v][lane] = the chunk's incoming state, for every wave to read
+  uint32_t *s_kind;      // [look wave] kind of that offer
+  uint32_t *s_resolved;  // look-back finished (one word per workgroup)
+#ifdef FSS_TRACE
+  int trace_wave;
+#endif
+};
+
+// One look at what chunk `j` of this column tile offers: its outgoing state if it
+// has published one, else (j > 0) its map.  Split in two so that other work can be
+// placed between the loads and the use of what they return.
+template <int VEC>
+struct ChunkWords {
+  uint64_t a[VEC], b[VEC], s[VEC];
+};
+
+template <int VEC>
+__device__ __forceinline__ void poll_issue(const ScanArgs &p, const TileCtx &c, int j, ChunkWords<VEC> &w) {
+  const uint64_t *theirs = p.words + (static_cast<size_t>(j) * p.n_ctiles + c.ctile) * 3 * (64 * VEC) + c.lane;
+#pragma unroll
+  for (int v = 0; v < VEC; ++v) {
+    w.s[v] = ld_word(theirs + (2 * VEC + v) * 64);
+    w.a[v] = ld_word(theirs + (0 * VEC + v) * 64);
+    w.b[v] = ld_word(theirs + (1 * VEC + v) * 64);
+  }
+}
+
+// The answer is taken for the whole wave, so that one word per wave can describe
+// it.  Returns kPredNone when neither a state nor a map is there yet.
+template <int VEC>
+__device__ __forceinline__ uint32_t poll_eval(const TileCtx &c, int j, const ChunkWords<VEC> &w, float *qA,
+                                              float *qB) {
+  bool have_state = true, have_map = true;
+#pragma unroll
+  for (int v = 0; v < VEC; ++v) {
+    have_state = have_state && word_tag(w.s[v]) == c.tag;
+    have_map = have_map && word_tag(w.a[v]) == c.tag && word_tag(w.b[v]) == c.tag;
+  }
+  if (__builtin_amdgcn_ballot_w64(have_state) == ~0ull) {
+#pragma unroll
+    for (int v = 0; v < VEC; ++v) {
+      qA[v] = 0.0f;
+      qB[v] = word_val(w.s[v]);
+    }
+    return kPredState;
+  }
+  if (j > 0 && __builtin_amdgcn_ballot_w64(have_map) == ~0ull) {
+#pragma unroll
+    for (int v = 0; v < VEC; ++v) {
+      qA[v] = word_val(w.a[v]);
+      qB[v] = word_val(w.b[v]);
+    }
+    return kPredMap;
+  }
+  return kPredNone;
+}
+
+template <int VEC>
+__device__ __forceinline__ uint32_t poll_chunk(const ScanArgs &p, const TileCtx &c, int j, float *qA,
+                                               float *qB) {
+  ChunkWords<VEC> w;
+  poll_issue<VEC>(p, c, j, w);
+  return poll_eval<VEC>(c, j, w, qA, qB);
+}
+
+// (A, B) <- map[count-1] o ... o map[0] for this lane's channels: the maps of the
+// first `count` waves of the workgroup composed in scan order.  Reads go out in
+// small batches so that their LDS latencies overlap.
+template <int VEC>
+__device__ __forceinline__ void fold_wave_maps(const float2 *lds_map, int lane, int count, float *A,
+                                               float *B) {
+  constexpr int kBatch = 4;
+#pragma unroll
+  for (int v = 0; v < VEC; ++v) {
+    A[v] = 1.0f;
+    B[v] = 0.0f;
+  }
+  for (int w0 = 0; w0 < count; w0 += kBatch) {
+    float2 m[kBatch][VEC];
+#pragma unroll
+    for (int i = 0; i < kBatch; ++i) {
+      const int w = w0 + i < count ? w0 + i : count - 1;  // clamped: the read stays in bounds
+#pragma unroll
+      for (int v = 0; v < VEC; ++v) m[i][v] = lds_map[(w * VEC + v) * 64 + lane];
+    }
+#pragma unroll
+    for (int i = 0; i < kBatch; ++i) {
+      if (w0 + i < count) {
+#pragma unroll
+        for (int v = 0; v < VEC; ++v) {
+          B[v] = __builtin_fmaf(m[i][v].x, B[v], m[i][v].y);
+          A[v] *= m[i][v].x;
+        }
+      }
+    }
+  }
+}
+
+// Phase 2.  In: this wave's slice as the map x -> mA*x + mB.  Out: the state
+// entering the slice.  Every wave of the workgroup must call it (barriers).
+//
+// After one barrier every wave composes the maps of the waves before it (its state
+// is then one multiply-add away from the chunk's incoming state), and wave 0 composes
+// all of them into the chunk's map and publishes it.  Meanwhile wave w (w < look)
+// fetches what chunk-1-w offers - its outgoing state if it has one, else its map -
+// so a look-back over `look` chunks costs one memory round trip instead of one per
+// chunk; wave 0 folds what they found and hands the chunk's incoming state to all
+// waves through LDS.  Chains longer than `look` repeat the fetch.
+template <int VEC>
+__device__ __forceinline__ void chain_chunks(const ScanArgs &p, const TileCtx &c, const float *mA,
+                                             const float *mB, float *state) {
+  constexpr int kLaneSlots = 64 * VEC;
+  const int lane = c.lane, wave = c.wave;
+#pragma unroll
+  for (int v = 0; v < VEC; ++v) c.lds_map[(wave * VEC + v) * 64 + lane] = make_float2(mA[v], mB[v]);
+  __syncthreads();
+  FSS_STAMP(c, p, 2);
+
+  const bool look_back = c.chained && c.chunk > 0;
+  uint64_t *mine = nullptr;
+  float cA[VEC], cB[VEC];
+  if (wave == 0 && c.chained && !c.last) {
+    // the chunk's own map, needed by later chunks: out as early as possible
+    fold_wave_maps<VEC>(c.lds_map, lane, c.n_waves, cA, cB);
+    mine = p.words + (static_cast<size_t>(c.chunk) * p.n_ctiles + c.ctile) * 3 * kLaneSlots + lane;
+    if (c.chunk > 0) {
+#pragma unroll
+      for (int v = 0; v < VEC; ++v) {
+        st_word(mine + (0 * VEC + v) * 64, c.tag, cA[v]);
+        st_word(mine + (1 * VEC + v) * 64, c.tag, cB[v]);
+      }
+    }
+  }
+  FSS_STAMP(c, p, 3);
+
+  // (pA, pB): what the waves before this one do to the chunk's incoming state
+  float pA[VEC], pB[VEC];
+  if (!look_back) fold_wave_maps<VEC>(c.lds_map, lane, wave, pA, pB);
+
+  if (!look_back) {
+    // first chunk of the sequence (or the only one): the incoming state is 0
+    if (wave == 0 && c.chained && !c.last) {
+#pragma unroll
+      for (int v = 0; v < VEC; ++v) st_word(mine + (2 * VEC + v) * 64, c.tag, cB[v]);
+    }
+#pragma unroll
+    for (int v = 0; v < VEC; ++v) state[v] = pB[v];
+    FSS_STAMP(c, p, 5);
+    return;
+  }
+
+  float hin[VEC], accA[VEC], accB[VEC];
+#pragma unroll
+  for (int v = 0; v < VEC; ++v) {
+    accA[v] = 1.0f;
+    accB[v] = hin[v] = 0.0f;
+  }
+  int nearest = c.chunk - 1;  // nearest earlier chunk not folded yet
+  for (;;) {
+    const int j = nearest - wave;
+    if (wave < c.look && j >= 0) {
+      float qA[VEC], qB[VEC];
+      uint32_t kind = kPredNone;
+      uint32_t polls = 0;
+      while ((kind = poll_chunk<VEC>(p, c, j, qA, qB)) == kPredNone) {
+        if (++polls > kSpinLimit) {
+          if (lane == 0) st_u32(p.hdr + HDR_ERROR, 1u);
+          kind = kPredState;  // give up: zero state, so that the grid still drains
+#pragma unroll
+          for (int v = 0; v < VEC; ++v) qA[v] = qB[v] = 0.0f;
+          break;
+        }
+        __builtin_amdgcn_s_sleep(2);
+      }
+#pragma unroll
+      for (int v = 0; v < VEC; ++v) c.lds_pred[(wave * VEC + v) * 64 + lane] = make_float2(qA[v], qB[v]);
+      if (lane == 0) c.s_kind[wave] = kind;
+    }
+    __syncthreads();
+    if (wave == 0) {
+      bool resolved = false;
+      for (int w = 0; w < c.look && nearest - w >= 0 && !resolved; ++w) {
+        const bool is_state = c.s_kind[w] == kPredState;
+#pragma unroll
+        for (int v = 0; v < VEC; ++v) {
+          const float2 m = c.lds_pred[(w * VEC + v) * 64 + lane];
+          if (is_state) {
+            hin[v] = __builtin_fmaf(accA[v], m.y, accB[v]);
+          } else {
+            accB[v] = __builtin_fmaf(accA[v], m.y, accB[v]);
+            accA[v] *= m.x;
+          }
+        }
+        resolved = is_state;
+      }
+      if (resolved) {
+#pragma unroll
+        for (int v = 0; v < VEC; ++v) c.lds_hin[v * 64 + lane] = hin[v];
+        if (!c.last) {
+#pragma unroll
+          for (int v = 0; v < VEC; ++v)
+            st_word(mine + (2 * VEC + v) * 64, c.tag, __builtin_fmaf(cA[v], hin[v], cB[v]));
+        }
+      }
+      if (lane == 0) *c.s_resolved = resolved ? 1u : 0u;
+    }
+    __syncthreads();
+    if (*c.s_resolved != 0u) break;  // chunk 0 always offers a state, so this is reached
+    nearest -= c.look;
+    if (nearest < 0) {  // cannot happen; never spin on a logic error
+      if (threadIdx.x == 0) st_u32(p.hdr + HDR_ERROR, 1u);
+      break;
+    }
+  }
+  FSS_STAMP(c, p, 4);
+  fold_wave_maps<VEC>(c.lds_map, lane, wave, pA, pB);  // after the polls: those are what is waited for
+#pragma unroll
+  for (int v = 0; v < VEC; ++v) state[v] = __builtin_fmaf(pA[v], c.lds_hin[v * 64 + lane], pB[v]);
+  FSS_STAMP(c, p, 5);
+}
+
+// One tile, all three phases.  FULL: every row this wave touches exists and is
+// interior and every lane has channels, so nothing is predicated; otherwise every
+// access is guarded.  The two variants share no registers, so the guarded one
+// costs the fast one nothing.
+template <typename E, int VEC, int STEPS, bool BWD, bool FULL>
+__device__ __forceinline__ void scan_tile(const ScanArgs &p, const TileCtx &c) {
+  using RowT = Row<E, VEC>;
+  const int64_t seq = c.seq, row_bytes = c.row_bytes, r0 = c.r0;
+  const uint32_t lane_off = c.lane_off;
+
+  RowT a[STEPS], b[STEPS];
+  RowT hp[BWD ? STEPS : 1];
+
+  // scan-order index r -> row: forward t = r; backward t = seq-1-r, with alpha taken
+  // from row t+1 and the saved h from row t-1
+  const int64_t t_first = BWD ? seq - 1 - r0 : r0;
+  gcptr_t pa = (gcptr_t)p.in_a + c.tile_base + (BWD ? t_first + 1 : t_first) * row_bytes;
+  gcptr_t pb = (gcptr_t)p.in_b + c.tile_base + t_first * row_bytes;
+  const int64_t step_bytes = BWD ? -row_bytes : row_bytes;  // one step in scan order
+
+  FSS_STAMP(c, p, 0);
+  // ---- phase 1a: issue every load of the slice -------------------------------------
+#pragma unroll
+  for (int s = 0; s < STEPS; ++s) {
+    if (FULL) {
+      a[s].template load<kNtA>(uniform_ptr(pa + s * step_bytes) + lane_off);
+      b[s].template load<kNtB>(uniform_ptr(pb + s * step_bytes) + lane_off);
+    } else {
+      const int64_t r = r0 + s;
+      // Outside the sequence the step is the identity map (a=1, b=0); the first step
+      // of the scan has no predecessor (a=0), whatever alpha holds there.
+      a[s].fill(r >= seq ? 1.0f : 0.0f);
+      b[s].fill(0.0f);
+      if (c.col_ok && r < seq) {
+        if (r >= 1) a[s].template load<kNtA>(uniform_ptr(pa + s * step_bytes) + lane_off);
+        b[s].template load<kNtB>(uniform_ptr(pb + s * step_bytes) + lane_off);
+      }
+    }
+  }
+
+  // the backward's third stream, h[t-1]: only phase 3 needs it, so it goes out last
+  if (BWD) {
+    gcptr_t ph = (gcptr_t)p.in_h + c.tile_base + (t_first - 1) * row_bytes;
+#pragma unroll
+    for (int s = 0; s < STEPS; ++s) {
+      if (FULL) {
+        hp[s].template load<kNtH>(uniform_ptr(ph + s * step_bytes) + lane_off);
+      } else {
+        hp[s].fill(0.0f);
+        if (c.col_ok && r0 + s < seq - 1)  // t - 1 >= 0
+          hp[s].template load<kNtH>(uniform_ptr(ph + s * step_bytes) + lane_off);
+      }
+    }
+  }
+
+
+  float state[VEC];
+  if (!c.chained && c.n_waves == 1) {
+    // the slice is the whole sequence: the state starts at 0, nothing to chain
+#pragma unroll
+    for (int v = 0; v < VEC; ++v) state[v] = 0.0f;
+  } else {
+    // ---- phase 1b: the slice as an affine map ----------------------------------------
+    float mA[VEC], mB[VEC];
+#pragma unroll
+    for (int v = 0; v < VEC; ++v) {
+      mA[v] = 1.0f;
+      mB[v] = 0.0f;
+    }
+#pragma unroll
+    for (int s = 0; s < STEPS; ++s) {
+#pragma unroll
+      for (int v = 0; v < VEC; ++v) {
+        const float av = a[s].get(v);
+        mB[v] = __builtin_fmaf(av, mB[v], b[s].get(v));
+        mA[v] *= av;
+      }
+    }
+    FSS_STAMP(c, p, 1);
+    chain_chunks<VEC>(p, c, mA, mB, state);
+  }
+
+  // ---- phase 3: the recurrence from the true incoming state, in order ---------------
+#pragma unroll
+  for (int s = 0; s < STEPS; ++s) {
+    keep_packed(a[s]);
+    keep_packed(b[s]);
+    if (BWD) keep_packed(hp[s]);
+  }
+  gptr_t po0 = (gptr_t)p.out0 + c.tile_base + t_first * row_bytes;
+  gptr_t po1 = BWD ? (gptr_t)p.out1 + c.tile_base + t_first * row_bytes : (gptr_t) nullptr;
+#pragma unroll
+  for (int s = 0; s < STEPS; ++s) {
+    float ga[VEC];
+#pragma unroll
+    for (int v = 0; v < VEC; ++v) {
+      state[v] = __builtin_fmaf(a[s].get(v), state[v], b[s].get(v));
+      if (BWD) ga[v] = state[v] * hp[s].get(v);
+    }
+    const int64_t r = r0 + s;
+    if (FULL || (c.col_ok && r < seq)) {
+      RowT o;
+      o.pack(state);
+      o.template store<(BWD ? kNtOutBwd : kNtOutFwd)>(uniform_ptr(po0 + s * step_bytes) + lane_off);
+      if (BWD) {
+        if (!FULL && r == seq - 1) {  // t = 0: grad_alpha[0] = 0 whatever the state is
+#pragma unroll
+          for (int v = 0; v < VEC; ++v) ga[v] = 0.0f;
+        }
+        RowT oa;
+        oa.pack(ga);
+        oa.template store<kNtOutBwd>(uniform_ptr(po1 + s * step_bytes) + lane_off);
+      }
+    }
+  }
+  FSS_STAMP(c, p, 6);
+}
+
 template <typename E, int VEC, int STEPS, bool BWD>
 __global__ __launch_bounds__(1024) void scan_kernel(const ScanArgs p) {
-  using RowT = Row<E, VEC>;
-  constexpr int kRowBytes = RowT::kBytes;
   constexpr int kLaneSlots = 64 * VEC;  // channels per tile
 
   extern __shared__ float lds[];
   __shared__ uint32_t s_kind[kMaxLookWaves];
   __shared__ uint32_t s_resolved;
 
-  const int lane = threadIdx.x & 63;
-  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-  const int n_waves = blockDim.x >> 6;
-  const int look = p.look_waves;
-  float2 *lds_map = reinterpret_cast<float2 *>(lds);   // [wave][v][lane] = (A, B), later .x = incoming state
-  float2 *lds_pred = lds_map + n_waves * kLaneSlots;   // [look wave][v][lane] = what an earlier chunk offers
+  TileCtx c;
+  c.lane = threadIdx.x & 63;
+  c.wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  c.n_waves = blockDim.x >> 6;
+  c.look = p.look_waves;
+  // LDS: two sets of per-wave maps (tiles alternate between them, so a wave that runs
+  // ahead into the next tile cannot overwrite a map a slower wave still reads), then
+  // the slots the look-back waves fill, then two rows for the chunk's incoming state
+  float2 *const lds_maps = reinterpret_cast<float2 *>(lds);
+  c.lds_pred = lds_maps + 2 * c.n_waves * kLaneSlots;
+  float *const lds_hins = reinterpret_cast<float *>(c.lds_pred + c.look * kLaneSlots);
+  c.s_kind = s_kind;
+  c.s_resolved = &s_resolved;
+  c.seq = p.seq;
+  c.row_bytes = p.d * E::kBytes;
+  c.lane_off = static_cast<uint32_t>(c.lane * Row<E, VEC>::kBytes);
+#ifdef FSS_TRACE
+  c.trace_wave = FSS_TRACE_WAVE < 0 ? c.n_waves - 1 : FSS_TRACE_WAVE;
+#endif
 
 #ifdef FSS_RESIDENCY_PROBE
   // debug build only: header words 8/9 = workgroups resident now / the most ever seen
@@ -287,304 +721,43 @@ __global__ __launch_bounds__(1024) void scan_kernel(const ScanArgs p) {
     __hip_atomic_fetch_max(p.hdr + 9, now, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   }
 #endif
-  const bool chained = p.n_chunks > 1;
+  c.chained = p.n_chunks > 1;
   // every workgroup of a launch reads the same value: it only changes when all are done
-  const uint32_t tag = chained ? __builtin_amdgcn_readfirstlane(ld_u32(p.hdr + HDR_EPOCH)) : 0u;
-
-  const int64_t seq = p.seq;
-  const int64_t row_bytes = p.d * E::kBytes;
-  const uint32_t lane_off = static_cast<uint32_t>(lane * kRowBytes);
+  c.tag = c.chained ? __builtin_amdgcn_readfirstlane(ld_u32(p.hdr + HDR_EPOCH)) : 0u;
 
   // The grid is sized to be resident all at once; each workgroup walks tiles
   // blockIdx, blockIdx + gridDim, ...  Tiles are numbered chunk-major, so a tile
   // only ever waits for tiles with smaller numbers: those belong to a resident
   // workgroup that reaches them no later than this one reaches its own.
-  for (uint32_t tile = blockIdx.x; tile < static_cast<uint32_t>(p.n_tiles); tile += gridDim.x) {
+  uint32_t parity = 0;
+  for (uint32_t tile = blockIdx.x; tile < static_cast<uint32_t>(p.n_tiles); tile += gridDim.x, parity ^= 1u) {
+    c.lds_map = lds_maps + parity * c.n_waves * kLaneSlots;
+    c.lds_hin = lds_hins + parity * kLaneSlots;
     // unsigned, wave-uniform arithmetic: stays on the scalar unit
-    const uint32_t uchunk = tile / static_cast<uint32_t>(p.n_ctiles);
-    const uint32_t uctile = tile - uchunk * static_cast<uint32_t>(p.n_ctiles);
-    const uint32_t batch = uctile / static_cast<uint32_t>(p.tiles_per_row);
-    const uint32_t coltile = uctile - batch * static_cast<uint32_t>(p.tiles_per_row);
-    const int chunk = static_cast<int>(uchunk);
-    const int ctile = static_cast<int>(uctile);
+    // (the compiler divides through a vector-unit reciprocal: pin the quotients back)
+    const uint32_t chunk = __builtin_amdgcn_readfirstlane(tile / static_cast<uint32_t>(p.n_ctiles));
+    const uint32_t ctile = tile - chunk * static_cast<uint32_t>(p.n_ctiles);
+    const uint32_t batch = __builtin_amdgcn_readfirstlane(ctile / static_cast<uint32_t>(p.tiles_per_row));
+    const uint32_t coltile = ctile - batch * static_cast<uint32_t>(p.tiles_per_row);
+    c.chunk = static_cast<int>(chunk);
+    c.ctile = static_cast<int>(ctile);
+    c.last = c.chunk == p.n_chunks - 1;
 
     const int64_t col0 = static_cast<int64_t>(coltile) * kLaneSlots;  // first channel of the tile
-    const bool col_ok = col0 + lane * VEC < p.d;                       // d % VEC == 0 (host)
-    // byte offset of (batch, row 0, col0); uniform over the wave
-    const int64_t tile_base = (static_cast<int64_t>(batch) * seq * p.d + col0) * E::kBytes;
-    // first scan-order index of this wave's slice (forward: r = t, backward: r = seq-1-t)
-    const int64_t r0 = (static_cast<int64_t>(chunk) * n_waves + wave) * STEPS;
+    c.col_ok = col0 + c.lane * VEC < p.d;
+    c.tile_base = (static_cast<int64_t>(batch) * c.seq * p.d + col0) * E::kBytes;
+    c.r0 = (static_cast<int64_t>(chunk) * c.n_waves + c.wave) * STEPS;
 
-    // Fast path: every row this wave touches exists, is interior, and every lane
-    // has channels.  Forward touches rows r0..r0+STEPS-1 and must not be at r = 0;
-    // backward additionally reads row t+1 and t-1.
-    const bool full = (col0 + kLaneSlots <= p.d) && (r0 >= 1) &&
-                      (BWD ? (r0 + STEPS <= seq - 1) : (r0 + STEPS <= seq));
-
-    RowT a[STEPS], b[STEPS];
-    RowT hp[BWD ? STEPS : 1];
-
-    // ---- phase 1a: issue every load of the slice ----------------------------------
-    if (full) {
-      if (!BWD) {
-        const char *pa = p.in_a + tile_base + r0 * row_bytes;
-        const char *pb = p.in_b + tile_base + r0 * row_bytes;
-#pragma unroll
-        for (int s = 0; s < STEPS; ++s) {
-          a[s].load(uniform_ptr(pa + s * row_bytes) + lane_off);
-          b[s].load(uniform_ptr(pb + s * row_bytes) + lane_off);
-        }
-      } else {
-        // t = seq-1-r: alpha row t+1, dout row t, h row t-1
-        const int64_t t0 = seq - 1 - r0;
-        const char *pa = p.in_a + tile_base + (t0 + 1) * row_bytes;
-        const char *pb = p.in_b + tile_base + t0 * row_bytes;
-        const char *ph = p.in_h + tile_base + (t0 - 1) * row_bytes;
-#pragma unroll
-        for (int s = 0; s < STEPS; ++s) {
-          a[s].load(uniform_ptr(pa - s * row_bytes) + lane_off);
-          b[s].load(uniform_ptr(pb - s * row_bytes) + lane_off);
-        }
-#pragma unroll
-        for (int s = 0; s < STEPS; ++s) hp[s].load(uniform_ptr(ph - s * row_bytes) + lane_off);
-      }
-    } else {
-#pragma unroll
-      for (int s = 0; s < STEPS; ++s) {
-        const int64_t r = r0 + s;
-        const int64_t t = BWD ? seq - 1 - r : r;
-        // Outside the sequence the step is the identity map (a=1, b=0); the first
-        // step of the scan has no predecessor (a=0), whatever alpha holds there.
-        a[s].fill(r >= seq ? 1.0f : 0.0f);
-        b[s].fill(0.0f);
-        if (BWD) hp[s].fill(0.0f);
-        if (col_ok && r < seq) {
-          if (r >= 1) a[s].load(uniform_ptr(p.in_a + tile_base + (BWD ? t + 1 : t) * row_bytes) + lane_off);
-          b[s].load(uniform_ptr(p.in_b + tile_base + t * row_bytes) + lane_off);
-          if (BWD && t >= 1) hp[s].load(uniform_ptr(p.in_h + tile_base + (t - 1) * row_bytes) + lane_off);
-        }
-      }
-    }
-
-    float state[VEC];
-    const bool solo = !chained && n_waves == 1;  // the slice is the whole sequence: state starts at 0
-    if (solo) {
-#pragma unroll
-      for (int v = 0; v < VEC; ++v) state[v] = 0.0f;
-    } else {
-      // ---- phase 1b: the slice as an affine map --------------------------------------
-      float mA[VEC], mB[VEC];
-#pragma unroll
-      for (int v = 0; v < VEC; ++v) {
-        mA[v] = 1.0f;
-        mB[v] = 0.0f;
-      }
-#pragma unroll
-      for (int s = 0; s < STEPS; ++s) {
-#pragma unroll
-        for (int v = 0; v < VEC; ++v) {
-          const float av = a[s].get(v);
-          mB[v] = __builtin_fmaf(av, mB[v], b[s].get(v));
-          mA[v] *= av;
-        }
-      }
-#pragma unroll
-      for (int v = 0; v < VEC; ++v)
-        lds_map[(wave * VEC + v) * 64 + lane] = make_float2(mA[v], mB[v]);
-      __syncthreads();
-
-      // ---- phase 2: compose the waves, chain the chunks --------------------------------
-      // Wave 0 folds the waves' maps into the chunk's map and publishes it.  Meanwhile
-      // wave w (w < look) fetches what chunk-1-w offers - its outgoing state if it has
-      // one, else its map - so a look-back over `look` chunks costs one memory round
-      // trip instead of one per chunk.  Chains longer than that repeat the step.
-      const bool last = chunk == p.n_chunks - 1;
-      uint64_t *mine = nullptr;
-      float cA[VEC], cB[VEC], hin[VEC], accA[VEC], accB[VEC];
-#pragma unroll
-      for (int v = 0; v < VEC; ++v) {
-        cA[v] = accA[v] = 1.0f;
-        cB[v] = accB[v] = hin[v] = 0.0f;
-      }
-      if (wave == 0) {
-        for (int w = 0; w < n_waves; ++w) {
-#pragma unroll
-          for (int v = 0; v < VEC; ++v) {
-            const float2 m = lds_map[(w * VEC + v) * 64 + lane];
-            cB[v] = __builtin_fmaf(m.x, cB[v], m.y);
-            cA[v] *= m.x;
-          }
-        }
-        if (chained) {
-          mine = p.words + (static_cast<size_t>(chunk) * p.n_ctiles + ctile) * 3 * kLaneSlots + lane;
-          if (chunk > 0 && !last) {
-#pragma unroll
-            for (int v = 0; v < VEC; ++v) {
-              st_word(mine + (0 * VEC + v) * 64, tag, cA[v]);
-              st_word(mine + (1 * VEC + v) * 64, tag, cB[v]);
-            }
-          }
-        }
-      }
-      if (chained && chunk > 0) {
-        int nearest = chunk - 1;  // nearest earlier chunk not folded yet
-        for (;;) {
-          const int j = nearest - wave;
-          if (wave < look && j >= 0) {
-            const uint64_t *theirs =
-                p.words + (static_cast<size_t>(j) * p.n_ctiles + ctile) * 3 * kLaneSlots + lane;
-            float pA[VEC], pB[VEC];
-            uint32_t kind = kPredNone;
-            uint32_t polls = 0;
-            while (kind == kPredNone) {
-              uint64_t wa[VEC], wb[VEC], ws[VEC];
-#pragma unroll
-              for (int v = 0; v < VEC; ++v) {
-                ws[v] = ld_word(theirs + (2 * VEC + v) * 64);
-                wa[v] = ld_word(theirs + (0 * VEC + v) * 64);
-                wb[v] = ld_word(theirs + (1 * VEC + v) * 64);
-              }
-              bool have_state = true, have_map = true;
-#pragma unroll
-              for (int v = 0; v < VEC; ++v) {
-                have_state = have_state && word_tag(ws[v]) == tag;
-                have_map = have_map && word_tag(wa[v]) == tag && word_tag(wb[v]) == tag;
-              }
-              // decide for the whole wave, so that one word per wave describes the slot
-              if (__builtin_amdgcn_ballot_w64(have_state) == ~0ull) {
-                kind = kPredState;
-#pragma unroll
-                for (int v = 0; v < VEC; ++v) {
-                  pA[v] = 0.0f;
-                  pB[v] = word_val(ws[v]);
-                }
-              } else if (j > 0 && __builtin_amdgcn_ballot_w64(have_map) == ~0ull) {
-                kind = kPredMap;
-#pragma unroll
-                for (int v = 0; v < VEC; ++v) {
-                  pA[v] = word_val(wa[v]);
-                  pB[v] = word_val(wb[v]);
-                }
-              } else if (++polls > kSpinLimit) {
-                if (lane == 0) st_u32(p.hdr + HDR_ERROR, 1u);
-                kind = kPredState;  // give up: zero state, so that the grid still drains
-#pragma unroll
-                for (int v = 0; v < VEC; ++v) pA[v] = pB[v] = 0.0f;
-              } else {
-                __builtin_amdgcn_s_sleep(2);
-              }
-            }
-#pragma unroll
-            for (int v = 0; v < VEC; ++v)
-              lds_pred[(wave * VEC + v) * 64 + lane] = make_float2(pA[v], pB[v]);
-            if (lane == 0) s_kind[wave] = kind;
-          }
-          __syncthreads();
-          if (wave == 0) {
-            bool resolved = false;
-            for (int w = 0; w < look && nearest - w >= 0 && !resolved; ++w) {
-              const bool is_state = s_kind[w] == kPredState;
-#pragma unroll
-              for (int v = 0; v < VEC; ++v) {
-                const float2 m = lds_pred[(w * VEC + v) * 64 + lane];
-                if (is_state) {
-                  hin[v] = __builtin_fmaf(accA[v], m.y, accB[v]);
-                } else {
-                  accB[v] = __builtin_fmaf(accA[v], m.y, accB[v]);
-                  accA[v] *= m.x;
-                }
-              }
-              resolved = is_state;
-            }
-            if (lane == 0) s_resolved = resolved ? 1u : 0u;
-          }
-          __syncthreads();
-          if (s_resolved != 0u) break;  // chunk 0 always offers a state, so this is reached
-          nearest -= look;
-        }
-      }
-
-      if (wave == 0) {
-        if (chained && !last) {
-#pragma unroll
-          for (int v = 0; v < VEC; ++v)
-            st_word(mine + (2 * VEC + v) * 64, tag, __builtin_fmaf(cA[v], hin[v], cB[v]));
-        }
-        // incoming state of every wave of this tile, left where the wave's map was
-        for (int w = 0; w < n_waves; ++w) {
-#pragma unroll
-          for (int v = 0; v < VEC; ++v) {
-            const float2 m = lds_map[(w * VEC + v) * 64 + lane];
-            lds_map[(w * VEC + v) * 64 + lane].x = hin[v];
-            hin[v] = __builtin_fmaf(m.x, hin[v], m.y);
-          }
-        }
-      }
-      __syncthreads();
-#pragma unroll
-      for (int v = 0; v < VEC; ++v) state[v] = lds_map[(wave * VEC + v) * 64 + lane].x;
-    }
-
-    // ---- phase 3: the recurrence from the true incoming state, in order -------------
-#pragma unroll
-    for (int s = 0; s < STEPS; ++s) {
-      keep_packed(a[s]);
-      keep_packed(b[s]);
-      if (BWD) keep_packed(hp[s]);
-    }
-    if (full) {
-      if (!BWD) {
-        char *po = p.out0 + tile_base + r0 * row_bytes;
-#pragma unroll
-        for (int s = 0; s < STEPS; ++s) {
-#pragma unroll
-          for (int v = 0; v < VEC; ++v) state[v] = __builtin_fmaf(a[s].get(v), state[v], b[s].get(v));
-          RowT o;
-          o.pack(state);
-          o.store(uniform_ptr(po + s * row_bytes) + lane_off);
-        }
-      } else {
-        const int64_t t0 = seq - 1 - r0;
-        char *pgb = p.out0 + tile_base + t0 * row_bytes;
-        char *pga = p.out1 + tile_base + t0 * row_bytes;
-#pragma unroll
-        for (int s = 0; s < STEPS; ++s) {
-          float ga[VEC];
-#pragma unroll
-          for (int v = 0; v < VEC; ++v) {
-            state[v] = __builtin_fmaf(a[s].get(v), state[v], b[s].get(v));
-            ga[v] = state[v] * hp[s].get(v);
-          }
-          RowT ob, oa;
-          ob.pack(state);
-          oa.pack(ga);
-          ob.store(uniform_ptr(pgb - s * row_bytes) + lane_off);
-          oa.store(uniform_ptr(pga - s * row_bytes) + lane_off);
-        }
-      }
-    } else {
-#pragma unroll
-      for (int s = 0; s < STEPS; ++s) {
-        const int64_t r = r0 + s;
-        const int64_t t = BWD ? seq - 1 - r : r;
-        float ga[VEC];
-#pragma unroll
-        for (int v = 0; v < VEC; ++v) {
-          state[v] = __builtin_fmaf(a[s].get(v), state[v], b[s].get(v));
-          if (BWD) ga[v] = (t >= 1) ? state[v] * hp[s].get(v) : 0.0f;  // grad_alpha[0] = 0
-        }
-        if (col_ok && r < seq) {
-          RowT o;
-          o.pack(state);
-          o.store(uniform_ptr(p.out0 + tile_base + t * row_bytes) + lane_off);
-          if (BWD) {
-            RowT oa;
-            oa.pack(ga);
-            oa.store(uniform_ptr(p.out1 + tile_base + t * row_bytes) + lane_off);
-          }
-        }
-      }
-    }
+    // Forward touches rows r0..r0+STEPS-1 and must not be at r = 0 (alpha[0] is never
+    // read); the backward additionally reads row t+1 and row t-1.
+    const bool full = (col0 + kLaneSlots <= p.d) && (c.r0 >= 1) &&
+                      (BWD ? (c.r0 + STEPS <= c.seq - 1) : (c.r0 + STEPS <= c.seq));
+    // wave-uniform, but waves of one workgroup may differ: both variants execute the
+    // same barriers, so they meet
+    if (full)
+      scan_tile<E, VEC, STEPS, BWD, true>(p, c);
+    else
+      scan_tile<E, VEC, STEPS, BWD, false>(p, c);
   }
 
 #ifdef FSS_RESIDENCY_PROBE
@@ -593,7 +766,7 @@ __global__ __launch_bounds__(1024) void scan_kernel(const ScanArgs p) {
   // Two-level completion count (16 first-level counters on separate lines keep the
   // atomics off one hot address).  Whoever counts last knows that no workgroup will
   // read the workspace again and advances the epoch for the next launch.
-  if (chained && threadIdx.x == 0) {
+  if (c.chained && threadIdx.x == 0) {
     const uint32_t slot = blockIdx.x % kDoneSlots;
     const uint32_t in_slot = (gridDim.x - slot + kDoneSlots - 1) / kDoneSlots;
     uint32_t *counter = p.hdr + HDR_SLOT0 + slot * HDR_SLOT_STRIDE;
@@ -603,7 +776,7 @@ __global__ __launch_bounds__(1024) void scan_kernel(const ScanArgs p) {
       if (add_u32(p.hdr + HDR_DONE, 1u) == slots_used - 1) {
         st_u32(p.hdr + HDR_DONE, 0u);
         // 0 is the tag of never-written words: skip it when the counter wraps
-        st_u32(p.hdr + HDR_EPOCH, tag + 1u == 0u ? 1u : tag + 1u);
+        st_u32(p.hdr + HDR_EPOCH, c.tag + 1u == 0u ? 1u : c.tag + 1u);
       }
     }
   }
@@ -625,22 +798,29 @@ __global__ void copy_kernel(const u32x4 *__restrict__ src, u32x4 *__restrict__ d
 // ---- host side --------------------------------------------------------------------
 
 thread_local int tls_hip_error = 0;
+#ifdef FSS_TRACE
+uint64_t *g_trace = nullptr;
+#ifndef FSS_TRACE_WAVE
+#define FSS_TRACE_WAVE 0
+#endif
+#endif
 
 inline int64_t ceil_div(int64_t a, int64_t b) { return (a + b - 1) / b; }
 
 // Register budget: packed dwords a lane may hold per input tensor.
 inline int max_vec_steps(int dtype) { return dtype == FSS_BF16 ? 64 : 32; }  // vec*steps
 
-// LDS: one (A,B) slot per lane and vector element for every wave, plus the same
-// for every wave that looks back.
+// LDS: one (A,B) slot per lane and vector element for every wave, twice (tiles
+// alternate between two sets), the same for every wave that looks back, and two
+// rows of incoming states.
 constexpr size_t kLdsBudget = 60 * 1024;
 inline int look_waves(int waves, int vec) {
   int look = waves < kMaxLookWaves ? waves : kMaxLookWaves;
-  while (look > 1 && static_cast<size_t>(waves + look) * vec * 512 > kLdsBudget) --look;
+  while (look > 1 && static_cast<size_t>(2 * waves + look + 1) * vec * 512 > kLdsBudget) --look;
   return look;
 }
 inline size_t lds_bytes(int waves, int vec) {
-  return static_cast<size_t>(waves + look_waves(waves, vec)) * vec * 512;
+  return static_cast<size_t>(2 * waves + look_waves(waves, vec) + 1) * vec * 512;
 }
 
 inline bool config_valid(const fss_config &c, int dtype) {
@@ -893,6 +1073,9 @@ int run_scan(int dtype, int dir, const void *alpha, const void *in_b, const void
   args.look_waves = look_waves(pl.cfg.waves, pl.cfg.vec);
   args.hdr = static_cast<uint32_t *>(workspace);
   args.words = workspace ? reinterpret_cast<uint64_t *>(static_cast<char *>(workspace) + kHeaderBytes) : nullptr;
+#ifdef FSS_TRACE
+  args.trace = g_trace;
+#endif
   hipStream_t s = static_cast<hipStream_t>(stream);
   if (dtype == FSS_BF16)
     return dir == FSS_BWD ? launch_typed<BF16, true>(args, pl, s) : launch_typed<BF16, false>(args, pl, s);
@@ -904,6 +1087,10 @@ int run_scan(int dtype, int dir, const void *alpha, const void *in_b, const void
 // ---- C ABI -------------------------------------------------------------------------
 
 extern "C" {
+
+#ifdef FSS_TRACE
+void fss_debug_set_trace(void *p) { fss::g_trace = static_cast<uint64_t *>(p); }
+#endif
 
 int fss_abi_version(void) { return FSS_ABI_VERSION; }
 
