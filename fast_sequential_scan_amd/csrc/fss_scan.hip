@@ -608,19 +608,24 @@ __device__ __forceinline__ void scan_tile(const ScanArgs &p, const TileCtx &c) {
     }
   }
 
-  // the backward's third stream, h[t-1]: only phase 3 needs it, so it goes out last
-  if (BWD) {
-    gcptr_t ph = (gcptr_t)p.in_h + c.tile_base + (t_first - 1) * row_bytes;
-#pragma unroll
-    for (int s = 0; s < STEPS; ++s) {
-      if (FULL) {
+  // The backward's third stream, h[t-1], only feeds phase 3.  Its first kHEarly rows go
+  // out now, behind the other two streams; the rest are loaded during phase 3 into
+  // the registers that the steps already done have released, which is what lets a
+  // lane of the backward hold as many timesteps as one of the forward.
+  constexpr int kHEarly = (BWD && STEPS * Row<E, VEC>::kDwords > 16) ? STEPS / 2 : STEPS;
+  gcptr_t ph = BWD ? (gcptr_t)p.in_h + c.tile_base + (t_first - 1) * row_bytes : (gcptr_t) nullptr;
+  auto load_h = [&](int s) {
+    if (FULL) {
+      hp[s].template load<kNtH>(uniform_ptr(ph + s * step_bytes) + lane_off);
+    } else {
+      hp[s].fill(0.0f);
+      if (c.col_ok && r0 + s < seq - 1)  // t - 1 >= 0
         hp[s].template load<kNtH>(uniform_ptr(ph + s * step_bytes) + lane_off);
-      } else {
-        hp[s].fill(0.0f);
-        if (c.col_ok && r0 + s < seq - 1)  // t - 1 >= 0
-          hp[s].template load<kNtH>(uniform_ptr(ph + s * step_bytes) + lane_off);
-      }
     }
+  };
+  if (BWD) {
+#pragma unroll
+    for (int s = 0; s < kHEarly; ++s) load_h(s);
   }
 
 
@@ -655,7 +660,7 @@ __device__ __forceinline__ void scan_tile(const ScanArgs &p, const TileCtx &c) {
   for (int s = 0; s < STEPS; ++s) {
     keep_packed(a[s]);
     keep_packed(b[s]);
-    if (BWD) keep_packed(hp[s]);
+    if (BWD && s < kHEarly) keep_packed(hp[s]);
   }
   gptr_t po0 = (gptr_t)p.out0 + c.tile_base + t_first * row_bytes;
   gptr_t po1 = BWD ? (gptr_t)p.out1 + c.tile_base + t_first * row_bytes : (gptr_t) nullptr;
@@ -682,6 +687,7 @@ __device__ __forceinline__ void scan_tile(const ScanArgs &p, const TileCtx &c) {
         oa.template store<kNtOutBwd>(uniform_ptr(po1 + s * step_bytes) + lane_off);
       }
     }
+    if (BWD && s + kHEarly < STEPS) load_h(s + kHEarly);
   }
   FSS_STAMP(c, p, 6);
 }
@@ -859,7 +865,7 @@ void complete_config(fss_config &c, int64_t bs, int64_t seq, int64_t d, int dtyp
   // packed dwords one lane holds per timestep and tensor
   const int dwords = dtype == FSS_BF16 ? (c.vec + 1) / 2 : c.vec;
   if (c.steps == 0) {
-    int s = (dir == FSS_BWD ? 16 : 32) / dwords;  // 2 (forward) or 3 (backward) tensors stay in registers
+    int s = 32 / dwords;  // 32 packed dwords per lane and tensor (the backward loads half of its third one late)
     if (s > 32) s = 32;
     if (s < 8) s = 8;
     // small problems: shorter slices until the machine has a few waves per SIMD
