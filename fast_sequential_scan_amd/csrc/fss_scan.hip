@@ -856,7 +856,8 @@ void complete_config(fss_config &c, int64_t bs, int64_t seq, int64_t d, int dtyp
   const int esize = dtype == FSS_BF16 ? 2 : 4;
   const int64_t channels = bs * d;
   if (c.vec == 0) {
-    const bool can2 = d % 2 == 0 && align % (2 * static_cast<size_t>(esize)) == 0;
+    // 4 bytes per lane and load either way: two bf16 channels or one fp32 channel
+    const bool can2 = dtype == FSS_BF16 && d % 2 == 0 && align % (2 * static_cast<size_t>(esize)) == 0;
     int v = can2 ? 2 : 1;
     // few channels: more, narrower column tiles; also never pad a row to twice its width
     if (v == 2 && (channels < 8192 || ceil_div(d, 128) * 128 >= 2 * ceil_div(d, 64) * 64)) v = 1;
@@ -868,8 +869,10 @@ void complete_config(fss_config &c, int64_t bs, int64_t seq, int64_t d, int dtyp
     int s = 32 / dwords;  // 32 packed dwords per lane and tensor (the backward loads half of its third one late)
     if (s > 32) s = 32;
     if (s < 8) s = 8;
-    // small problems: shorter slices until the machine has a few waves per SIMD
+    // small problems: shorter slices until there are two 8-wave tiles per CU (512), as
+    // long as the machine still gets a few waves per SIMD out of it
     const int64_t ctiles = bs * ceil_div(d, 64 * c.vec);
+    while (s > 16 && ctiles * ceil_div(seq, static_cast<int64_t>(8) * s) < 512) s >>= 1;
     while (s > 8 && ctiles * ceil_div(seq, s) < 1024) s >>= 1;
     // never longer than the sequence needs
     while (s > 8 && seq <= s / 2) s >>= 1;
@@ -880,6 +883,10 @@ void complete_config(fss_config &c, int64_t bs, int64_t seq, int64_t d, int dtyp
     // long chains of chunks (few channels, long sequence): the largest tile
     const int64_t cap = ceil_div(seq, static_cast<int64_t>(8) * c.steps) > 64 ? 16 : 8;
     if (w > cap) w = cap;
+    // many channels but a short sequence: half-size workgroups to reach 512 tiles
+    if (w == 8 && bs * ceil_div(d, 64 * c.vec) >= 64 &&
+        bs * ceil_div(d, 64 * c.vec) * ceil_div(seq, static_cast<int64_t>(8) * c.steps) < 512)
+      w = 4;
     while (w > 1 && lds_bytes(static_cast<int>(w), c.vec) > kLdsBudget) --w;
     c.waves = static_cast<int32_t>(w);
   }

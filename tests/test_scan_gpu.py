@@ -362,3 +362,40 @@ def test_c_abi_rejects_bad_arguments():
     odd = _native.FssConfig(2, 8, 1, 0)  # vec 2 needs 4-byte alignment
     assert lib.fss_scan_fwd_ex(0, a.data_ptr() + 2, a.data_ptr(), a.data_ptr(), 1, 8, 64, None, 0, s, ctypes.byref(odd)) == 3
     torch.cuda.synchronize()
+
+
+def test_hip_graph_replays_match_eager(oracle):
+    """A captured forward+backward step replays correctly: the chaining workspace keeps its
+    launch counter on the device, so every replay sees fresh tags.  Replays alternate with
+    eager launches and synchronisations, and each replay is checked."""
+    alpha, beta, dout = make_inputs("sigmoid", 4, 3000, 256, seed=81)
+    a, b, do = alpha.to(DEV), beta.to(DEV), dout.to(DEV)
+    h_ref, ga_ref, gb_ref = run_bf16(alpha, beta, dout)
+    lib = _native.lib()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        sp = side.cuda_stream
+        ws = torch.empty(lib.fss_workspace_bytes_max(*a.shape), dtype=torch.uint8, device=DEV)
+        _native.check(lib.fss_workspace_init(ws.data_ptr(), ws.numel(), sp))
+        h, ga, gb = torch.empty_like(a), torch.empty_like(a), torch.empty_like(a)
+
+        def step():
+            _native.check(lib.fss_scan_fwd_bf16(a.data_ptr(), b.data_ptr(), h.data_ptr(), *a.shape,
+                                                ws.data_ptr(), ws.numel(), sp))
+            _native.check(lib.fss_scan_bwd_bf16(a.data_ptr(), h.data_ptr(), do.data_ptr(), ga.data_ptr(),
+                                                gb.data_ptr(), *a.shape, ws.data_ptr(), ws.numel(), sp))
+
+        step()  # warm: device check, residency query
+        side.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph, stream=side):
+            step()
+        for i in range(5):
+            h.zero_(), ga.zero_(), gb.zero_()
+            graph.replay()
+            side.synchronize()
+            assert torch.equal(h, h_ref) and torch.equal(ga, ga_ref) and torch.equal(gb, gb_ref), i
+            step()  # eager work between replays, same workspace
+            side.synchronize()
+        assert lib.fss_workspace_status(ws.data_ptr(), sp) == 0
