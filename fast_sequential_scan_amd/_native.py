@@ -34,6 +34,8 @@ EXPORTED_SYMBOLS = (
     "fss_scan_bwd_f32",
     "fss_scan_fwd_ex",
     "fss_scan_bwd_ex",
+    "fss_scan_fwd_state",
+    "fss_scan_bwd_state",
     "fss_copy_bytes",
 )
 
@@ -93,6 +95,10 @@ def _declare(lib: ctypes.CDLL) -> None:
     lib.fss_scan_fwd_ex.argtypes = [_int] + fwd + [_cfgp]
     lib.fss_scan_bwd_ex.restype = _int
     lib.fss_scan_bwd_ex.argtypes = [_int] + bwd + [_cfgp]
+    lib.fss_scan_fwd_state.restype = _int
+    lib.fss_scan_fwd_state.argtypes = [_int, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _vp, _sz, _vp, _cfgp]
+    lib.fss_scan_bwd_state.restype = _int
+    lib.fss_scan_bwd_state.argtypes = [_int, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _vp, _sz, _vp, _cfgp]
     lib.fss_copy_bytes.restype = _int
     lib.fss_copy_bytes.argtypes = [_vp, _vp, _sz, _vp]
 

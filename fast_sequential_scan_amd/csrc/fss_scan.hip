@@ -305,6 +305,22 @@ struct ScanArgs {
 #endif
 };
 
+// Optional (bs, d) fp32 rows of the scans with a state entering/leaving the sequence.
+// The plain scan is compiled against the empty variant, whose members are constant
+// nulls: it carries no kernel arguments for them and every use folds away.
+template <bool STATE>
+struct StateArgs {
+  const float *state_in;  // forward: h[-1]; backward: gradient reaching the state after the last step
+  float *state_out;       // forward: un-rounded state after the last step; backward: gradient w.r.t. h[-1]
+  const float *h_before;  // backward only: h[-1] of the forward (grad_alpha[0] = g[0] * h[-1])
+};
+template <>
+struct StateArgs<false> {
+  static constexpr const float *state_in = nullptr;
+  static constexpr float *state_out = nullptr;
+  static constexpr const float *h_before = nullptr;
+};
+
 // ---- the kernel ----------------------------------------------------------------
 
 // Which streams are accessed non-temporally (bit 0: alpha, 1: beta/dout, 2: saved h,
@@ -341,6 +357,7 @@ struct TileCtx {
   bool chained, last;    // more than one chunk in the sequence; this is the last one
   uint32_t tag;          // epoch of this launch
   int64_t tile_base;     // byte offset of (batch, row 0, first channel of the tile)
+  int64_t chan_row;      // index of (batch, first channel of the tile) in a (bs, d) array; wave-uniform
   int64_t r0;            // first scan-order index of this wave's slice
   int64_t seq, row_bytes;
   uint32_t lane_off;     // byte offset of the lane's channels inside the tile's row segment
@@ -457,7 +474,7 @@ __device__ __forceinline__ void fold_wave_maps(const float2 *lds_map, int lane, 
 // waves through LDS.  Chains longer than `look` repeat the fetch.
 template <int VEC>
 __device__ __forceinline__ void chain_chunks(const ScanArgs &p, const TileCtx &c, const float *mA,
-                                             const float *mB, float *state) {
+                                             const float *mB, const float *seq_in, float *state) {
   constexpr int kLaneSlots = 64 * VEC;
   const int lane = c.lane, wave = c.wave;
 #pragma unroll
@@ -487,13 +504,15 @@ __device__ __forceinline__ void chain_chunks(const ScanArgs &p, const TileCtx &c
   if (!look_back) fold_wave_maps<VEC>(c.lds_map, lane, wave, pA, pB);
 
   if (!look_back) {
-    // first chunk of the sequence (or the only one): the incoming state is 0
+    // first chunk of the sequence (or the only one): the incoming state is the
+    // sequence's own (0 in the plain scan)
     if (wave == 0 && c.chained && !c.last) {
 #pragma unroll
-      for (int v = 0; v < VEC; ++v) st_word(mine + (2 * VEC + v) * 64, c.tag, cB[v]);
+      for (int v = 0; v < VEC; ++v)
+        st_word(mine + (2 * VEC + v) * 64, c.tag, seq_in ? __builtin_fmaf(cA[v], seq_in[v], cB[v]) : cB[v]);
     }
 #pragma unroll
-    for (int v = 0; v < VEC; ++v) state[v] = pB[v];
+    for (int v = 0; v < VEC; ++v) state[v] = seq_in ? __builtin_fmaf(pA[v], seq_in[v], pB[v]) : pB[v];
     FSS_STAMP(c, p, 5);
     return;
   }
@@ -572,8 +591,8 @@ __device__ __forceinline__ void chain_chunks(const ScanArgs &p, const TileCtx &c
 // interior and every lane has channels, so nothing is predicated; otherwise every
 // access is guarded.  The two variants share no registers, so the guarded one
 // costs the fast one nothing.
-template <typename E, int VEC, int STEPS, bool BWD, bool FULL>
-__device__ __forceinline__ void scan_tile(const ScanArgs &p, const TileCtx &c) {
+template <typename E, int VEC, int STEPS, bool BWD, bool STATE, bool FULL>
+__device__ __forceinline__ void scan_tile(const ScanArgs &p, const StateArgs<STATE> &st, const TileCtx &c) {
   using RowT = Row<E, VEC>;
   const int64_t seq = c.seq, row_bytes = c.row_bytes, r0 = c.r0;
   const uint32_t lane_off = c.lane_off;
@@ -597,12 +616,14 @@ __device__ __forceinline__ void scan_tile(const ScanArgs &p, const TileCtx &c) {
       b[s].template load<kNtB>(uniform_ptr(pb + s * step_bytes) + lane_off);
     } else {
       const int64_t r = r0 + s;
-      // Outside the sequence the step is the identity map (a=1, b=0); the first step
-      // of the scan has no predecessor (a=0), whatever alpha holds there.
-      a[s].fill(r >= seq ? 1.0f : 0.0f);
+      // Outside the sequence the step is the identity map (a=1, b=0).  The first step
+      // of the plain scan has no predecessor (a=0), whatever alpha holds there; with a
+      // state coming in, the forward applies alpha[0] to it and the backward adds it (a=1).
+      a[s].fill((r >= seq || (STATE && BWD && r == 0 && st.state_in)) ? 1.0f : 0.0f);
       b[s].fill(0.0f);
       if (c.col_ok && r < seq) {
-        if (r >= 1) a[s].template load<kNtA>(uniform_ptr(pa + s * step_bytes) + lane_off);
+        if (r >= 1 || (STATE && !BWD && st.state_in))
+          a[s].template load<kNtA>(uniform_ptr(pa + s * step_bytes) + lane_off);
         b[s].template load<kNtB>(uniform_ptr(pb + s * step_bytes) + lane_off);
       }
     }
@@ -629,11 +650,20 @@ __device__ __forceinline__ void scan_tile(const ScanArgs &p, const TileCtx &c) {
   }
 
 
+  // the state the whole sequence starts from: only its first chunk needs it
+  float seq_in[VEC];
+#pragma unroll
+  for (int v = 0; v < VEC; ++v) seq_in[v] = 0.0f;
+  if (STATE && st.state_in && c.chunk == 0 && c.col_ok) {
+#pragma unroll
+    for (int v = 0; v < VEC; ++v) seq_in[v] = st.state_in[c.chan_row + c.lane * VEC + v];
+  }
+
   float state[VEC];
   if (!c.chained && c.n_waves == 1) {
-    // the slice is the whole sequence: the state starts at 0, nothing to chain
+    // the slice is the whole sequence: nothing to chain
 #pragma unroll
-    for (int v = 0; v < VEC; ++v) state[v] = 0.0f;
+    for (int v = 0; v < VEC; ++v) state[v] = seq_in[v];
   } else {
     // ---- phase 1b: the slice as an affine map ----------------------------------------
     float mA[VEC], mB[VEC];
@@ -652,7 +682,7 @@ __device__ __forceinline__ void scan_tile(const ScanArgs &p, const TileCtx &c) {
       }
     }
     FSS_STAMP(c, p, 1);
-    chain_chunks<VEC>(p, c, mA, mB, state);
+    chain_chunks<VEC>(p, c, mA, mB, STATE ? seq_in : nullptr, state);
   }
 
   // ---- phase 3: the recurrence from the true incoming state, in order ---------------
@@ -678,9 +708,10 @@ __device__ __forceinline__ void scan_tile(const ScanArgs &p, const TileCtx &c) {
       o.pack(state);
       o.template store<(BWD ? kNtOutBwd : kNtOutFwd)>(uniform_ptr(po0 + s * step_bytes) + lane_off);
       if (BWD) {
-        if (!FULL && r == seq - 1) {  // t = 0: grad_alpha[0] = 0 whatever the state is
+        if (!FULL && r == seq - 1) {  // t = 0: grad_alpha[0] = g[0] * h[-1], 0 in the plain scan
 #pragma unroll
-          for (int v = 0; v < VEC; ++v) ga[v] = 0.0f;
+          for (int v = 0; v < VEC; ++v)
+            ga[v] = (STATE && st.h_before) ? state[v] * st.h_before[c.chan_row + c.lane * VEC + v] : 0.0f;
         }
         RowT oa;
         oa.pack(ga);
@@ -689,11 +720,27 @@ __device__ __forceinline__ void scan_tile(const ScanArgs &p, const TileCtx &c) {
     }
     if (BWD && s + kHEarly < STEPS) load_h(s + kHEarly);
   }
+  // The wave whose slice holds the last step of the scan hands out the final state: the
+  // forward as it is (the steps past the end are identity maps), the backward times
+  // alpha[0] (the gradient with respect to h[-1]).
+  if (STATE && st.state_out && c.col_ok && r0 <= seq - 1 && seq - 1 < r0 + STEPS) {
+    if (BWD) {
+      RowT a0;
+      a0.template load<false>((gcptr_t)p.in_a + c.tile_base + lane_off);
+#pragma unroll
+      for (int v = 0; v < VEC; ++v) st.state_out[c.chan_row + c.lane * VEC + v] = a0.get(v) * state[v];
+    } else {
+#pragma unroll
+      for (int v = 0; v < VEC; ++v) st.state_out[c.chan_row + c.lane * VEC + v] = state[v];
+    }
+  }
   FSS_STAMP(c, p, 6);
 }
 
-template <typename E, int VEC, int STEPS, bool BWD>
-__global__ __launch_bounds__(1024) void scan_kernel(const ScanArgs p) {
+// STATE: the variant that honours the optional incoming/outgoing state rows of ScanArgs;
+// the plain scan is compiled without them.
+template <typename E, int VEC, int STEPS, bool BWD, bool STATE>
+__global__ __launch_bounds__(1024) void scan_kernel(const ScanArgs p, const StateArgs<STATE> st) {
   constexpr int kLaneSlots = 64 * VEC;  // channels per tile
 
   extern __shared__ float lds[];
@@ -752,6 +799,7 @@ __global__ __launch_bounds__(1024) void scan_kernel(const ScanArgs p) {
     const int64_t col0 = static_cast<int64_t>(coltile) * kLaneSlots;  // first channel of the tile
     c.col_ok = col0 + c.lane * VEC < p.d;
     c.tile_base = (static_cast<int64_t>(batch) * c.seq * p.d + col0) * E::kBytes;
+    c.chan_row = static_cast<int64_t>(batch) * p.d + col0;
     c.r0 = (static_cast<int64_t>(chunk) * c.n_waves + c.wave) * STEPS;
 
     // Forward touches rows r0..r0+STEPS-1 and must not be at r = 0 (alpha[0] is never
@@ -761,9 +809,9 @@ __global__ __launch_bounds__(1024) void scan_kernel(const ScanArgs p) {
     // wave-uniform, but waves of one workgroup may differ: both variants execute the
     // same barriers, so they meet
     if (full)
-      scan_tile<E, VEC, STEPS, BWD, true>(p, c);
+      scan_tile<E, VEC, STEPS, BWD, STATE, true>(p, st, c);
     else
-      scan_tile<E, VEC, STEPS, BWD, false>(p, c);
+      scan_tile<E, VEC, STEPS, BWD, STATE, false>(p, st, c);
   }
 
 #ifdef FSS_RESIDENCY_PROBE
@@ -993,8 +1041,8 @@ int resident_workgroups(Kernel kernel, int waves, size_t lds) {
   return per_cu * cu_count;
 }
 
-template <typename E, int VEC, int STEPS, bool BWD>
-int launch_one(const ScanArgs &args, const Plan &pl, hipStream_t stream) {
+template <typename E, int VEC, int STEPS, bool BWD, bool STATE>
+int launch_one(const ScanArgs &args, const StateArgs<true> &state, const Plan &pl, hipStream_t stream) {
   // The kernel's waits are only safe if every workgroup of the grid is resident,
   // so the grid never exceeds what the device holds at once; workgroups loop.
   static int resident[17] = {0};  // by waves per workgroup; same answer on every call
@@ -1002,7 +1050,7 @@ int launch_one(const ScanArgs &args, const Plan &pl, hipStream_t stream) {
   const size_t lds = lds_bytes(waves, VEC);
   int fit = __atomic_load_n(&resident[waves], __ATOMIC_RELAXED);
   if (fit == 0) {
-    fit = resident_workgroups(scan_kernel<E, VEC, STEPS, BWD>, waves, lds);
+    fit = resident_workgroups(scan_kernel<E, VEC, STEPS, BWD, STATE>, waves, lds);
     if (fit <= 0) return FSS_ERR_LAUNCH;
     __atomic_store_n(&resident[waves], fit, __ATOMIC_RELAXED);
   }
@@ -1010,7 +1058,9 @@ int launch_one(const ScanArgs &args, const Plan &pl, hipStream_t stream) {
   if (pl.cfg.max_groups > 0 && pl.cfg.max_groups < n_groups) n_groups = pl.cfg.max_groups;
   const dim3 grid(static_cast<uint32_t>(n_groups));
   const dim3 block(static_cast<uint32_t>(waves) * 64);
-  hipLaunchKernelGGL((scan_kernel<E, VEC, STEPS, BWD>), grid, block, lds, stream, args);
+  StateArgs<STATE> st;
+  if constexpr (STATE) st = state;
+  hipLaunchKernelGGL((scan_kernel<E, VEC, STEPS, BWD, STATE>), grid, block, lds, stream, args, st);
   const hipError_t e = hipGetLastError();
   if (e != hipSuccess) {
     tls_hip_error = static_cast<int>(e);
@@ -1019,14 +1069,14 @@ int launch_one(const ScanArgs &args, const Plan &pl, hipStream_t stream) {
   return FSS_OK;
 }
 
-template <typename E, bool BWD>
-int launch_typed(const ScanArgs &args, const Plan &pl, hipStream_t stream) {
+template <typename E, bool BWD, bool STATE>
+int launch_typed(const ScanArgs &args, const StateArgs<true> &state, const Plan &pl, hipStream_t stream) {
   constexpr bool is_bf16 = E::kBytes == 2;
   const int key = pl.cfg.vec * 100 + pl.cfg.steps;
   switch (key) {
 #define FSS_CASE(V, S) \
   case V * 100 + S:    \
-    return launch_one<E, V, S, BWD>(args, pl, stream);
+    return launch_one<E, V, S, BWD, STATE>(args, state, pl, stream);
     FSS_CASE(1, 8)
     FSS_CASE(1, 16)
     FSS_CASE(1, 32)
@@ -1051,7 +1101,8 @@ int launch_typed(const ScanArgs &args, const Plan &pl, hipStream_t stream) {
 
 int run_scan(int dtype, int dir, const void *alpha, const void *in_b, const void *in_h, void *out0,
              void *out1, int64_t bs, int64_t seq, int64_t d, void *workspace, size_t workspace_bytes,
-             void *stream, const fss_config *cfg) {
+             void *stream, const fss_config *cfg, const float *state_in = nullptr,
+             float *state_out = nullptr, const float *h_before = nullptr) {
   if (bs < 0 || seq < 0 || d < 0) return FSS_ERR_BAD_SHAPE;
   if (dtype != FSS_BF16 && dtype != FSS_F32) return FSS_ERR_BAD_CONFIG;
   if (bs == 0 || seq == 0 || d == 0) return FSS_OK;
@@ -1061,6 +1112,9 @@ int run_scan(int dtype, int dir, const void *alpha, const void *in_b, const void
   const size_t align = dir == FSS_BWD ? common_alignment({alpha, in_b, in_h, out0, out1})
                                       : common_alignment({alpha, in_b, out0});
   if (align < esize) return FSS_ERR_MISALIGNED;
+  if ((reinterpret_cast<uintptr_t>(state_in) | reinterpret_cast<uintptr_t>(state_out) |
+       reinterpret_cast<uintptr_t>(h_before)) % 4 != 0)
+    return FSS_ERR_MISALIGNED;
   Plan pl;
   int rc = make_plan(pl, bs, seq, d, dtype, dir, align, cfg);
   if (rc != FSS_OK) return rc;
@@ -1084,15 +1138,20 @@ int run_scan(int dtype, int dir, const void *alpha, const void *in_b, const void
   args.n_chunks = static_cast<int32_t>(pl.n_chunks);
   args.n_tiles = static_cast<int32_t>(pl.n_tiles);
   args.look_waves = look_waves(pl.cfg.waves, pl.cfg.vec);
+  const StateArgs<true> state = {state_in, state_out, h_before};
   args.hdr = static_cast<uint32_t *>(workspace);
   args.words = workspace ? reinterpret_cast<uint64_t *>(static_cast<char *>(workspace) + kHeaderBytes) : nullptr;
 #ifdef FSS_TRACE
   args.trace = g_trace;
 #endif
   hipStream_t s = static_cast<hipStream_t>(stream);
-  if (dtype == FSS_BF16)
-    return dir == FSS_BWD ? launch_typed<BF16, true>(args, pl, s) : launch_typed<BF16, false>(args, pl, s);
-  return dir == FSS_BWD ? launch_typed<F32, true>(args, pl, s) : launch_typed<F32, false>(args, pl, s);
+  const bool st = state_in || state_out || h_before;
+  if (dtype == FSS_BF16) {
+    if (dir == FSS_BWD) return st ? launch_typed<BF16, true, true>(args, state, pl, s) : launch_typed<BF16, true, false>(args, state, pl, s);
+    return st ? launch_typed<BF16, false, true>(args, state, pl, s) : launch_typed<BF16, false, false>(args, state, pl, s);
+  }
+  if (dir == FSS_BWD) return st ? launch_typed<F32, true, true>(args, state, pl, s) : launch_typed<F32, true, false>(args, state, pl, s);
+  return st ? launch_typed<F32, false, true>(args, state, pl, s) : launch_typed<F32, false, false>(args, state, pl, s);
 }
 
 }  // namespace fss
@@ -1201,6 +1260,22 @@ int fss_scan_bwd_ex(int dtype, const void *alpha, const void *h, const void *dou
                     size_t workspace_bytes, void *stream, const fss_config *cfg) {
   return fss::run_scan(dtype, FSS_BWD, alpha, dout, h, grad_beta, grad_alpha, bs, seq, d, workspace,
                        workspace_bytes, stream, cfg);
+}
+
+int fss_scan_fwd_state(int dtype, const void *alpha, const void *beta, void *h, const float *h_before,
+                       float *h_last, int64_t bs, int64_t seq, int64_t d, void *workspace,
+                       size_t workspace_bytes, void *stream, const fss_config *cfg) {
+  return fss::run_scan(dtype, FSS_FWD, alpha, beta, nullptr, h, nullptr, bs, seq, d, workspace,
+                       workspace_bytes, stream, cfg, h_before, h_last, nullptr);
+}
+
+int fss_scan_bwd_state(int dtype, const void *alpha, const void *h, const void *dout, const float *h_before,
+                       const float *grad_h_last, void *grad_alpha, void *grad_beta, float *grad_h_before,
+                       int64_t bs, int64_t seq, int64_t d, void *workspace, size_t workspace_bytes,
+                       void *stream, const fss_config *cfg) {
+  if (grad_h_before && !h_before) return FSS_ERR_NULL_POINTER;
+  return fss::run_scan(dtype, FSS_BWD, alpha, dout, h, grad_beta, grad_alpha, bs, seq, d, workspace,
+                       workspace_bytes, stream, cfg, grad_h_last, grad_h_before, h_before);
 }
 
 int fss_scan_fwd_bf16(const void *alpha, const void *beta, void *h, int64_t bs, int64_t seq, int64_t d,

@@ -8,7 +8,7 @@ memory (reference scan_cuda.py:20,42) - and the backward returns
 """
 from __future__ import annotations
 
-from typing import Any, Tuple
+from typing import Any, Optional, Tuple
 
 import torch
 from torch.autograd import Function
@@ -16,7 +16,7 @@ from torch.autograd.function import once_differentiable
 
 from . import sequential_scan_cuda as _ext
 
-__all__ = ["SequentialScan", "SequentialScanSingle", "scan", "scan_single"]
+__all__ = ["SequentialScan", "SequentialScanSingle", "SequentialScanState", "scan", "scan_single", "scan_with_state"]
 
 
 class SequentialScan(Function):
@@ -66,3 +66,38 @@ def scan(alpha: torch.Tensor, beta: torch.Tensor) -> torch.Tensor:
 def scan_single(alpha: torch.Tensor, beta: torch.Tensor) -> torch.Tensor:
     """The same recurrence on fp32 tensors."""
     return SequentialScanSingle.apply(alpha, beta)
+
+
+class SequentialScanState(Function):
+    """The scan with a state entering and leaving the sequence: ``(h, h_last) = f(alpha, beta, h_before)``.
+    Not in the reference.  bf16 or fp32 tensors; the states are fp32 ``(bs, d_model)``.  Differentiable
+    in all three inputs, through both outputs."""
+
+    @staticmethod
+    def forward(ctx: Any, alpha: torch.Tensor, beta: torch.Tensor, h_before: Optional[torch.Tensor]):
+        h, h_last = _ext.scan_forward_state(alpha, beta, h_before)
+        ctx.has_state = h_before is not None
+        if ctx.has_state:
+            ctx.save_for_backward(alpha, h, h_before)
+        else:
+            ctx.save_for_backward(alpha, h)
+        return h, h_last
+
+    @staticmethod
+    @once_differentiable
+    def backward(ctx: Any, grad_h: torch.Tensor, grad_h_last: torch.Tensor):
+        if ctx.has_state:
+            alpha, h, h_before = ctx.saved_tensors
+        else:
+            (alpha, h), h_before = ctx.saved_tensors, None
+        grad_alpha, grad_beta, grad_h_before = _ext.scan_backward_state(alpha, h, grad_h, h_before, grad_h_last)
+        return grad_alpha, grad_beta, grad_h_before
+
+
+def scan_with_state(
+    alpha: torch.Tensor, beta: torch.Tensor, h_before: Optional[torch.Tensor] = None
+) -> Tuple[torch.Tensor, torch.Tensor]:
+    """``h[t] = alpha[t]*h[t-1] + beta[t]`` from ``h[-1] = h_before`` (zeros when None; when given,
+    ``alpha[:, 0]`` multiplies it).  Returns ``(h, h_last)`` with ``h_last`` the fp32 state after the
+    last step, to be passed as ``h_before`` of the next segment."""
+    return SequentialScanState.apply(alpha, beta, h_before)

@@ -21,7 +21,10 @@ import torch
 
 from . import _native
 
-__all__ = ["scan_forward", "scan_backward", "scan_forward_half", "scan_backward_half"]
+__all__ = [
+    "scan_forward", "scan_backward", "scan_forward_half", "scan_backward_half",
+    "scan_forward_state", "scan_backward_state",
+]
 
 _DTYPE_CODE = {torch.bfloat16: _native.FSS_BF16, torch.float32: _native.FSS_F32}
 
@@ -150,3 +153,94 @@ def scan_forward_half(alpha: torch.Tensor, beta: torch.Tensor) -> torch.Tensor:
 def scan_backward_half(alpha_saved: torch.Tensor, h_saved: torch.Tensor, grad_out: torch.Tensor) -> List[torch.Tensor]:
     """bf16 backward -> [grad_alpha, grad_beta]: csrc/sequential_scan.cpp:21 / sequential_scan_kernel.cu:189-268."""
     return _backward(torch.bfloat16, alpha_saved, h_saved, grad_out)
+
+
+# ---- scans with a state entering and leaving the sequence (no counterpart in the reference) ----
+
+
+def _state(name: str, t: Optional[torch.Tensor], like: torch.Tensor) -> Optional[torch.Tensor]:
+    if t is None:
+        return None
+    bs, _, d = like.shape
+    if not t.is_cuda or t.device != like.device:
+        raise RuntimeError(f"{name} must be on {like.device}")
+    if t.dtype != torch.float32:
+        raise RuntimeError(f"expected scalar type torch.float32 for {name} but found {t.dtype}")
+    if tuple(t.shape) != (bs, d):
+        raise RuntimeError(f"{name} must have shape (bs, d_model) = {(bs, d)}, got {tuple(t.shape)}")
+    return t.contiguous()
+
+
+def scan_forward_state(
+    alpha: torch.Tensor, beta: torch.Tensor, h_before: Optional[torch.Tensor] = None, config=None
+) -> Tuple[torch.Tensor, torch.Tensor]:
+    """(h, h_last): the scan started from ``h[-1] = h_before`` (fp32 ``(bs, d)``, zeros when None;
+    given, ``alpha[:, 0]`` is applied to it) and the un-rounded fp32 state after the last step."""
+    dtype = alpha.dtype
+    if dtype not in _DTYPE_CODE:
+        raise RuntimeError(f"expected scalar type torch.bfloat16 or torch.float32 for alpha but found {dtype}")
+    bs, seq, d = _validate(dtype, alpha=alpha, beta=beta)
+    h_before = _state("h_before", h_before, alpha)
+    alpha, beta = alpha.contiguous(), beta.contiguous()
+    out = torch.empty_like(alpha, memory_format=torch.contiguous_format)
+    h_last = torch.zeros((bs, d), dtype=torch.float32, device=alpha.device)
+    if out.numel() == 0:
+        if h_before is not None and seq == 0:
+            h_last.copy_(h_before)
+        return out, h_last
+    lib = _native.lib()
+    code = _DTYPE_CODE[dtype]
+    with torch.cuda.device(alpha.device):
+        stream = torch.cuda.current_stream()
+        need = lib.fss_workspace_bytes(bs, seq, d, code, _native.FSS_FWD, _native.make_config(config))
+        ws = _workspace(alpha.device, stream, need)
+        _native.check(
+            lib.fss_scan_fwd_state(
+                code, alpha.data_ptr(), beta.data_ptr(), out.data_ptr(),
+                h_before.data_ptr() if h_before is not None else None, h_last.data_ptr(),
+                bs, seq, d, ws.data_ptr(), ws.numel(), stream.cuda_stream, _native.make_config(config),
+            )
+        )
+    return out, h_last
+
+
+def scan_backward_state(
+    alpha_saved: torch.Tensor,
+    h_saved: torch.Tensor,
+    grad_out: torch.Tensor,
+    h_before: Optional[torch.Tensor] = None,
+    grad_h_last: Optional[torch.Tensor] = None,
+    config=None,
+) -> Tuple[torch.Tensor, torch.Tensor, Optional[torch.Tensor]]:
+    """(grad_alpha, grad_beta, grad_h_before); the last is None when ``h_before`` is None."""
+    dtype = alpha_saved.dtype
+    if dtype not in _DTYPE_CODE:
+        raise RuntimeError(f"expected scalar type torch.bfloat16 or torch.float32 for alpha but found {dtype}")
+    bs, seq, d = _validate(dtype, alpha_saved=alpha_saved, h_saved=h_saved, grad_out=grad_out)
+    h_before = _state("h_before", h_before, alpha_saved)
+    grad_h_last = _state("grad_h_last", grad_h_last, alpha_saved)
+    alpha_saved, h_saved, grad_out = alpha_saved.contiguous(), h_saved.contiguous(), grad_out.contiguous()
+    grad_alpha = torch.empty_like(alpha_saved, memory_format=torch.contiguous_format)
+    grad_beta = torch.empty_like(alpha_saved, memory_format=torch.contiguous_format)
+    grad_h_before = torch.zeros((bs, d), dtype=torch.float32, device=alpha_saved.device) if h_before is not None else None
+    if grad_alpha.numel() == 0:
+        if grad_h_before is not None and grad_h_last is not None and seq == 0:
+            grad_h_before.copy_(grad_h_last)
+        return grad_alpha, grad_beta, grad_h_before
+    lib = _native.lib()
+    code = _DTYPE_CODE[dtype]
+    with torch.cuda.device(alpha_saved.device):
+        stream = torch.cuda.current_stream()
+        need = lib.fss_workspace_bytes(bs, seq, d, code, _native.FSS_BWD, _native.make_config(config))
+        ws = _workspace(alpha_saved.device, stream, need)
+        _native.check(
+            lib.fss_scan_bwd_state(
+                code, alpha_saved.data_ptr(), h_saved.data_ptr(), grad_out.data_ptr(),
+                h_before.data_ptr() if h_before is not None else None,
+                grad_h_last.data_ptr() if grad_h_last is not None else None,
+                grad_alpha.data_ptr(), grad_beta.data_ptr(),
+                grad_h_before.data_ptr() if grad_h_before is not None else None,
+                bs, seq, d, ws.data_ptr(), ws.numel(), stream.cuda_stream, _native.make_config(config),
+            )
+        )
+    return grad_alpha, grad_beta, grad_h_before

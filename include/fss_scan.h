@@ -31,8 +31,8 @@
  *
  * Workspace
  *   When the sequence is split into more than one chunk the kernels chain the
- *   chunks through a small workspace (per-chunk carries with validity tags, a
- *   ticket counter).  Size it with fss_workspace_bytes, zero it ONCE with
+ *   chunks through a small workspace (per-chunk carries with validity tags,
+ *   completion counters).  Size it with fss_workspace_bytes, reset it ONCE with
  *   fss_workspace_init; after that every scan call leaves it ready for the
  *   next one, so steady-state calls launch exactly one kernel.  One workspace
  *   must not be used by two calls that may run concurrently (use one per
@@ -157,6 +157,31 @@ int fss_scan_bwd_ex(int dtype, const void *alpha, const void *h, const void *dou
                     void *grad_alpha, void *grad_beta, int64_t bs, int64_t seq,
                     int64_t d, void *workspace, size_t workspace_bytes,
                     void *stream, const fss_config *cfg);
+
+/*
+ * The same scans with a state entering and leaving the sequence, for streaming
+ * over segments of a longer sequence (and for sharding one over devices).  No
+ * counterpart in the reference, whose scan always starts from h[-1] = 0.
+ * States are fp32 (bs, d) row-major whatever the tensors' dtype; any may be NULL.
+ *
+ *   forward   h[-1] = h_before (then alpha[:,0,:] IS read: h[0] = alpha[0]*h[-1] + beta[0]);
+ *             h_last = the un-rounded state after the last step.
+ *   backward  g[seq-1] = dout[seq-1] + grad_h_last;
+ *             grad_alpha[0] = g[0]*h_before (0 without h_before);
+ *             grad_h_before = alpha[0]*g[0] (needs h_before).
+ * Scanning two adjacent segments with h_last of the first as h_before of the second,
+ * and grad_h_before of the second as grad_h_last of the first, equals scanning their
+ * concatenation.
+ */
+int fss_scan_fwd_state(int dtype, const void *alpha, const void *beta, void *h,
+                       const float *h_before, float *h_last, int64_t bs, int64_t seq,
+                       int64_t d, void *workspace, size_t workspace_bytes,
+                       void *stream, const fss_config *cfg);
+int fss_scan_bwd_state(int dtype, const void *alpha, const void *h, const void *dout,
+                       const float *h_before, const float *grad_h_last,
+                       void *grad_alpha, void *grad_beta, float *grad_h_before,
+                       int64_t bs, int64_t seq, int64_t d, void *workspace,
+                       size_t workspace_bytes, void *stream, const fss_config *cfg);
 
 /* Plain device-to-device copy kernel of `bytes` bytes (a multiple of 16; both
  * pointers 16-byte aligned).  Exists so that hardware counters read for the

@@ -66,6 +66,8 @@ def test_entry_points_reject_bad_arguments_without_a_gpu():
     assert lib.fss_scan_fwd_ex(7, p, p, p, 1, 4, 8, None, 0, None, None) == 5
     assert lib.fss_workspace_init(None, 1024, None) == 1
     assert lib.fss_copy_bytes(p, p + 1, 16, None) == 3
+    assert lib.fss_scan_bwd_state(0, p, p, p, None, None, p, p, p, 1, 4, 8, None, 0, None, None) == 1  # grad_h_before needs h_before
+    assert lib.fss_scan_fwd_state(0, p, p, p, p + 2, None, 1, 4, 8, None, 0, None, None) == 3
     two_chunks = _native.FssConfig(1, 8, 1, 0)
     assert lib.fss_scan_fwd_ex(0, p, p, p, 1, 9, 8, None, 0, None, ctypes.byref(two_chunks)) == 4
 

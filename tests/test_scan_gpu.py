@@ -399,3 +399,29 @@ def test_hip_graph_replays_match_eager(oracle):
             step()  # eager work between replays, same workspace
             side.synchronize()
         assert lib.fss_workspace_status(ws.data_ptr(), sp) == 0
+
+
+def test_tensors_larger_than_4_GiB():
+    """Byte offsets beyond 2^32 (the reference's index math is 32-bit:
+    csrc/include/sequential_scan_kernel_bf16.cuh:63-70).  Checked through closed forms, on the device."""
+    bs, seq, d = 3, 8192, 90000  # 2.2e9 elements, 4.4 GB per bf16 tensor
+    g = torch.Generator(device=DEV).manual_seed(3)
+    beta = torch.randn(bs, seq, d, generator=g, device=DEV, dtype=torch.bfloat16)
+    alpha = torch.zeros_like(beta)
+    h = ext.scan_forward_half(alpha, beta)
+    assert torch.equal(h, beta)
+    # alpha == 1 on one channel per batch row, beta == 1/128 there: h[t] = (t+1)/128
+    alpha[:, :, d - 2] = 1.0
+    beta[:, :, d - 2] = 1.0 / 128
+    h = ext.scan_forward_half(alpha, beta)
+    expect = ((torch.arange(seq, device=DEV, dtype=torch.float32) + 1) / 128).to(torch.bfloat16)
+    assert torch.equal(h[:, :, d - 2], expect[None, :].expand(bs, seq))
+    assert torch.equal(h[:, :, d - 1], beta[:, :, d - 1])
+    # backward: alpha == 0 elsewhere -> grad_beta == dout, grad_alpha[t] = dout[t]*h[t-1]
+    ga, gb = ext.scan_backward_half(alpha, h, beta)
+    assert torch.equal(gb[:, :, : d - 2], beta[:, :, : d - 2])
+    last = (slice(None), slice(1, None), d - 1)
+    assert torch.equal(ga[last].float(), (beta[last].float() * h[:, :-1, d - 1].float()).to(torch.bfloat16).float())
+    ext.workspace_status()
+    del alpha, beta, h, ga, gb
+    torch.cuda.empty_cache()
