@@ -4,13 +4,14 @@ Public names follow the reference package (sequential_scan/__init__.py:1-3):
 ``scan_cu`` (bf16) and ``scan_cu_single`` (fp32).  ``scan_tr`` - the
 reference's Triton backend - has no counterpart here and raises.
 """
-from .scan_cuda import SequentialScan, SequentialScanSingle, SequentialScanState, scan_with_state
+from .scan_cuda import (SequentialScan, SequentialScanGated, SequentialScanSingle, SequentialScanState,
+                        scan_gated, scan_with_state)
 from .scan_cuda import scan as scan_cu
 from .scan_cuda import scan_single as scan_cu_single
 
 __all__ = [
-    "scan_cu", "scan_cu_single", "scan_tr", "scan_with_state",
-    "SequentialScan", "SequentialScanSingle", "SequentialScanState",
+    "scan_cu", "scan_cu_single", "scan_tr", "scan_with_state", "scan_gated",
+    "SequentialScan", "SequentialScanSingle", "SequentialScanState", "SequentialScanGated",
 ]
 
 

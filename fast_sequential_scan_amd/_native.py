@@ -15,7 +15,7 @@ PKG_DIR = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.environ.get("FSS_SCAN_LIBRARY") or os.path.join(PKG_DIR, "_lib", "libfss_scan.so")
 
 FSS_BF16, FSS_F32 = 0, 1
-FSS_FWD, FSS_BWD = 0, 1
+FSS_FWD, FSS_BWD, FSS_GATED_FWD, FSS_GATED_BWD = 0, 1, 2, 3
 FSS_OK = 0
 FSS_ERR_CHAIN_TIMEOUT = 7
 
@@ -36,6 +36,8 @@ EXPORTED_SYMBOLS = (
     "fss_scan_bwd_ex",
     "fss_scan_fwd_state",
     "fss_scan_bwd_state",
+    "fss_gated_scan_fwd",
+    "fss_gated_scan_bwd",
     "fss_copy_bytes",
 )
 
@@ -100,6 +102,10 @@ def _declare(lib: ctypes.CDLL) -> None:
     lib.fss_scan_bwd_state.restype = _int
     lib.fss_scan_bwd_state.argtypes = [_int, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _vp, _sz, _vp, _cfgp]
     lib.fss_copy_bytes.restype = _int
+    lib.fss_gated_scan_fwd.restype = _int
+    lib.fss_gated_scan_fwd.argtypes = [_int, _vp, _vp, _vp, _i64, _i64, _i64, _vp, _sz, _vp, _cfgp]
+    lib.fss_gated_scan_bwd.restype = _int
+    lib.fss_gated_scan_bwd.argtypes = [_int, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _vp, _sz, _vp, _cfgp]
     lib.fss_copy_bytes.argtypes = [_vp, _vp, _sz, _vp]
 
 

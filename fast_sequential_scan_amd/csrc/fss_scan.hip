@@ -300,6 +300,7 @@ struct ScanArgs {
   int32_t look_waves;     // waves that look back in parallel (1..min(WAVES, kMaxLookWaves))
   uint32_t *hdr;          // workspace header
   uint64_t *words;        // tagged words
+  const char *in_x;       // gated backward only: the scan's input x (in_a is the gate there)
 #ifdef FSS_TRACE
   uint64_t *trace;        // debug build: 8 timestamps per tile, written by lane 0 of every wave 0
 #endif
@@ -737,9 +738,178 @@ __device__ __forceinline__ void scan_tile(const ScanArgs &p, const StateArgs<STA
   FSS_STAMP(c, p, 6);
 }
 
+// ---- the gated scan --------------------------------------------------------------
+//
+//   alpha[t] = sigmoid(gate[t]),  beta[t] = x[t] * sqrt(1 - alpha[t]^2),  h = scan(alpha, beta)
+//
+// computed from the pre-activations inside the scan's own tile, so alpha and beta
+// never exist in memory.  alpha and beta are rounded to the storage type where the
+// plain scan would have read them from memory (they stay packed in registers), so
+// the result is that of the plain scan on the rounded alpha and beta.
+
+// 1/(1 + 2^(-z log2 e)): one exp2 and one reciprocal instruction, about 1 ulp each.
+// +-inf and large |z| saturate to exactly 0 or 1.
+__device__ __forceinline__ float sigmoid_f32(float z) {
+  return __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(-1.4426950408889634f * z));
+}
+
+// One tile of the gated scan.  Forward: in_a = gate, in_b = x, out0 = h.
+// Backward: in_a = gate, in_b = dout, in_h = stored h, in_x = x, out0 = grad_x,
+// out1 = grad_gate, with g the reversed-time scan of dout under alpha:
+//   grad_x[t]    = g[t] * s[t]                                     s = sqrt(1 - alpha^2)
+//   grad_gate[t] = g[t] * (h[t-1] - x[t]*alpha[t]/s[t]) * alpha[t]*(1 - alpha[t])
+// (h[-1] = 0; the x term is dropped where alpha rounds to exactly 1, i.e. s = 0).
+// The backward needs alpha[t+1] as the coefficient of step t and alpha[t] for its
+// elementwise part: a slice of STEPS steps loads STEPS+1 rows of the gate.
+template <typename E, int VEC, int STEPS, bool BWD, bool FULL>
+__device__ __forceinline__ void gated_tile(const ScanArgs &p, const TileCtx &c) {
+  using RowT = Row<E, VEC>;
+  const int64_t seq = c.seq, row_bytes = c.row_bytes, r0 = c.r0;
+  const uint32_t lane_off = c.lane_off;
+  constexpr int kARows = BWD ? STEPS + 1 : STEPS;
+
+  RowT a[kARows], b[STEPS];
+  RowT hp[BWD ? STEPS : 1], xs[BWD ? STEPS : 1];
+
+  // forward: a[s] = gate row t = r0+s.  backward: a[s] = gate row t+1 = seq-(r0+s), s = 0..STEPS
+  const int64_t t_first = BWD ? seq - 1 - r0 : r0;
+  gcptr_t pa = (gcptr_t)p.in_a + c.tile_base + (BWD ? t_first + 1 : t_first) * row_bytes;
+  gcptr_t pb = (gcptr_t)p.in_b + c.tile_base + t_first * row_bytes;
+  const int64_t step_bytes = BWD ? -row_bytes : row_bytes;
+
+  // ---- phase 1a: loads ---------------------------------------------------------------
+#pragma unroll
+  for (int s = 0; s < kARows; ++s) {
+    const int64_t r = r0 + s;
+    // the gate row of a[s] exists: forward r < seq; backward 1 <= r <= seq
+    const bool a_ok = FULL || (c.col_ok && (BWD ? (r >= 1 && r <= seq) : (r < seq)));
+    if (!FULL) a[s].fill(0.0f);
+    if (a_ok) a[s].template load<kNtA>(uniform_ptr(pa + s * step_bytes) + lane_off);
+    if (s < STEPS) {
+      if (!FULL) b[s].fill(0.0f);
+      if (FULL || (c.col_ok && r < seq)) b[s].template load<kNtB>(uniform_ptr(pb + s * step_bytes) + lane_off);
+    }
+  }
+  // x and the saved h only feed phase 3 of the backward: half of their rows now, the
+  // rest during phase 3 into registers that finished steps have released
+  constexpr int kEarly = BWD ? (STEPS >= 16 ? STEPS / 2 : STEPS) : 0;
+  gcptr_t ph = BWD ? (gcptr_t)p.in_h + c.tile_base + (t_first - 1) * row_bytes : (gcptr_t) nullptr;
+  gcptr_t px = BWD ? (gcptr_t)p.in_x + c.tile_base + t_first * row_bytes : (gcptr_t) nullptr;
+  auto load_hx = [&](int s) {
+    if (FULL) {
+      hp[s].template load<kNtH>(uniform_ptr(ph + s * step_bytes) + lane_off);
+      xs[s].template load<kNtH>(uniform_ptr(px + s * step_bytes) + lane_off);
+    } else {
+      hp[s].fill(0.0f);
+      xs[s].fill(0.0f);
+      if (c.col_ok && r0 + s < seq - 1)  // t - 1 >= 0
+        hp[s].template load<kNtH>(uniform_ptr(ph + s * step_bytes) + lane_off);
+      if (c.col_ok && r0 + s < seq) xs[s].template load<kNtH>(uniform_ptr(px + s * step_bytes) + lane_off);
+    }
+  };
+  if (BWD) {
+#pragma unroll
+    for (int s = 0; s < kEarly; ++s) load_hx(s);
+  }
+
+  // ---- phase 1b: gate -> alpha (and x -> beta), in place; the slice as an affine map ----
+  // The coefficient of a step outside the sequence is 1 (identity).  The first step of
+  // the scan starts from a zero state, so its coefficient is immaterial as long as it
+  // is finite: it is sigmoid(gate[0]) in the forward and sigmoid(0) in the backward.
+  float mA[VEC], mB[VEC];
+#pragma unroll
+  for (int v = 0; v < VEC; ++v) {
+    mA[v] = 1.0f;
+    mB[v] = 0.0f;
+  }
+#pragma unroll
+  for (int s = 0; s < kARows; ++s) {
+    const int64_t r = r0 + s;
+    float al[VEC];
+#pragma unroll
+    for (int v = 0; v < VEC; ++v) al[v] = sigmoid_f32(a[s].get(v));
+    if (!FULL && (r >= seq + (BWD ? 1 : 0) || !c.col_ok)) {
+#pragma unroll
+      for (int v = 0; v < VEC; ++v) al[v] = 1.0f;
+    }
+    a[s].pack(al);
+    if (s < STEPS) {
+      if (!BWD) {
+        float be[VEC];
+#pragma unroll
+        for (int v = 0; v < VEC; ++v) {
+          const float ar = a[s].get(v);  // as rounded
+          be[v] = b[s].get(v) * __builtin_amdgcn_sqrtf(__builtin_fmaf(-ar, ar, 1.0f));
+        }
+        b[s].pack(be);  // rows outside the sequence hold x = 0, so beta = 0 there
+      }
+      const bool ident = !FULL && BWD && r >= seq;  // backward: a[s] with r == seq is alpha[0], not a coefficient
+#pragma unroll
+      for (int v = 0; v < VEC; ++v) {
+        const float av = ident ? 1.0f : a[s].get(v);
+        mB[v] = __builtin_fmaf(av, mB[v], b[s].get(v));
+        mA[v] *= av;
+      }
+    }
+  }
+
+  float state[VEC];
+  if (!c.chained && c.n_waves == 1) {
+#pragma unroll
+    for (int v = 0; v < VEC; ++v) state[v] = 0.0f;
+  } else {
+    chain_chunks<VEC>(p, c, mA, mB, nullptr, state);
+  }
+
+  // ---- phase 3 -------------------------------------------------------------------------
+#pragma unroll
+  for (int s = 0; s < kARows; ++s) keep_packed(a[s]);
+#pragma unroll
+  for (int s = 0; s < STEPS; ++s) {
+    keep_packed(b[s]);
+    if (BWD && s < kEarly) {
+      keep_packed(hp[s]);
+      keep_packed(xs[s]);
+    }
+  }
+  gptr_t po0 = (gptr_t)p.out0 + c.tile_base + t_first * row_bytes;
+  gptr_t po1 = BWD ? (gptr_t)p.out1 + c.tile_base + t_first * row_bytes : (gptr_t) nullptr;
+#pragma unroll
+  for (int s = 0; s < STEPS; ++s) {
+    const int64_t r = r0 + s;
+    const bool ident = !FULL && BWD && r >= seq;
+    float o0[VEC], o1[VEC];
+#pragma unroll
+    for (int v = 0; v < VEC; ++v) {
+      state[v] = __builtin_fmaf(ident ? 1.0f : a[s].get(v), state[v], b[s].get(v));
+      if (BWD) {
+        const float at = a[s + 1].get(v);  // alpha[t]
+        const float om = __builtin_fmaf(-at, at, 1.0f);
+        const float rs = om > 0.0f ? __builtin_amdgcn_rsqf(om) : 0.0f;
+        o0[v] = state[v] * (om * rs);
+        const float inner = __builtin_fmaf(-xs[s].get(v) * at, rs, hp[s].get(v));
+        o1[v] = state[v] * inner * (at - at * at);
+      } else {
+        o0[v] = state[v];
+      }
+    }
+    if (FULL || (c.col_ok && r < seq)) {
+      RowT o;
+      o.pack(o0);
+      o.template store<(BWD ? kNtOutBwd : kNtOutFwd)>(uniform_ptr(po0 + s * step_bytes) + lane_off);
+      if (BWD) {
+        RowT oz;
+        oz.pack(o1);
+        oz.template store<kNtOutBwd>(uniform_ptr(po1 + s * step_bytes) + lane_off);
+      }
+    }
+    if (BWD && s + kEarly < STEPS) load_hx(s + kEarly);
+  }
+}
+
 // STATE: the variant that honours the optional incoming/outgoing state rows of ScanArgs;
-// the plain scan is compiled without them.
-template <typename E, int VEC, int STEPS, bool BWD, bool STATE>
+// the plain scan is compiled without them.  GATED: the gated scan (never with STATE).
+template <typename E, int VEC, int STEPS, bool BWD, bool STATE, bool GATED = false>
 __global__ __launch_bounds__(1024) void scan_kernel(const ScanArgs p, const StateArgs<STATE> st) {
   constexpr int kLaneSlots = 64 * VEC;  // channels per tile
 
@@ -804,14 +974,22 @@ __global__ __launch_bounds__(1024) void scan_kernel(const ScanArgs p, const Stat
 
     // Forward touches rows r0..r0+STEPS-1 and must not be at r = 0 (alpha[0] is never
     // read); the backward additionally reads row t+1 and row t-1.
-    const bool full = (col0 + kLaneSlots <= p.d) && (c.r0 >= 1) &&
+    // (the gated forward does read row 0 of its first input)
+    const bool full = (col0 + kLaneSlots <= p.d) && (c.r0 >= ((GATED && !BWD) ? 0 : 1)) &&
                       (BWD ? (c.r0 + STEPS <= c.seq - 1) : (c.r0 + STEPS <= c.seq));
     // wave-uniform, but waves of one workgroup may differ: both variants execute the
     // same barriers, so they meet
-    if (full)
-      scan_tile<E, VEC, STEPS, BWD, STATE, true>(p, st, c);
-    else
-      scan_tile<E, VEC, STEPS, BWD, STATE, false>(p, st, c);
+    if constexpr (GATED) {
+      if (full)
+        gated_tile<E, VEC, STEPS, BWD, true>(p, c);
+      else
+        gated_tile<E, VEC, STEPS, BWD, false>(p, c);
+    } else {
+      if (full)
+        scan_tile<E, VEC, STEPS, BWD, STATE, true>(p, st, c);
+      else
+        scan_tile<E, VEC, STEPS, BWD, STATE, false>(p, st, c);
+    }
   }
 
 #ifdef FSS_RESIDENCY_PROBE
@@ -877,7 +1055,10 @@ inline size_t lds_bytes(int waves, int vec) {
   return static_cast<size_t>(2 * waves + look_waves(waves, vec) + 1) * vec * 512;
 }
 
-inline bool config_valid(const fss_config &c, int dtype) {
+inline bool config_valid(const fss_config &c, int dtype, bool gated = false, int dir = FSS_FWD) {
+  // the gated kernels exist for 4 bytes (or one element) per lane; their backward holds
+  // four tensors, so at most 16 timesteps per lane
+  if (gated && (c.vec > (dtype == FSS_BF16 ? 2 : 1) || (dir == FSS_BWD && c.steps > 16))) return false;
   const bool vec_ok = dtype == FSS_BF16 ? (c.vec == 1 || c.vec == 2 || c.vec == 4 || c.vec == 8)
                                         : (c.vec == 1 || c.vec == 2 || c.vec == 4);
   const bool steps_ok = c.steps == 8 || c.steps == 16 || c.steps == 32;
@@ -892,7 +1073,7 @@ inline bool config_valid(const fss_config &c, int dtype) {
 // Fills the zero fields of `c`.  `align` is the common alignment in bytes of all
 // tensors of the call.
 void complete_config(fss_config &c, int64_t bs, int64_t seq, int64_t d, int dtype, int dir,
-                     size_t align) {
+                     size_t align, bool gated = false) {
   // Choices below come from sweeps on MI355X over the five measured workloads
   // (bs8 d1024 seq512..8192, bs16 d512 seq2048, bs4 d2048 seq8192, bs2 d768
   // seq1024, bs1 d256 seq65521).  What they showed: 4 bytes per lane per load
@@ -920,7 +1101,9 @@ void complete_config(fss_config &c, int64_t bs, int64_t seq, int64_t d, int dtyp
     // backward: 32-step slices cost it a dozen spilled registers per lane (5 % more HBM
     // traffic); that only pays where the chain of chunks is long.  Elsewhere 16 steps are
     // as fast in bf16 and 6 % faster in fp32 (forward and backward alternating).
-    if (dir == FSS_BWD && s == 32 && ceil_div(seq, static_cast<int64_t>(8) * 32) <= 16) s = 16;
+    if (dir == FSS_BWD && s == 32 && (gated || ceil_div(seq, static_cast<int64_t>(8) * 32) <= 16)) s = 16;
+    // gated forward in bf16: 32 steps spill (the gating needs temporaries), 16 measured faster
+    if (gated && dir == FSS_FWD && dtype == FSS_BF16 && s == 32) s = 16;
     // small problems: shorter slices until there are two 8-wave tiles per CU (512), as
     // long as the machine still gets a few waves per SIMD out of it
     const int64_t ctiles = bs * ceil_div(d, 64 * c.vec);
@@ -954,7 +1137,9 @@ int make_plan(Plan &pl, int64_t bs, int64_t seq, int64_t d, int dtype, int dir, 
               const fss_config *user) {
   if (bs < 0 || seq < 0 || d < 0) return FSS_ERR_BAD_SHAPE;
   if (dtype != FSS_BF16 && dtype != FSS_F32) return FSS_ERR_BAD_CONFIG;
-  if (dir != FSS_FWD && dir != FSS_BWD) return FSS_ERR_BAD_CONFIG;
+  if (dir < FSS_FWD || dir > FSS_GATED_BWD) return FSS_ERR_BAD_CONFIG;
+  const bool gated = dir >= FSS_GATED_FWD;
+  dir &= 1;
   const int esize = dtype == FSS_BF16 ? 2 : 4;
   // bs*seq*d*esize must fit int64
   if (bs > 0 && seq > 0 && d > 0) {
@@ -965,8 +1150,8 @@ int make_plan(Plan &pl, int64_t bs, int64_t seq, int64_t d, int dtype, int dir, 
   if (user) c = *user;
   if (c.max_groups < 0) return FSS_ERR_BAD_CONFIG;
   const int64_t dd = d > 0 ? d : 1, ss = seq > 0 ? seq : 1, bb = bs > 0 ? bs : 1;
-  complete_config(c, bb, ss, dd, dtype, dir, align);
-  if (!config_valid(c, dtype)) return FSS_ERR_BAD_CONFIG;
+  complete_config(c, bb, ss, dd, dtype, dir, align, gated);
+  if (!config_valid(c, dtype, gated, dir)) return FSS_ERR_BAD_CONFIG;
   if (dd % c.vec != 0) return FSS_ERR_BAD_CONFIG;
   if (align % (static_cast<size_t>(c.vec) * esize) != 0) return FSS_ERR_MISALIGNED;
   pl.cfg = c;
@@ -1045,7 +1230,7 @@ int resident_workgroups(Kernel kernel, int waves, size_t lds) {
   return per_cu * cu_count;
 }
 
-template <typename E, int VEC, int STEPS, bool BWD, bool STATE>
+template <typename E, int VEC, int STEPS, bool BWD, bool STATE, bool GATED = false>
 int launch_one(const ScanArgs &args, const StateArgs<true> &state, const Plan &pl, hipStream_t stream) {
   // The kernel's waits are only safe if every workgroup of the grid is resident,
   // so the grid never exceeds what the device holds at once; workgroups loop.
@@ -1054,7 +1239,7 @@ int launch_one(const ScanArgs &args, const StateArgs<true> &state, const Plan &p
   const size_t lds = lds_bytes(waves, VEC);
   int fit = __atomic_load_n(&resident[waves], __ATOMIC_RELAXED);
   if (fit == 0) {
-    fit = resident_workgroups(scan_kernel<E, VEC, STEPS, BWD, STATE>, waves, lds);
+    fit = resident_workgroups(scan_kernel<E, VEC, STEPS, BWD, STATE, GATED>, waves, lds);
     if (fit <= 0) return FSS_ERR_LAUNCH;
     __atomic_store_n(&resident[waves], fit, __ATOMIC_RELAXED);
   }
@@ -1064,7 +1249,7 @@ int launch_one(const ScanArgs &args, const StateArgs<true> &state, const Plan &p
   const dim3 block(static_cast<uint32_t>(waves) * 64);
   StateArgs<STATE> st;
   if constexpr (STATE) st = state;
-  hipLaunchKernelGGL((scan_kernel<E, VEC, STEPS, BWD, STATE>), grid, block, lds, stream, args, st);
+  hipLaunchKernelGGL((scan_kernel<E, VEC, STEPS, BWD, STATE, GATED>), grid, block, lds, stream, args, st);
   const hipError_t e = hipGetLastError();
   if (e != hipSuccess) {
     tls_hip_error = static_cast<int>(e);
@@ -1103,24 +1288,61 @@ int launch_typed(const ScanArgs &args, const StateArgs<true> &state, const Plan 
   return FSS_ERR_BAD_CONFIG;
 }
 
+// The gated kernels: 4 bytes (bf16 x2, fp32 x1) or one bf16 element per lane.
+template <typename E, bool BWD>
+int launch_gated(const ScanArgs &args, const Plan &pl, hipStream_t stream) {
+  constexpr bool is_bf16 = E::kBytes == 2;
+  const StateArgs<true> none = {nullptr, nullptr, nullptr};
+  const int key = pl.cfg.vec * 100 + pl.cfg.steps;
+  switch (key) {
+#define FSS_CASE(V, S) \
+  case V * 100 + S:    \
+    return launch_one<E, V, S, BWD, false, true>(args, none, pl, stream);
+    FSS_CASE(1, 8)
+    FSS_CASE(1, 16)
+    default:
+      break;
+  }
+  if constexpr (!BWD) {
+    if (key == 132) return launch_one<E, 1, 32, BWD, false, true>(args, none, pl, stream);
+  }
+  if constexpr (is_bf16) {
+    switch (key) {
+      FSS_CASE(2, 8)
+      FSS_CASE(2, 16)
+      default:
+        break;
+    }
+    if constexpr (!BWD) {
+      if (key == 232) return launch_one<E, 2, 32, BWD, false, true>(args, none, pl, stream);
+    }
+  }
+#undef FSS_CASE
+  return FSS_ERR_BAD_CONFIG;
+}
+
 int run_scan(int dtype, int dir, const void *alpha, const void *in_b, const void *in_h, void *out0,
              void *out1, int64_t bs, int64_t seq, int64_t d, void *workspace, size_t workspace_bytes,
              void *stream, const fss_config *cfg, const float *state_in = nullptr,
-             float *state_out = nullptr, const float *h_before = nullptr) {
+             float *state_out = nullptr, const float *h_before = nullptr, const void *in_x = nullptr) {
+  const bool gated = dir >= FSS_GATED_FWD;
+  const int plan_dir = dir;
+  dir &= 1;
   if (bs < 0 || seq < 0 || d < 0) return FSS_ERR_BAD_SHAPE;
   if (dtype != FSS_BF16 && dtype != FSS_F32) return FSS_ERR_BAD_CONFIG;
   if (bs == 0 || seq == 0 || d == 0) return FSS_OK;
   if (!alpha || !in_b || !out0) return FSS_ERR_NULL_POINTER;
   if (dir == FSS_BWD && (!in_h || !out1)) return FSS_ERR_NULL_POINTER;
+  if (gated && dir == FSS_BWD && !in_x) return FSS_ERR_NULL_POINTER;
   const size_t esize = dtype == FSS_BF16 ? 2 : 4;
-  const size_t align = dir == FSS_BWD ? common_alignment({alpha, in_b, in_h, out0, out1})
+  const size_t align = dir == FSS_BWD ? common_alignment({alpha, in_b, in_h, out0, out1, in_x})
                                       : common_alignment({alpha, in_b, out0});
   if (align < esize) return FSS_ERR_MISALIGNED;
   if ((reinterpret_cast<uintptr_t>(state_in) | reinterpret_cast<uintptr_t>(state_out) |
        reinterpret_cast<uintptr_t>(h_before)) % 4 != 0)
     return FSS_ERR_MISALIGNED;
   Plan pl;
-  int rc = make_plan(pl, bs, seq, d, dtype, dir, align, cfg);
+  int rc = make_plan(pl, bs, seq, d, dtype, plan_dir, align, cfg);
   if (rc != FSS_OK) return rc;
   if (pl.n_chunks > 1) {
     if (!workspace || workspace_bytes < pl.ws_bytes) return FSS_ERR_WORKSPACE_SMALL;
@@ -1135,6 +1357,7 @@ int run_scan(int dtype, int dir, const void *alpha, const void *in_b, const void
   args.in_h = static_cast<const char *>(in_h);
   args.out0 = static_cast<char *>(out0);
   args.out1 = static_cast<char *>(out1);
+  args.in_x = static_cast<const char *>(in_x);
   args.seq = seq;
   args.d = d;
   args.tiles_per_row = static_cast<int32_t>(pl.tiles_per_row);
@@ -1149,6 +1372,10 @@ int run_scan(int dtype, int dir, const void *alpha, const void *in_b, const void
   args.trace = g_trace;
 #endif
   hipStream_t s = static_cast<hipStream_t>(stream);
+  if (gated) {
+    if (dtype == FSS_BF16) return dir == FSS_BWD ? launch_gated<BF16, true>(args, pl, s) : launch_gated<BF16, false>(args, pl, s);
+    return dir == FSS_BWD ? launch_gated<F32, true>(args, pl, s) : launch_gated<F32, false>(args, pl, s);
+  }
   const bool st = state_in || state_out || h_before;
   if (dtype == FSS_BF16) {
     if (dir == FSS_BWD) return st ? launch_typed<BF16, true, true>(args, state, pl, s) : launch_typed<BF16, true, false>(args, state, pl, s);
@@ -1198,7 +1425,7 @@ size_t fss_workspace_bytes(int64_t bs, int64_t seq, int64_t d, int dtype, int di
 size_t fss_workspace_bytes_max(int64_t bs, int64_t seq, int64_t d) {
   size_t best = fss::kHeaderBytes;
   for (int dtype = 0; dtype < 2; ++dtype)
-    for (int dir = 0; dir < 2; ++dir)
+    for (int dir = FSS_FWD; dir <= FSS_GATED_BWD; ++dir)
       for (size_t align = 2; align <= 16; align <<= 1) {
         fss::Plan pl;
         if (fss::make_plan(pl, bs, seq, d, dtype, dir, align, nullptr) == FSS_OK && pl.ws_bytes > best)
@@ -1280,6 +1507,20 @@ int fss_scan_bwd_state(int dtype, const void *alpha, const void *h, const void *
   if (grad_h_before && !h_before) return FSS_ERR_NULL_POINTER;
   return fss::run_scan(dtype, FSS_BWD, alpha, dout, h, grad_beta, grad_alpha, bs, seq, d, workspace,
                        workspace_bytes, stream, cfg, grad_h_last, grad_h_before, h_before);
+}
+
+int fss_gated_scan_fwd(int dtype, const void *gate, const void *x, void *h, int64_t bs, int64_t seq,
+                       int64_t d, void *workspace, size_t workspace_bytes, void *stream,
+                       const fss_config *cfg) {
+  return fss::run_scan(dtype, FSS_GATED_FWD, gate, x, nullptr, h, nullptr, bs, seq, d, workspace,
+                       workspace_bytes, stream, cfg);
+}
+
+int fss_gated_scan_bwd(int dtype, const void *gate, const void *x, const void *h, const void *dout,
+                       void *grad_gate, void *grad_x, int64_t bs, int64_t seq, int64_t d,
+                       void *workspace, size_t workspace_bytes, void *stream, const fss_config *cfg) {
+  return fss::run_scan(dtype, FSS_GATED_BWD, gate, dout, h, grad_x, grad_gate, bs, seq, d, workspace,
+                       workspace_bytes, stream, cfg, nullptr, nullptr, nullptr, x);
 }
 
 int fss_scan_fwd_bf16(const void *alpha, const void *beta, void *h, int64_t bs, int64_t seq, int64_t d,

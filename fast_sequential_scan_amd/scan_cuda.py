@@ -101,3 +101,27 @@ def scan_with_state(
     ``alpha[:, 0]`` multiplies it).  Returns ``(h, h_last)`` with ``h_last`` the fp32 state after the
     last step, to be passed as ``h_before`` of the next segment."""
     return SequentialScanState.apply(alpha, beta, h_before)
+
+
+class SequentialScanGated(Function):
+    """``h = scan(sigmoid(gate), x * sqrt(1 - sigmoid(gate)**2))`` with the gating computed inside the
+    scan kernels, forward and backward.  Not in the reference.  bf16 or fp32 tensors."""
+
+    @staticmethod
+    def forward(ctx: Any, gate: torch.Tensor, x: torch.Tensor) -> torch.Tensor:
+        h = _ext.gated_scan_forward(gate, x)
+        ctx.save_for_backward(gate, x, h)
+        return h
+
+    @staticmethod
+    @once_differentiable
+    def backward(ctx: Any, grad_output: torch.Tensor) -> Tuple[torch.Tensor, torch.Tensor]:
+        gate, x, h = ctx.saved_tensors
+        grad_gate, grad_x = _ext.gated_scan_backward(gate, x, h, grad_output)
+        return grad_gate, grad_x
+
+
+def scan_gated(gate: torch.Tensor, x: torch.Tensor) -> torch.Tensor:
+    """The Hawk / RG-LRU style gated recurrence from its pre-activations:
+    ``a = sigmoid(gate)``, ``h[t] = a[t]*h[t-1] + sqrt(1 - a[t]**2) * x[t]``."""
+    return SequentialScanGated.apply(gate, x)

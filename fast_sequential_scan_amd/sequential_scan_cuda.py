@@ -24,6 +24,7 @@ from . import _native
 __all__ = [
     "scan_forward", "scan_backward", "scan_forward_half", "scan_backward_half",
     "scan_forward_state", "scan_backward_state",
+    "gated_scan_forward", "gated_scan_backward",
 ]
 
 _DTYPE_CODE = {torch.bfloat16: _native.FSS_BF16, torch.float32: _native.FSS_F32}
@@ -244,3 +245,63 @@ def scan_backward_state(
             )
         )
     return grad_alpha, grad_beta, grad_h_before
+
+
+# ---- gated scan: alpha = sigmoid(gate), beta = x*sqrt(1-alpha^2) inside the kernel (no counterpart
+# in the reference, which is handed alpha and beta) ----
+
+
+def _either_dtype(t: torch.Tensor, name: str) -> torch.dtype:
+    if t.dtype not in _DTYPE_CODE:
+        raise RuntimeError(f"expected scalar type torch.bfloat16 or torch.float32 for {name} but found {t.dtype}")
+    return t.dtype
+
+
+def gated_scan_forward(gate: torch.Tensor, x: torch.Tensor, config=None) -> torch.Tensor:
+    """h of the scan with ``alpha = sigmoid(gate)`` and ``beta = x * sqrt(1 - alpha**2)``."""
+    dtype = _either_dtype(gate, "gate")
+    bs, seq, d = _validate(dtype, gate=gate, x=x)
+    gate, x = gate.contiguous(), x.contiguous()
+    out = torch.empty_like(gate, memory_format=torch.contiguous_format)
+    if out.numel() == 0:
+        return out
+    lib = _native.lib()
+    code = _DTYPE_CODE[dtype]
+    cfg = _native.make_config(config)
+    with torch.cuda.device(gate.device):
+        stream = torch.cuda.current_stream()
+        ws = _workspace(gate.device, stream, lib.fss_workspace_bytes(bs, seq, d, code, _native.FSS_GATED_FWD, cfg))
+        _native.check(
+            lib.fss_gated_scan_fwd(
+                code, gate.data_ptr(), x.data_ptr(), out.data_ptr(), bs, seq, d,
+                ws.data_ptr(), ws.numel(), stream.cuda_stream, cfg,
+            )
+        )
+    return out
+
+
+def gated_scan_backward(
+    gate: torch.Tensor, x: torch.Tensor, h_saved: torch.Tensor, grad_out: torch.Tensor, config=None
+) -> List[torch.Tensor]:
+    """[grad_gate, grad_x] of :func:`gated_scan_forward`, given its inputs and stored output."""
+    dtype = _either_dtype(gate, "gate")
+    bs, seq, d = _validate(dtype, gate=gate, x=x, h_saved=h_saved, grad_out=grad_out)
+    gate, x, h_saved, grad_out = gate.contiguous(), x.contiguous(), h_saved.contiguous(), grad_out.contiguous()
+    grad_gate = torch.empty_like(gate, memory_format=torch.contiguous_format)
+    grad_x = torch.empty_like(gate, memory_format=torch.contiguous_format)
+    if grad_gate.numel() == 0:
+        return [grad_gate, grad_x]
+    lib = _native.lib()
+    code = _DTYPE_CODE[dtype]
+    cfg = _native.make_config(config)
+    with torch.cuda.device(gate.device):
+        stream = torch.cuda.current_stream()
+        ws = _workspace(gate.device, stream, lib.fss_workspace_bytes(bs, seq, d, code, _native.FSS_GATED_BWD, cfg))
+        _native.check(
+            lib.fss_gated_scan_bwd(
+                code, gate.data_ptr(), x.data_ptr(), h_saved.data_ptr(), grad_out.data_ptr(),
+                grad_gate.data_ptr(), grad_x.data_ptr(), bs, seq, d,
+                ws.data_ptr(), ws.numel(), stream.cuda_stream, cfg,
+            )
+        )
+    return [grad_gate, grad_x]

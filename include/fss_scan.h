@@ -66,7 +66,8 @@ typedef enum fss_status {
 } fss_status;
 
 typedef enum fss_dtype { FSS_BF16 = 0, FSS_F32 = 1 } fss_dtype;
-typedef enum fss_dir { FSS_FWD = 0, FSS_BWD = 1 } fss_dir;
+/* FSS_GATED_*: the gated scans below (they chunk the sequence differently) */
+typedef enum fss_dir { FSS_FWD = 0, FSS_BWD = 1, FSS_GATED_FWD = 2, FSS_GATED_BWD = 3 } fss_dir;
 
 /*
  * Launch configuration.  Zero in a field means "choose for me".
@@ -98,8 +99,8 @@ int fss_last_hip_error(void);
  * cfg may be NULL. */
 size_t fss_workspace_bytes(int64_t bs, int64_t seq, int64_t d, int dtype, int dir,
                            const fss_config *cfg);
-/* Upper bound over both directions, both dtypes and every configuration the
- * library may choose by itself. */
+/* Upper bound over all directions (gated included), both dtypes and every
+ * configuration the library may choose by itself. */
 size_t fss_workspace_bytes_max(int64_t bs, int64_t seq, int64_t d);
 /* Resets the workspace with a fill kernel on `stream` (graph-capturable). */
 int fss_workspace_init(void *workspace, size_t bytes, void *stream);
@@ -182,6 +183,36 @@ int fss_scan_bwd_state(int dtype, const void *alpha, const void *h, const void *
                        void *grad_alpha, void *grad_beta, float *grad_h_before,
                        int64_t bs, int64_t seq, int64_t d, void *workspace,
                        size_t workspace_bytes, void *stream, const fss_config *cfg);
+
+/*
+ * Gated scan: the gating of a Hawk / RG-LRU style block fused in front of the scan,
+ *
+ *   alpha = sigmoid(gate),  beta = x * sqrt(1 - alpha^2),  h = scan(alpha, beta)
+ *
+ * from the pre-activations `gate` and `x`, both (bs, seq, d) of `dtype`; alpha and beta
+ * never exist in memory (forward 3 tensors of traffic instead of 7, forward+backward 9
+ * instead of 18).  No counterpart in the reference, which is handed alpha and beta
+ * (sequential_scan/scan_cuda.py:16-27); a model computes them with elementwise kernels first.
+ * alpha and beta are rounded to `dtype` exactly where the plain scan would have read
+ * them from memory, so h equals fss_scan_fwd on those rounded tensors.
+ *
+ * Backward, with g the reversed-time scan of dout under alpha (as in fss_scan_bwd) and
+ * s = sqrt(1 - alpha^2):
+ *   grad_x[t]    = g[t] * s[t]
+ *   grad_gate[t] = g[t] * (h[t-1] - x[t]*alpha[t]/s[t]) * alpha[t]*(1 - alpha[t])   (h[-1] = 0)
+ * Where alpha rounds to exactly 1 (s = 0) the x term is dropped (torch's autograd gives
+ * inf/nan there).  gate[:,0,:] is read (beta[0] depends on it).  The six tensors of a
+ * backward must not overlap.  vec is 1 or 2 (bf16) / 1 (fp32); steps at most 16 in the
+ * backward.  Use FSS_GATED_FWD / FSS_GATED_BWD as `dir` of fss_workspace_bytes and
+ * fss_choose_config.
+ */
+int fss_gated_scan_fwd(int dtype, const void *gate, const void *x, void *h, int64_t bs,
+                       int64_t seq, int64_t d, void *workspace, size_t workspace_bytes,
+                       void *stream, const fss_config *cfg);
+int fss_gated_scan_bwd(int dtype, const void *gate, const void *x, const void *h,
+                       const void *dout, void *grad_gate, void *grad_x, int64_t bs,
+                       int64_t seq, int64_t d, void *workspace, size_t workspace_bytes,
+                       void *stream, const fss_config *cfg);
 
 /* Plain device-to-device copy kernel of `bytes` bytes (a multiple of 16; both
  * pointers 16-byte aligned).  Exists so that hardware counters read for the

@@ -234,3 +234,51 @@ def ref_scan_bwd(alpha, h, dout):
     if rc != 0:
         raise ValueError(f"shape {a.shape} is not instantiated in oracle/ref_driver.cpp")
     return ga, gb
+
+
+# ---- gated scan (not in the reference: alpha = sigmoid(gate), beta = x*sqrt(1-alpha^2)) ----
+#
+# Elementwise arithmetic in float64 NumPy around the scans above.  `rounding` is where the
+# storage type takes effect: "bf16" rounds alpha, beta and the outputs to bf16 (to nearest
+# even), "f32" to float32.  Inputs are float32 arrays already holding storage-type values.
+
+
+def _round_to(a: np.ndarray, rounding: str) -> np.ndarray:
+    a32 = np.asarray(a, dtype=np.float64).astype(np.float32)
+    if rounding == "f32":
+        return a32
+    if rounding == "bf16":
+        return bf16_bits_to_f32(f32_to_bf16_bits(a32))
+    raise ValueError(rounding)
+
+
+def gate_transform(gate, x, rounding: str) -> Tuple[np.ndarray, np.ndarray]:
+    """(alpha, beta) as float32 arrays of storage-type values."""
+    g64 = np.asarray(gate, dtype=np.float64)
+    alpha = _round_to(1.0 / (1.0 + np.exp(-g64)), rounding)
+    a64 = alpha.astype(np.float64)
+    beta = _round_to(np.asarray(x, dtype=np.float64) * np.sqrt(1.0 - a64 * a64), rounding)
+    return alpha, beta
+
+
+def gated_scan_fwd(gate, x, rounding: str) -> np.ndarray:
+    """Un-rounded fp32 h of the scan over the rounded alpha and beta."""
+    alpha, beta = gate_transform(gate, x, rounding)
+    return scan_fwd_f32(alpha, beta)
+
+
+def gated_scan_bwd(gate, x, h, dout, rounding: str) -> Tuple[np.ndarray, np.ndarray]:
+    """(grad_gate, grad_x) in float32, un-rounded: the plain backward, then the chain rule
+    through beta = x*s, s = sqrt(1-alpha^2), alpha = sigmoid(gate).  Where alpha is exactly 1
+    the x term of grad_gate is dropped."""
+    alpha, _ = gate_transform(gate, x, rounding)
+    grad_alpha, grad_beta = scan_bwd_f32(alpha, np.asarray(h, dtype=np.float32), np.asarray(dout, dtype=np.float32))
+    a = alpha.astype(np.float64)
+    om = 1.0 - a * a
+    s = np.sqrt(om)
+    with np.errstate(divide="ignore", invalid="ignore"):
+        a_over_s = np.where(om > 0.0, a / s, 0.0)
+    gb = grad_beta.astype(np.float64)
+    grad_x = gb * s
+    grad_gate = (grad_alpha.astype(np.float64) - gb * np.asarray(x, dtype=np.float64) * a_over_s) * a * (1.0 - a)
+    return grad_gate.astype(np.float32), grad_x.astype(np.float32)

@@ -47,3 +47,29 @@ def torch_loop_bwd(alpha: torch.Tensor, h: torch.Tensor, dout: torch.Tensor) -> 
         else:
             galpha[:, t, :] = 0.0
     return galpha, gbeta
+
+
+# ---- gated scan (not in the reference): the gating as torch elementwise ops, then the loops above ----
+
+
+def torch_gated_fwd(gate: torch.Tensor, x: torch.Tensor) -> Tuple[torch.Tensor, torch.Tensor]:
+    """(alpha, h): alpha and beta are rounded to the inputs' dtype, as tensors in memory would be."""
+    dtype = gate.dtype
+    alpha = torch.sigmoid(gate.float()).to(dtype)
+    a = alpha.double()
+    beta = (x.double() * torch.sqrt(1.0 - a * a)).float().to(dtype)
+    return alpha, torch_loop_fwd(alpha, beta)
+
+
+def torch_gated_bwd(
+    alpha: torch.Tensor, x: torch.Tensor, h: torch.Tensor, dout: torch.Tensor
+) -> Tuple[torch.Tensor, torch.Tensor]:
+    """(grad_gate, grad_x) from the rounded alpha of torch_gated_fwd."""
+    galpha, gbeta = torch_loop_bwd(alpha, h, dout)
+    a = alpha.double()
+    om = 1.0 - a * a
+    s = torch.sqrt(om)
+    a_over_s = torch.where(om > 0, a / s, torch.zeros_like(a))
+    grad_x = gbeta.double() * s
+    grad_gate = (galpha.double() - gbeta.double() * x.double() * a_over_s) * a * (1.0 - a)
+    return grad_gate.float(), grad_x.float()
