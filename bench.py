@@ -43,7 +43,7 @@ def parse_args():
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=25)
     ap.add_argument("--case", default="C3_4096", help="workload name from fast_sequential_scan_amd.workloads")
-    ap.add_argument("--dtype", default="bf16", choices=("bf16", "f32"),
+    ap.add_argument("--dtype", default="bf16", choices=("bf16", "f32", "f16"),
                     help="storage type of the tensors (the headline metric is bf16; carries are fp32 either way)")
     ap.add_argument("--op", default="scan", choices=("scan", "gated"),
                     help="scan: the reference's operator (headline metric); gated: the scan with the sigmoid/"
@@ -74,7 +74,7 @@ def main() -> int:
 
     import torch
 
-    from fast_sequential_scan_amd import _native, scan_cu, scan_cu_single, scan_gated
+    from fast_sequential_scan_amd import _native, scan_cu, scan_cu_fp16, scan_cu_single, scan_gated
     from fast_sequential_scan_amd import sequential_scan_cuda as ext
     from fast_sequential_scan_amd.workloads import BASELINE_CASES, make_inputs
 
@@ -107,17 +107,17 @@ def main() -> int:
 
     recipe, bs, seq, d = BASELINE_CASES[args.case]
     n_elem = bs * seq * d
-    is_bf16 = args.dtype == "bf16"
+    is_16bit = args.dtype != "f32"
     gated = args.op == "gated"
-    scan_fn = scan_gated if gated else (scan_cu if is_bf16 else scan_cu_single)
-    tol = 1e-2 if is_bf16 else 1e-4  # the reference's test tolerance for bf16; fp32 differs by carry re-association only
-    kname = "BF16" if is_bf16 else "F32"
-    fss_dtype = _native.FSS_BF16 if is_bf16 else _native.FSS_F32
-    esize = 2 if is_bf16 else 4
+    scan_fn = scan_gated if gated else {"bf16": scan_cu, "f16": scan_cu_fp16, "f32": scan_cu_single}[args.dtype]
+    tol = {"bf16": 1e-2, "f16": 2e-3, "f32": 1e-4}[args.dtype]  # bf16: the reference's test tolerance; fp32 differs by carry re-association only
+    kname = args.dtype.upper()
+    fss_dtype = {"bf16": _native.FSS_BF16, "f16": _native.FSS_F16, "f32": _native.FSS_F32}[args.dtype]
+    esize = 2 if is_16bit else 4
     fwd_bytes_per_elem = FWD_BYTES_PER_ELEM * esize // 2
     # gated backward: reads gate, x, h, dout and writes grad_gate, grad_x = 6 tensors
     bwd_bytes_per_elem = (12 if gated else BWD_BYTES_PER_ELEM) * esize // 2
-    tdtype = torch.bfloat16 if is_bf16 else torch.float32
+    tdtype = {"bf16": torch.bfloat16, "f16": torch.float16, "f32": torch.float32}[args.dtype]
     alpha_c, beta_c, dout_c = make_inputs(recipe, bs, seq, d, dtype=tdtype)
     if gated:
         # first input = the gate pre-activation, second = x; both N(0,1) (the "hawk" recipe before its gating)
@@ -291,7 +291,7 @@ def main() -> int:
 
         # gated bf16: sigmoid lands on the other side of a bf16 rounding boundary for a few elements in
         # 10^5 (device exp2/rcp against the CPU's), so a stated fraction may sit outside the tolerance
-        allowed = 2e-4 if (gated and is_bf16) else 0.0
+        allowed = 2e-4 if (gated and is_16bit) else 0.0
 
         def ok(got, want):
             return bool(((got - want).abs() > tol + tol * want.abs()).float().mean().item() <= allowed)
@@ -323,7 +323,7 @@ def main() -> int:
     try:
         with open(os.path.join(ROOT, "profiles", "hbm_traffic_bs8_seq4096_d1024.json")) as f:
             prof = json.load(f)
-        if prof["case"] == args.case and is_bf16 and not gated:
+        if prof["case"] == args.case and args.dtype == "bf16" and not gated:
             scale_r = prof["copy"]["bytes_read"] / (prof["copy"]["fetch_kib"] * 1024.0)
             scale_w = prof["copy"]["bytes_written"] / (prof["copy"]["write_kib"] * 1024.0)
             for name in ("fwd", "bwd"):
@@ -334,7 +334,7 @@ def main() -> int:
 
     out = {
         "metric": "fwd+bwd scan ms & achieved HBM GB/s (% peak), bf16 bs8 d1024 seq4096"
-        if args.case == "C3_4096" and is_bf16 and not gated
+        if args.case == "C3_4096" and args.dtype == "bf16" and not gated
         else f"fwd+bwd {'gated ' if gated else ''}scan ms & achieved HBM GB/s (% peak), {args.dtype} {args.case}",
         "value": round(value, 1),
         "unit": "GB/s",

@@ -14,7 +14,7 @@ PKG_DIR = os.path.dirname(os.path.abspath(__file__))
 # FSS_SCAN_LIBRARY points at an alternative build of the same library (tuning experiments)
 LIB_PATH = os.environ.get("FSS_SCAN_LIBRARY") or os.path.join(PKG_DIR, "_lib", "libfss_scan.so")
 
-FSS_BF16, FSS_F32 = 0, 1
+FSS_BF16, FSS_F32, FSS_F16 = 0, 1, 2
 FSS_FWD, FSS_BWD, FSS_GATED_FWD, FSS_GATED_BWD = 0, 1, 2, 3
 FSS_OK = 0
 FSS_ERR_CHAIN_TIMEOUT = 7

@@ -76,15 +76,43 @@ typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 typedef float f32x2 __attribute__((ext_vector_type(2)));
 typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
 
+typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
+
+__device__ __forceinline__ float as_f32(uint32_t u) { return __builtin_bit_cast(float, u); }
+__device__ __forceinline__ uint32_t as_u32(float f) { return __builtin_bit_cast(uint32_t, f); }
+
+// Storage types.  The 16-bit ones say how the two halves of a packed dword become
+// fp32 and back (round to nearest even both ways).
 struct BF16 {
   static constexpr int kBytes = 2;
+  static __device__ __forceinline__ float lo(uint32_t w) { return as_f32(w << 16); }
+  static __device__ __forceinline__ float hi(uint32_t w) { return as_f32(w & 0xffff0000u); }
+  // as __float2bfloat16 of the reference (csrc/include/sequential_scan_kernel_bf16.cuh:54)
+  static __device__ __forceinline__ uint32_t pack2(float a, float b) {
+    f32x2 v = {a, b};
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, bf16x2));
+  }
+  static __device__ __forceinline__ uint32_t bits(float x) { return as_u32(x) >> 16; }  // x exactly representable
+};
+struct F16 {
+  static constexpr int kBytes = 2;
+  static __device__ __forceinline__ float lo(uint32_t w) {
+    return static_cast<float>(__builtin_bit_cast(_Float16, static_cast<uint16_t>(w)));
+  }
+  static __device__ __forceinline__ float hi(uint32_t w) {
+    return static_cast<float>(__builtin_bit_cast(_Float16, static_cast<uint16_t>(w >> 16)));
+  }
+  static __device__ __forceinline__ uint32_t pack2(float a, float b) {
+    f32x2 v = {a, b};
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, f16x2));
+  }
+  static __device__ __forceinline__ uint32_t bits(float x) {
+    return __builtin_bit_cast(uint16_t, static_cast<_Float16>(x));
+  }
 };
 struct F32 {
   static constexpr int kBytes = 4;
 };
-
-__device__ __forceinline__ float as_f32(uint32_t u) { return __builtin_bit_cast(float, u); }
-__device__ __forceinline__ uint32_t as_u32(float f) { return __builtin_bit_cast(uint32_t, f); }
 
 // Pins a wave-uniform pointer into scalar registers, so that `p + lane_offset`
 // becomes the scalar-base + 32-bit-vector-offset form of a global access and
@@ -153,12 +181,12 @@ struct DwordIO<4, NT> {
 };
 
 // One row segment owned by a lane: VEC channels of element type E, kept packed.
-template <typename E, int VEC>
+template <typename E, int VEC, int BYTES = E::kBytes>
 struct Row;
 
-template <int VEC>
-struct Row<BF16, VEC> {
-  static_assert(VEC == 2 || VEC == 4 || VEC == 8, "bf16 vector width");
+template <typename E, int VEC>
+struct Row<E, VEC, 2> {
+  static_assert(VEC == 2 || VEC == 4 || VEC == 8, "16-bit vector width");
   static constexpr int kDwords = VEC / 2;
   static constexpr int kBytes = VEC * 2;
   uint32_t dw[kDwords];
@@ -170,27 +198,20 @@ struct Row<BF16, VEC> {
   __device__ __forceinline__ void store(gptr_t p) const {
     DwordIO<kDwords, NT>::store(p, dw);
   }
-  __device__ __forceinline__ float get(int i) const {
-    const uint32_t w = dw[i >> 1];
-    return (i & 1) ? as_f32(w & 0xffff0000u) : as_f32(w << 16);
-  }
-  __device__ __forceinline__ void fill(float x) {  // x exactly representable in bf16
-    const uint32_t hi = as_u32(x) >> 16;
+  __device__ __forceinline__ float get(int i) const { return (i & 1) ? E::hi(dw[i >> 1]) : E::lo(dw[i >> 1]); }
+  __device__ __forceinline__ void fill(float x) {  // x exactly representable in E
+    const uint32_t b = E::bits(x);
 #pragma unroll
-    for (int i = 0; i < kDwords; ++i) dw[i] = hi | (hi << 16);
+    for (int i = 0; i < kDwords; ++i) dw[i] = b | (b << 16);
   }
-  // round-to-nearest-even, as __float2bfloat16 of the reference (bf16.cuh:54)
   __device__ __forceinline__ void pack(const float *f) {
 #pragma unroll
-    for (int i = 0; i < kDwords; ++i) {
-      f32x2 v = {f[2 * i], f[2 * i + 1]};
-      dw[i] = __builtin_bit_cast(uint32_t, __builtin_convertvector(v, bf16x2));
-    }
+    for (int i = 0; i < kDwords; ++i) dw[i] = E::pack2(f[2 * i], f[2 * i + 1]);
   }
 };
 
-template <>
-struct Row<BF16, 1> {
+template <typename E>
+struct Row<E, 1, 2> {
   static constexpr int kDwords = 1;
   static constexpr int kBytes = 2;
   uint32_t dw[1];
@@ -207,16 +228,13 @@ struct Row<BF16, 1> {
     else
       *q = static_cast<uint16_t>(dw[0]);
   }
-  __device__ __forceinline__ float get(int) const { return as_f32(dw[0] << 16); }
-  __device__ __forceinline__ void fill(float x) { dw[0] = as_u32(x) >> 16; }
-  __device__ __forceinline__ void pack(const float *f) {
-    f32x2 v = {f[0], 0.0f};
-    dw[0] = __builtin_bit_cast(uint32_t, __builtin_convertvector(v, bf16x2)) & 0xffffu;
-  }
+  __device__ __forceinline__ float get(int) const { return E::lo(dw[0]); }
+  __device__ __forceinline__ void fill(float x) { dw[0] = E::bits(x); }
+  __device__ __forceinline__ void pack(const float *f) { dw[0] = E::pack2(f[0], 0.0f) & 0xffffu; }
 };
 
-template <int VEC>
-struct Row<F32, VEC> {
+template <typename E, int VEC>
+struct Row<E, VEC, 4> {
   static_assert(VEC == 1 || VEC == 2 || VEC == 4, "fp32 vector width");
   static constexpr int kDwords = VEC;
   static constexpr int kBytes = VEC * 4;
@@ -1040,7 +1058,7 @@ uint64_t *g_trace = nullptr;
 inline int64_t ceil_div(int64_t a, int64_t b) { return (a + b - 1) / b; }
 
 // Register budget: packed dwords a lane may hold per input tensor.
-inline int max_vec_steps(int dtype) { return dtype == FSS_BF16 ? 64 : 32; }  // vec*steps
+inline int max_vec_steps(int dtype) { return dtype != FSS_F32 ? 64 : 32; }  // vec*steps
 
 // LDS: one (A,B) slot per lane and vector element for every wave, twice (tiles
 // alternate between two sets), the same for every wave that looks back, and two
@@ -1058,13 +1076,13 @@ inline size_t lds_bytes(int waves, int vec) {
 inline bool config_valid(const fss_config &c, int dtype, bool gated = false, int dir = FSS_FWD) {
   // the gated kernels exist for 4 bytes (or one element) per lane; their backward holds
   // four tensors, so at most 16 timesteps per lane
-  if (gated && (c.vec > (dtype == FSS_BF16 ? 2 : 1) || (dir == FSS_BWD && c.steps > 16))) return false;
-  const bool vec_ok = dtype == FSS_BF16 ? (c.vec == 1 || c.vec == 2 || c.vec == 4 || c.vec == 8)
+  if (gated && (c.vec > (dtype != FSS_F32 ? 2 : 1) || (dir == FSS_BWD && c.steps > 16))) return false;
+  const bool vec_ok = dtype != FSS_F32 ? (c.vec == 1 || c.vec == 2 || c.vec == 4 || c.vec == 8)
                                         : (c.vec == 1 || c.vec == 2 || c.vec == 4);
   const bool steps_ok = c.steps == 8 || c.steps == 16 || c.steps == 32;
   if (!vec_ok || !steps_ok) return false;
   if (c.vec * c.steps > max_vec_steps(dtype)) return false;
-  if (dtype == FSS_BF16 && c.vec == 1 && c.steps > 32) return false;
+  if (dtype != FSS_F32 && c.vec == 1 && c.steps > 32) return false;
   if (c.waves < 1 || c.waves > 16) return false;
   if (lds_bytes(c.waves, c.vec) > kLdsBudget) return false;
   return true;
@@ -1082,18 +1100,18 @@ void complete_config(fss_config &c, int64_t bs, int64_t seq, int64_t d, int dtyp
   // chains and stores) beats 16 unless the chain of chunks is long; with few
   // channels, one channel per lane (twice the column tiles) and shorter slices
   // put more waves in flight.
-  const int esize = dtype == FSS_BF16 ? 2 : 4;
+  const int esize = dtype != FSS_F32 ? 2 : 4;
   const int64_t channels = bs * d;
   if (c.vec == 0) {
     // 4 bytes per lane and load either way: two bf16 channels or one fp32 channel
-    const bool can2 = dtype == FSS_BF16 && d % 2 == 0 && align % (2 * static_cast<size_t>(esize)) == 0;
+    const bool can2 = dtype != FSS_F32 && d % 2 == 0 && align % (2 * static_cast<size_t>(esize)) == 0;
     int v = can2 ? 2 : 1;
     // few channels: more, narrower column tiles; also never pad a row to twice its width
     if (v == 2 && (channels < 8192 || ceil_div(d, 128) * 128 >= 2 * ceil_div(d, 64) * 64)) v = 1;
     c.vec = v;
   }
   // packed dwords one lane holds per timestep and tensor
-  const int dwords = dtype == FSS_BF16 ? (c.vec + 1) / 2 : c.vec;
+  const int dwords = dtype != FSS_F32 ? (c.vec + 1) / 2 : c.vec;
   if (c.steps == 0) {
     int s = 32 / dwords;  // 32 packed dwords per lane and tensor (the backward loads half of its third one late)
     if (s > 32) s = 32;
@@ -1103,7 +1121,7 @@ void complete_config(fss_config &c, int64_t bs, int64_t seq, int64_t d, int dtyp
     // as fast in bf16 and 6 % faster in fp32 (forward and backward alternating).
     if (dir == FSS_BWD && s == 32 && (gated || ceil_div(seq, static_cast<int64_t>(8) * 32) <= 16)) s = 16;
     // gated forward in bf16: 32 steps spill (the gating needs temporaries), 16 measured faster
-    if (gated && dir == FSS_FWD && dtype == FSS_BF16 && s == 32) s = 16;
+    if (gated && dir == FSS_FWD && dtype != FSS_F32 && s == 32) s = 16;
     // small problems: shorter slices until there are two 8-wave tiles per CU (512), as
     // long as the machine still gets a few waves per SIMD out of it
     const int64_t ctiles = bs * ceil_div(d, 64 * c.vec);
@@ -1136,11 +1154,11 @@ struct Plan {
 int make_plan(Plan &pl, int64_t bs, int64_t seq, int64_t d, int dtype, int dir, size_t align,
               const fss_config *user) {
   if (bs < 0 || seq < 0 || d < 0) return FSS_ERR_BAD_SHAPE;
-  if (dtype != FSS_BF16 && dtype != FSS_F32) return FSS_ERR_BAD_CONFIG;
+  if (dtype != FSS_BF16 && dtype != FSS_F32 && dtype != FSS_F16) return FSS_ERR_BAD_CONFIG;
   if (dir < FSS_FWD || dir > FSS_GATED_BWD) return FSS_ERR_BAD_CONFIG;
   const bool gated = dir >= FSS_GATED_FWD;
   dir &= 1;
-  const int esize = dtype == FSS_BF16 ? 2 : 4;
+  const int esize = dtype != FSS_F32 ? 2 : 4;
   // bs*seq*d*esize must fit int64
   if (bs > 0 && seq > 0 && d > 0) {
     const __int128 total = static_cast<__int128>(bs) * seq * d * esize;
@@ -1260,7 +1278,7 @@ int launch_one(const ScanArgs &args, const StateArgs<true> &state, const Plan &p
 
 template <typename E, bool BWD, bool STATE>
 int launch_typed(const ScanArgs &args, const StateArgs<true> &state, const Plan &pl, hipStream_t stream) {
-  constexpr bool is_bf16 = E::kBytes == 2;
+  constexpr bool is_16bit = E::kBytes == 2;
   const int key = pl.cfg.vec * 100 + pl.cfg.steps;
   switch (key) {
 #define FSS_CASE(V, S) \
@@ -1275,7 +1293,7 @@ int launch_typed(const ScanArgs &args, const StateArgs<true> &state, const Plan 
     default:
       break;
   }
-  if constexpr (is_bf16) {
+  if constexpr (is_16bit) {
     switch (key) {
       FSS_CASE(2, 32)
       FSS_CASE(4, 16)
@@ -1291,7 +1309,7 @@ int launch_typed(const ScanArgs &args, const StateArgs<true> &state, const Plan 
 // The gated kernels: 4 bytes (bf16 x2, fp32 x1) or one bf16 element per lane.
 template <typename E, bool BWD>
 int launch_gated(const ScanArgs &args, const Plan &pl, hipStream_t stream) {
-  constexpr bool is_bf16 = E::kBytes == 2;
+  constexpr bool is_16bit = E::kBytes == 2;
   const StateArgs<true> none = {nullptr, nullptr, nullptr};
   const int key = pl.cfg.vec * 100 + pl.cfg.steps;
   switch (key) {
@@ -1306,7 +1324,7 @@ int launch_gated(const ScanArgs &args, const Plan &pl, hipStream_t stream) {
   if constexpr (!BWD) {
     if (key == 132) return launch_one<E, 1, 32, BWD, false, true>(args, none, pl, stream);
   }
-  if constexpr (is_bf16) {
+  if constexpr (is_16bit) {
     switch (key) {
       FSS_CASE(2, 8)
       FSS_CASE(2, 16)
@@ -1329,12 +1347,12 @@ int run_scan(int dtype, int dir, const void *alpha, const void *in_b, const void
   const int plan_dir = dir;
   dir &= 1;
   if (bs < 0 || seq < 0 || d < 0) return FSS_ERR_BAD_SHAPE;
-  if (dtype != FSS_BF16 && dtype != FSS_F32) return FSS_ERR_BAD_CONFIG;
+  if (dtype != FSS_BF16 && dtype != FSS_F32 && dtype != FSS_F16) return FSS_ERR_BAD_CONFIG;
   if (bs == 0 || seq == 0 || d == 0) return FSS_OK;
   if (!alpha || !in_b || !out0) return FSS_ERR_NULL_POINTER;
   if (dir == FSS_BWD && (!in_h || !out1)) return FSS_ERR_NULL_POINTER;
   if (gated && dir == FSS_BWD && !in_x) return FSS_ERR_NULL_POINTER;
-  const size_t esize = dtype == FSS_BF16 ? 2 : 4;
+  const size_t esize = dtype != FSS_F32 ? 2 : 4;
   const size_t align = dir == FSS_BWD ? common_alignment({alpha, in_b, in_h, out0, out1, in_x})
                                       : common_alignment({alpha, in_b, out0});
   if (align < esize) return FSS_ERR_MISALIGNED;
@@ -1372,17 +1390,18 @@ int run_scan(int dtype, int dir, const void *alpha, const void *in_b, const void
   args.trace = g_trace;
 #endif
   hipStream_t s = static_cast<hipStream_t>(stream);
-  if (gated) {
-    if (dtype == FSS_BF16) return dir == FSS_BWD ? launch_gated<BF16, true>(args, pl, s) : launch_gated<BF16, false>(args, pl, s);
-    return dir == FSS_BWD ? launch_gated<F32, true>(args, pl, s) : launch_gated<F32, false>(args, pl, s);
-  }
   const bool st = state_in || state_out || h_before;
-  if (dtype == FSS_BF16) {
-    if (dir == FSS_BWD) return st ? launch_typed<BF16, true, true>(args, state, pl, s) : launch_typed<BF16, true, false>(args, state, pl, s);
-    return st ? launch_typed<BF16, false, true>(args, state, pl, s) : launch_typed<BF16, false, false>(args, state, pl, s);
-  }
-  if (dir == FSS_BWD) return st ? launch_typed<F32, true, true>(args, state, pl, s) : launch_typed<F32, true, false>(args, state, pl, s);
-  return st ? launch_typed<F32, false, true>(args, state, pl, s) : launch_typed<F32, false, false>(args, state, pl, s);
+  const bool bwd = dir == FSS_BWD;
+#define FSS_DISPATCH(E)                                                                        \
+  do {                                                                                         \
+    if (gated) return bwd ? launch_gated<E, true>(args, pl, s) : launch_gated<E, false>(args, pl, s); \
+    if (bwd) return st ? launch_typed<E, true, true>(args, state, pl, s) : launch_typed<E, true, false>(args, state, pl, s); \
+    return st ? launch_typed<E, false, true>(args, state, pl, s) : launch_typed<E, false, false>(args, state, pl, s); \
+  } while (0)
+  if (dtype == FSS_BF16) FSS_DISPATCH(BF16);
+  if (dtype == FSS_F16) FSS_DISPATCH(F16);
+  FSS_DISPATCH(F32);
+#undef FSS_DISPATCH
 }
 
 }  // namespace fss
@@ -1424,7 +1443,7 @@ size_t fss_workspace_bytes(int64_t bs, int64_t seq, int64_t d, int dtype, int di
 
 size_t fss_workspace_bytes_max(int64_t bs, int64_t seq, int64_t d) {
   size_t best = fss::kHeaderBytes;
-  for (int dtype = 0; dtype < 2; ++dtype)
+  for (int dtype = FSS_BF16; dtype <= FSS_F16; ++dtype)
     for (int dir = FSS_FWD; dir <= FSS_GATED_BWD; ++dir)
       for (size_t align = 2; align <= 16; align <<= 1) {
         fss::Plan pl;

@@ -16,7 +16,10 @@ from torch.autograd.function import once_differentiable
 
 from . import sequential_scan_cuda as _ext
 
-__all__ = ["SequentialScan", "SequentialScanSingle", "SequentialScanState", "scan", "scan_single", "scan_with_state"]
+__all__ = [
+    "SequentialScan", "SequentialScanSingle", "SequentialScanFp16", "SequentialScanState", "SequentialScanGated",
+    "scan", "scan_single", "scan_fp16", "scan_with_state", "scan_gated",
+]
 
 
 class SequentialScan(Function):
@@ -66,6 +69,28 @@ def scan(alpha: torch.Tensor, beta: torch.Tensor) -> torch.Tensor:
 def scan_single(alpha: torch.Tensor, beta: torch.Tensor) -> torch.Tensor:
     """The same recurrence on fp32 tensors."""
     return SequentialScanSingle.apply(alpha, beta)
+
+
+class SequentialScanFp16(Function):
+    """The recurrence on IEEE half tensors (not in the reference, whose half type is bf16)."""
+
+    @staticmethod
+    def forward(ctx: Any, input_alpha: torch.Tensor, input_beta: torch.Tensor) -> torch.Tensor:
+        out = _ext.scan_forward_fp16(input_alpha, input_beta)
+        ctx.save_for_backward(input_alpha, out)
+        return out
+
+    @staticmethod
+    @once_differentiable
+    def backward(ctx: Any, grad_output: torch.Tensor) -> Tuple[torch.Tensor, torch.Tensor]:
+        input_alpha, out = ctx.saved_tensors
+        grad_alpha, grad_beta = _ext.scan_backward_fp16(input_alpha, out, grad_output)
+        return grad_alpha, grad_beta
+
+
+def scan_fp16(alpha: torch.Tensor, beta: torch.Tensor) -> torch.Tensor:
+    """The same recurrence on fp16 tensors."""
+    return SequentialScanFp16.apply(alpha, beta)
 
 
 class SequentialScanState(Function):

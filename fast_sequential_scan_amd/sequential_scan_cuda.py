@@ -23,11 +23,12 @@ from . import _native
 
 __all__ = [
     "scan_forward", "scan_backward", "scan_forward_half", "scan_backward_half",
+    "scan_forward_fp16", "scan_backward_fp16",
     "scan_forward_state", "scan_backward_state",
     "gated_scan_forward", "gated_scan_backward",
 ]
 
-_DTYPE_CODE = {torch.bfloat16: _native.FSS_BF16, torch.float32: _native.FSS_F32}
+_DTYPE_CODE = {torch.bfloat16: _native.FSS_BF16, torch.float32: _native.FSS_F32, torch.float16: _native.FSS_F16}
 
 # one workspace per (device, stream): calls on one stream are ordered, calls on
 # different streams must not share the chaining words
@@ -156,6 +157,16 @@ def scan_backward_half(alpha_saved: torch.Tensor, h_saved: torch.Tensor, grad_ou
     return _backward(torch.bfloat16, alpha_saved, h_saved, grad_out)
 
 
+def scan_forward_fp16(alpha: torch.Tensor, beta: torch.Tensor) -> torch.Tensor:
+    """IEEE half forward (no counterpart in the reference; same kernels, fp32 carries)."""
+    return _forward(torch.float16, alpha, beta)
+
+
+def scan_backward_fp16(alpha_saved: torch.Tensor, h_saved: torch.Tensor, grad_out: torch.Tensor) -> List[torch.Tensor]:
+    """IEEE half backward -> [grad_alpha, grad_beta]."""
+    return _backward(torch.float16, alpha_saved, h_saved, grad_out)
+
+
 # ---- scans with a state entering and leaving the sequence (no counterpart in the reference) ----
 
 
@@ -179,7 +190,7 @@ def scan_forward_state(
     given, ``alpha[:, 0]`` is applied to it) and the un-rounded fp32 state after the last step."""
     dtype = alpha.dtype
     if dtype not in _DTYPE_CODE:
-        raise RuntimeError(f"expected scalar type torch.bfloat16 or torch.float32 for alpha but found {dtype}")
+        raise RuntimeError(f"expected scalar type torch.bfloat16, torch.float16 or torch.float32 for alpha but found {dtype}")
     bs, seq, d = _validate(dtype, alpha=alpha, beta=beta)
     h_before = _state("h_before", h_before, alpha)
     alpha, beta = alpha.contiguous(), beta.contiguous()
@@ -216,7 +227,7 @@ def scan_backward_state(
     """(grad_alpha, grad_beta, grad_h_before); the last is None when ``h_before`` is None."""
     dtype = alpha_saved.dtype
     if dtype not in _DTYPE_CODE:
-        raise RuntimeError(f"expected scalar type torch.bfloat16 or torch.float32 for alpha but found {dtype}")
+        raise RuntimeError(f"expected scalar type torch.bfloat16, torch.float16 or torch.float32 for alpha but found {dtype}")
     bs, seq, d = _validate(dtype, alpha_saved=alpha_saved, h_saved=h_saved, grad_out=grad_out)
     h_before = _state("h_before", h_before, alpha_saved)
     grad_h_last = _state("grad_h_last", grad_h_last, alpha_saved)
@@ -253,7 +264,7 @@ def scan_backward_state(
 
 def _either_dtype(t: torch.Tensor, name: str) -> torch.dtype:
     if t.dtype not in _DTYPE_CODE:
-        raise RuntimeError(f"expected scalar type torch.bfloat16 or torch.float32 for {name} but found {t.dtype}")
+        raise RuntimeError(f"expected scalar type torch.bfloat16, torch.float16 or torch.float32 for {name} but found {t.dtype}")
     return t.dtype
 
 

@@ -65,13 +65,14 @@ typedef enum fss_status {
   FSS_ERR_UNSUPPORTED_DEVICE = 8 /* current device is not gfx950                  */
 } fss_status;
 
-typedef enum fss_dtype { FSS_BF16 = 0, FSS_F32 = 1 } fss_dtype;
+/* FSS_F16 (IEEE half) has no counterpart in the reference; same kernels, same fp32 carries */
+typedef enum fss_dtype { FSS_BF16 = 0, FSS_F32 = 1, FSS_F16 = 2 } fss_dtype;
 /* FSS_GATED_*: the gated scans below (they chunk the sequence differently) */
 typedef enum fss_dir { FSS_FWD = 0, FSS_BWD = 1, FSS_GATED_FWD = 2, FSS_GATED_BWD = 3 } fss_dir;
 
 /*
  * Launch configuration.  Zero in a field means "choose for me".
- *   vec    channels per lane (bf16: 1,2,4,8; fp32: 1,2,4); needs d % vec == 0 and
+ *   vec    channels per lane (bf16/fp16: 1,2,4,8; fp32: 1,2,4); needs d % vec == 0 and
  *          tensors aligned to vec elements
  *   steps  timesteps each lane keeps in registers (8, 16 or 32; vec*steps bounded
  *          by the register budget of the direction)
@@ -202,7 +203,7 @@ int fss_scan_bwd_state(int dtype, const void *alpha, const void *h, const void *
  *   grad_gate[t] = g[t] * (h[t-1] - x[t]*alpha[t]/s[t]) * alpha[t]*(1 - alpha[t])   (h[-1] = 0)
  * Where alpha rounds to exactly 1 (s = 0) the x term is dropped (torch's autograd gives
  * inf/nan there).  gate[:,0,:] is read (beta[0] depends on it).  The six tensors of a
- * backward must not overlap.  vec is 1 or 2 (bf16) / 1 (fp32); steps at most 16 in the
+ * backward must not overlap.  vec is 1 or 2 (bf16, fp16) / 1 (fp32); steps at most 16 in the
  * backward.  Use FSS_GATED_FWD / FSS_GATED_BWD as `dir` of fss_workspace_bytes and
  * fss_choose_config.
  */

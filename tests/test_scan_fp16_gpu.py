@@ -1,0 +1,116 @@
+"""GPU tests of the scans on IEEE half tensors (FSS_F16; not in the reference, whose
+16-bit type is bf16).  Same kernels, fp32 carries, outputs rounded to nearest even.
+
+Oracle: the pinned fp32 scan on the same fp16-valued inputs.  Two bars: rtol = atol = 2e-3
+against its fp32 output (fp16 keeps 11 significant bits: half an ulp is 4.9e-4 relative),
+and at most 2 fp16 ulps from that output rounded to fp16 (bit-exact where one wave
+covers the whole sequence, since nothing is re-associated there).
+"""
+import numpy as np
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+from fast_sequential_scan_amd import scan_cu_fp16, scan_gated, scan_with_state  # noqa: E402
+from fast_sequential_scan_amd import sequential_scan_cuda as ext  # noqa: E402
+from fast_sequential_scan_amd.workloads import make_inputs  # noqa: E402
+
+DEV = "cuda:0"
+RTOL = ATOL = 2e-3
+
+
+def _bits(a16: np.ndarray) -> np.ndarray:
+    u = a16.view(np.uint16).astype(np.int32)
+    return np.where(u & 0x8000, -(u & 0x7FFF), u & 0x7FFF)
+
+
+def _check(got: torch.Tensor, want32: np.ndarray, what: str, exact: bool):
+    got16 = got.detach().cpu().numpy()
+    assert got16.dtype == np.float16
+    got32 = got16.astype(np.float32)
+    bad = ~(np.abs(got32 - want32) <= ATOL + RTOL * np.abs(want32))
+    assert not bad.any(), f"{what}: {bad.sum()} of {bad.size} outside rtol=atol=2e-3, worst {np.abs(got32 - want32).max():.4g}"
+    want16 = want32.astype(np.float16)
+    if exact:
+        np.testing.assert_array_equal(got16.view(np.uint16), want16.view(np.uint16), err_msg=what)
+    else:
+        finite = np.isfinite(want16)
+        dist = np.abs(_bits(got16[finite]) - _bits(want16[finite]))
+        close = np.abs(got32[finite] - want32[finite]) <= 2e-4  # near-cancelling results
+        assert ((dist <= 2) | close).all(), f"{what}: max ulp distance {dist.max()}"
+
+
+def _run(oracle, shape, recipe="sigmoid", config=None, exact=False, seed=0):
+    alpha, beta, dout = make_inputs(recipe, *shape, dtype=torch.float16, seed=seed)
+    a, b, do = alpha.to(DEV), beta.to(DEV), dout.to(DEV)
+    h = ext._forward(torch.float16, a, b, config)
+    ga, gb = ext._backward(torch.float16, a, h, do, config)
+    ext.workspace_status()
+    a32, b32, d32 = alpha.float().numpy(), beta.float().numpy(), dout.float().numpy()
+    _check(h, oracle.scan_fwd_f32(a32, b32, fused=True), "h", exact)
+    # the backward is fed the stored (rounded) h, as the product path does
+    ga32, gb32 = oracle.scan_bwd_f32(a32, h.float().cpu().numpy(), d32, fused=True)
+    _check(gb, gb32, "grad_beta", exact)
+    _check(ga, ga32, "grad_alpha", exact)
+
+
+@pytest.mark.parametrize("seq", [1, 2, 7, 8])
+@pytest.mark.parametrize("d", [1, 6, 64, 136])
+def test_fp16_one_wave_is_bit_exact(oracle, seq, d):
+    for v in {1, 2 if d % 2 == 0 else 1}:
+        _run(oracle, (3, seq, d), recipe="normal", config=(v, 8, 1), exact=True, seed=seq * 100 + d)
+    _run(oracle, (3, seq, d), recipe="normal", exact=True, seed=seq * 100 + d)
+
+
+@pytest.mark.parametrize("shape", [(2, 31, 24), (3, 257, 192), (2, 1000, 768), (2, 3000, 130), (8, 2048, 1024), (1, 20011, 256)])
+def test_fp16_default_config(oracle, shape):
+    _run(oracle, shape, seed=sum(shape))
+
+
+@pytest.mark.parametrize("config", [(1, 8, 4), (2, 8, 16), (2, 16, 2), (4, 8, 8), (8, 8, 6), (2, 32, 8), (2, 16, 8, 5)],
+                         ids=lambda c: "v%d_s%d_w%d" % c[:3])
+def test_fp16_result_does_not_depend_on_chunking(oracle, config):
+    _run(oracle, (2, 1203, 256), config=config, seed=3)
+
+
+def test_fp16_headline_shape_and_scaling_property(oracle):
+    """bs8 seq4096 d1024 against the oracle, and a size-independent property: scaling beta by a
+    power of two scales h by it exactly (no overflow or underflow at these magnitudes)."""
+    _run(oracle, (8, 4096, 1024), seed=4)
+    alpha, beta, _ = (t.to(DEV) for t in make_inputs("sigmoid", 8, 4096, 1024, dtype=torch.float16, seed=4))
+    h = ext.scan_forward_fp16(alpha, beta)
+    h4 = ext.scan_forward_fp16(alpha, 4 * beta)
+    big = h.abs().float() >= 2.0 ** -12  # fp16 subnormals do not scale exactly
+    assert torch.equal(h4[big], (4 * h)[big])
+
+
+def test_fp16_overflow_saturates_to_inf_like_a_cast():
+    alpha = torch.full((1, 40, 64), 2.0, dtype=torch.float16, device=DEV)
+    beta = torch.ones_like(alpha)
+    h = ext.scan_forward_fp16(alpha, beta)  # h[t] = 2^(t+1) - 1
+    want = torch.tensor([2.0 ** (t + 1) - 1 for t in range(40)]).to(torch.float16).to(DEV)
+    assert torch.equal(h[0, :, 0], want) and torch.isinf(h[0, 20:, :]).all()
+
+
+def test_fp16_autograd_state_and_gated(oracle):
+    g = torch.Generator().manual_seed(5)
+    shape = (2, 300, 96)
+    alpha = torch.sigmoid(torch.randn(shape, generator=g)).to(torch.float16)
+    beta, dout = torch.randn(shape, generator=g).to(torch.float16), torch.randn(shape, generator=g).to(torch.float16)
+    a, b = alpha.to(DEV).requires_grad_(True), beta.to(DEV).requires_grad_(True)
+    h = scan_cu_fp16(a, b)
+    h.backward(dout.to(DEV))
+    a32, b32 = alpha.float().numpy(), beta.float().numpy()
+    _check(h, oracle.scan_fwd_f32(a32, b32, fused=True), "h", False)
+    ga32, gb32 = oracle.scan_bwd_f32(a32, h.detach().float().cpu().numpy(), dout.float().numpy(), fused=True)
+    _check(a.grad, ga32, "grad_alpha", False)
+    _check(b.grad, gb32, "grad_beta", False)
+    # the state entry points and the gated scan take fp16 as well
+    h2, last = scan_with_state(alpha.to(DEV), beta.to(DEV), None)
+    assert torch.equal(h2, h.detach()) and last.dtype == torch.float32
+    gate = torch.randn(shape, generator=g).to(torch.float16)
+    hg = scan_gated(gate.to(DEV), beta.to(DEV))
+    want = oracle.gated_scan_fwd(gate.float().numpy(), b32, "f32")  # fp16 rounding of alpha/beta: within tolerance
+    got = hg.float().cpu().numpy()
+    assert (np.abs(got - want) <= 5e-3 + 5e-3 * np.abs(want)).all()
