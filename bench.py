@@ -45,9 +45,10 @@ def parse_args():
     ap.add_argument("--case", default="C3_4096", help="workload name from fast_sequential_scan_amd.workloads")
     ap.add_argument("--dtype", default="bf16", choices=("bf16", "f32", "f16"),
                     help="storage type of the tensors (the headline metric is bf16; carries are fp32 either way)")
-    ap.add_argument("--op", default="scan", choices=("scan", "gated"),
+    ap.add_argument("--op", default="scan", choices=("scan", "gated", "cm"),
                     help="scan: the reference's operator (headline metric); gated: the scan with the sigmoid/"
-                         "sqrt(1-alpha^2) gating computed inside the kernels (9 tensors of traffic per step)")
+                         "sqrt(1-alpha^2) gating computed inside the kernels (9 tensors of traffic per step); "
+                         "cm: the scan on channel-major (bs, d, seq) tensors")
     ap.add_argument("--config", default=None, help="explicit vec,steps,waves for both kernels (tuning)")
     ap.add_argument("--fwd-config", default=None)
     ap.add_argument("--bwd-config", default=None)
@@ -74,7 +75,7 @@ def main() -> int:
 
     import torch
 
-    from fast_sequential_scan_amd import _native, scan_cu, scan_cu_fp16, scan_cu_single, scan_gated
+    from fast_sequential_scan_amd import _native, scan_cm, scan_cu, scan_cu_fp16, scan_cu_single, scan_gated
     from fast_sequential_scan_amd import sequential_scan_cuda as ext
     from fast_sequential_scan_amd.workloads import BASELINE_CASES, make_inputs
 
@@ -109,7 +110,8 @@ def main() -> int:
     n_elem = bs * seq * d
     is_16bit = args.dtype != "f32"
     gated = args.op == "gated"
-    scan_fn = scan_gated if gated else {"bf16": scan_cu, "f16": scan_cu_fp16, "f32": scan_cu_single}[args.dtype]
+    cm = args.op == "cm"
+    scan_fn = scan_gated if gated else scan_cm if cm else {"bf16": scan_cu, "f16": scan_cu_fp16, "f32": scan_cu_single}[args.dtype]
     tol = {"bf16": 1e-2, "f16": 2e-3, "f32": 1e-4}[args.dtype]  # bf16: the reference's test tolerance; fp32 differs by carry re-association only
     kname = args.dtype.upper()
     fss_dtype = {"bf16": _native.FSS_BF16, "f16": _native.FSS_F16, "f32": _native.FSS_F32}[args.dtype]
@@ -124,7 +126,10 @@ def main() -> int:
         gen = torch.Generator().manual_seed(4242)
         alpha_c = torch.randn(bs, seq, d, generator=gen).to(tdtype)
         beta_c = torch.randn(bs, seq, d, generator=gen).to(tdtype)
-    alpha, beta, dout = alpha_c.to(dev), beta_c.to(dev), dout_c.to(dev)
+    if cm:  # the same values, time contiguous on the device; the CPU loop keeps its (bs, seq, d) view
+        alpha, beta, dout = (t.transpose(1, 2).contiguous().to(dev) for t in (alpha_c, beta_c, dout_c))
+    else:
+        alpha, beta, dout = alpha_c.to(dev), beta_c.to(dev), dout_c.to(dev)
     h = torch.empty_like(alpha)
     galpha = torch.empty_like(alpha)
     gbeta = torch.empty_like(alpha)
@@ -139,10 +144,16 @@ def main() -> int:
     stream = torch.cuda.current_stream()
     sp = stream.cuda_stream
     dir_fwd, dir_bwd = (_native.FSS_GATED_FWD, _native.FSS_GATED_BWD) if gated else (_native.FSS_FWD, _native.FSS_BWD)
-    ws_bytes = max(
-        lib.fss_workspace_bytes(bs, seq, d, fss_dtype, dir_fwd, fwd_cfg_p),
-        lib.fss_workspace_bytes(bs, seq, d, fss_dtype, dir_bwd, bwd_cfg_p),
-    )
+    if cm:
+        ws_bytes = max(
+            lib.fss_cm_workspace_bytes(bs, d, seq, fss_dtype, dir_fwd, fwd_cfg_p),
+            lib.fss_cm_workspace_bytes(bs, d, seq, fss_dtype, dir_bwd, bwd_cfg_p),
+        )
+    else:
+        ws_bytes = max(
+            lib.fss_workspace_bytes(bs, seq, d, fss_dtype, dir_fwd, fwd_cfg_p),
+            lib.fss_workspace_bytes(bs, seq, d, fss_dtype, dir_bwd, bwd_cfg_p),
+        )
     ws = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
     _native.check(lib.fss_workspace_init(ws.data_ptr(), ws.numel(), sp))
     pa, pb, pd, ph, pga, pgb, pws = (t.data_ptr() for t in (alpha, beta, dout, h, galpha, gbeta, ws))
@@ -150,6 +161,8 @@ def main() -> int:
     def fwd():
         if gated:
             rc = lib.fss_gated_scan_fwd(fss_dtype, pa, pb, ph, bs, seq, d, pws, ws_bytes, sp, fwd_cfg_p)
+        elif cm:
+            rc = lib.fss_scan_fwd_cm(fss_dtype, pa, pb, ph, bs, d, seq, pws, ws_bytes, sp, fwd_cfg_p)
         else:
             rc = lib.fss_scan_fwd_ex(fss_dtype, pa, pb, ph, bs, seq, d, pws, ws_bytes, sp, fwd_cfg_p)
         if rc:
@@ -158,6 +171,8 @@ def main() -> int:
     def bwd():
         if gated:  # pga receives grad_gate, pgb grad_x
             rc = lib.fss_gated_scan_bwd(fss_dtype, pa, pb, ph, pd, pga, pgb, bs, seq, d, pws, ws_bytes, sp, bwd_cfg_p)
+        elif cm:
+            rc = lib.fss_scan_bwd_cm(fss_dtype, pa, ph, pd, pga, pgb, bs, d, seq, pws, ws_bytes, sp, bwd_cfg_p)
         else:
             rc = lib.fss_scan_bwd_ex(fss_dtype, pa, ph, pd, pga, pgb, bs, seq, d, pws, ws_bytes, sp, bwd_cfg_p)
         if rc:
@@ -166,7 +181,11 @@ def main() -> int:
     chosen = {}
     for name, direction, user in (("fwd", dir_fwd, fwd_cfg), ("bwd", dir_bwd, bwd_cfg)):
         c = _native.FssConfig()
-        lib.fss_choose_config(bs, seq, d, fss_dtype, direction, 16, ctypes.byref(c))
+        if cm:  # 16 bytes per lane; 8 waves, fewer when the sequence is shorter than their reach
+            c.vec = 16 // esize
+            c.waves = min(8, -(-seq // (64 * c.vec)))
+        else:
+            lib.fss_choose_config(bs, seq, d, fss_dtype, direction, 16, ctypes.byref(c))
         chosen[name] = list(user) if user else [c.vec, c.steps, c.waves]
 
     # ---- warm-up, then the timed region: exactly K steps between two synchronisations ----
@@ -270,6 +289,8 @@ def main() -> int:
         bwd()
         torch.cuda.synchronize()
         h_gpu, ga_gpu, gb_gpu = h.float().cpu(), galpha.float().cpu(), gbeta.float().cpu()
+        if cm:
+            h_gpu, ga_gpu, gb_gpu = (t.transpose(1, 2) for t in (h_gpu, ga_gpu, gb_gpu))
         reps, spent = 0, 0.0
         f_times, b_times = [], []
         while reps < 1 or (spent < args.cpu_seconds and reps < 20):
@@ -323,7 +344,7 @@ def main() -> int:
     try:
         with open(os.path.join(ROOT, "profiles", "hbm_traffic_bs8_seq4096_d1024.json")) as f:
             prof = json.load(f)
-        if prof["case"] == args.case and args.dtype == "bf16" and not gated:
+        if prof["case"] == args.case and args.dtype == "bf16" and args.op == "scan":
             scale_r = prof["copy"]["bytes_read"] / (prof["copy"]["fetch_kib"] * 1024.0)
             scale_w = prof["copy"]["bytes_written"] / (prof["copy"]["write_kib"] * 1024.0)
             for name in ("fwd", "bwd"):
@@ -334,8 +355,8 @@ def main() -> int:
 
     out = {
         "metric": "fwd+bwd scan ms & achieved HBM GB/s (% peak), bf16 bs8 d1024 seq4096"
-        if args.case == "C3_4096" and args.dtype == "bf16" and not gated
-        else f"fwd+bwd {'gated ' if gated else ''}scan ms & achieved HBM GB/s (% peak), {args.dtype} {args.case}",
+        if args.case == "C3_4096" and args.dtype == "bf16" and args.op == "scan"
+        else f"fwd+bwd {'gated ' if gated else 'channel-major ' if cm else ''}scan ms & achieved HBM GB/s (% peak), {args.dtype} {args.case}",
         "value": round(value, 1),
         "unit": "GB/s",
         "n_gpus": 1,
@@ -348,7 +369,7 @@ def main() -> int:
         "dtype": args.dtype,
         "data": "synthetic",
         "config": {
-            "workload": f"{args.case}: bs{bs} seq{seq} d{d}, {'gated scan of N(0,1) gate and x' if gated else 'recipe ' + recipe}, {args.dtype} storage / fp32 carries, forward+backward",
+            "workload": f"{args.case}: bs{bs} seq{seq} d{d}, {'gated scan of N(0,1) gate and x' if gated else 'recipe ' + recipe}{', tensors (bs, d, seq)' if cm else ''}, {args.dtype} storage / fp32 carries, forward+backward",
             "bs": bs, "seq": seq, "d_model": d,
             "launch_config_fwd_vec_steps_waves": chosen["fwd"],
             "launch_config_bwd_vec_steps_waves": chosen["bwd"],
@@ -365,7 +386,7 @@ def main() -> int:
         "bwd_ms_event_raw": round(statistics.fmean(bwd_raw), 5),
         "roofline": {
             "bound": "hbm",
-            "kernel": f"scan_kernel<{kname},...,BWD=true{',GATED' if gated else ''}> (backward scan)",
+            "kernel": f"{'cm_' if cm else ''}scan_kernel<{kname},...,BWD=true{',GATED' if gated else ''}> (backward scan)",
             "achieved": round(bwd_gbps, 1),
             "peak": HBM_PEAK_GBPS,
             "unit": "GB/s",
@@ -376,7 +397,7 @@ def main() -> int:
         },
         "roofline_fwd": {
             "bound": "hbm",
-            "kernel": f"scan_kernel<{kname},...,BWD=false{',GATED' if gated else ''}> (forward scan)",
+            "kernel": f"{'cm_' if cm else ''}scan_kernel<{kname},...,BWD=false{',GATED' if gated else ''}> (forward scan)",
             "achieved": round(fwd_gbps, 1),
             "peak": HBM_PEAK_GBPS,
             "unit": "GB/s",

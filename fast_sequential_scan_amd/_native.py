@@ -38,6 +38,9 @@ EXPORTED_SYMBOLS = (
     "fss_scan_bwd_state",
     "fss_gated_scan_fwd",
     "fss_gated_scan_bwd",
+    "fss_cm_workspace_bytes",
+    "fss_scan_fwd_cm",
+    "fss_scan_bwd_cm",
     "fss_copy_bytes",
 )
 
@@ -106,6 +109,12 @@ def _declare(lib: ctypes.CDLL) -> None:
     lib.fss_gated_scan_fwd.argtypes = [_int, _vp, _vp, _vp, _i64, _i64, _i64, _vp, _sz, _vp, _cfgp]
     lib.fss_gated_scan_bwd.restype = _int
     lib.fss_gated_scan_bwd.argtypes = [_int, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _vp, _sz, _vp, _cfgp]
+    lib.fss_cm_workspace_bytes.restype = _sz
+    lib.fss_cm_workspace_bytes.argtypes = [_i64, _i64, _i64, _int, _int, _cfgp]
+    lib.fss_scan_fwd_cm.restype = _int
+    lib.fss_scan_fwd_cm.argtypes = [_int, _vp, _vp, _vp, _i64, _i64, _i64, _vp, _sz, _vp, _cfgp]
+    lib.fss_scan_bwd_cm.restype = _int
+    lib.fss_scan_bwd_cm.argtypes = [_int, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _vp, _sz, _vp, _cfgp]
     lib.fss_copy_bytes.argtypes = [_vp, _vp, _sz, _vp]
 
 

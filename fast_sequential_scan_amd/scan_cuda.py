@@ -18,7 +18,7 @@ from . import sequential_scan_cuda as _ext
 
 __all__ = [
     "SequentialScan", "SequentialScanSingle", "SequentialScanFp16", "SequentialScanState", "SequentialScanGated",
-    "scan", "scan_single", "scan_fp16", "scan_with_state", "scan_gated",
+    "SequentialScanChannelMajor", "scan", "scan_single", "scan_fp16", "scan_with_state", "scan_gated", "scan_cm",
 ]
 
 
@@ -150,3 +150,26 @@ def scan_gated(gate: torch.Tensor, x: torch.Tensor) -> torch.Tensor:
     """The Hawk / RG-LRU style gated recurrence from its pre-activations:
     ``a = sigmoid(gate)``, ``h[t] = a[t]*h[t-1] + sqrt(1 - a[t]**2) * x[t]``."""
     return SequentialScanGated.apply(gate, x)
+
+
+class SequentialScanChannelMajor(Function):
+    """The scan on ``(bs, d_model, seq)`` tensors (time contiguous), bf16, fp16 or fp32.  Not in the
+    reference, whose kernels take ``(bs, seq, d_model)`` only."""
+
+    @staticmethod
+    def forward(ctx: Any, alpha: torch.Tensor, beta: torch.Tensor) -> torch.Tensor:
+        h = _ext.scan_forward_cm(alpha, beta)
+        ctx.save_for_backward(alpha, h)
+        return h
+
+    @staticmethod
+    @once_differentiable
+    def backward(ctx: Any, grad_output: torch.Tensor) -> Tuple[torch.Tensor, torch.Tensor]:
+        alpha, h = ctx.saved_tensors
+        grad_alpha, grad_beta = _ext.scan_backward_cm(alpha, h, grad_output)
+        return grad_alpha, grad_beta
+
+
+def scan_cm(alpha: torch.Tensor, beta: torch.Tensor) -> torch.Tensor:
+    """``h[..., t] = alpha[..., t]*h[..., t-1] + beta[..., t]`` for ``(bs, d_model, seq)`` tensors."""
+    return SequentialScanChannelMajor.apply(alpha, beta)

@@ -26,6 +26,7 @@ __all__ = [
     "scan_forward_fp16", "scan_backward_fp16",
     "scan_forward_state", "scan_backward_state",
     "gated_scan_forward", "gated_scan_backward",
+    "scan_forward_cm", "scan_backward_cm",
 ]
 
 _DTYPE_CODE = {torch.bfloat16: _native.FSS_BF16, torch.float32: _native.FSS_F32, torch.float16: _native.FSS_F16}
@@ -316,3 +317,57 @@ def gated_scan_backward(
             )
         )
     return [grad_gate, grad_x]
+
+
+# ---- channel-major layout: tensors (bs, d_model, seq), time contiguous (what the accelerated-scan
+# package takes; the reference permutes to it in benchmark.py:67-72) ----
+
+
+def scan_forward_cm(alpha: torch.Tensor, beta: torch.Tensor, config=None) -> torch.Tensor:
+    """h for ``(bs, d_model, seq)`` tensors: the same recurrence along the last axis."""
+    dtype = _either_dtype(alpha, "alpha")
+    bs, d, seq = _validate(dtype, alpha=alpha, beta=beta)
+    alpha, beta = alpha.contiguous(), beta.contiguous()
+    out = torch.empty_like(alpha, memory_format=torch.contiguous_format)
+    if out.numel() == 0:
+        return out
+    lib = _native.lib()
+    code = _DTYPE_CODE[dtype]
+    cfg = _native.make_config(config)
+    with torch.cuda.device(alpha.device):
+        stream = torch.cuda.current_stream()
+        ws = _workspace(alpha.device, stream, lib.fss_cm_workspace_bytes(bs, d, seq, code, _native.FSS_FWD, cfg))
+        _native.check(
+            lib.fss_scan_fwd_cm(
+                code, alpha.data_ptr(), beta.data_ptr(), out.data_ptr(), bs, d, seq,
+                ws.data_ptr(), ws.numel(), stream.cuda_stream, cfg,
+            )
+        )
+    return out
+
+
+def scan_backward_cm(
+    alpha_saved: torch.Tensor, h_saved: torch.Tensor, grad_out: torch.Tensor, config=None
+) -> List[torch.Tensor]:
+    """[grad_alpha, grad_beta] for ``(bs, d_model, seq)`` tensors."""
+    dtype = _either_dtype(alpha_saved, "alpha_saved")
+    bs, d, seq = _validate(dtype, alpha_saved=alpha_saved, h_saved=h_saved, grad_out=grad_out)
+    alpha_saved, h_saved, grad_out = alpha_saved.contiguous(), h_saved.contiguous(), grad_out.contiguous()
+    grad_alpha = torch.empty_like(alpha_saved, memory_format=torch.contiguous_format)
+    grad_beta = torch.empty_like(alpha_saved, memory_format=torch.contiguous_format)
+    if grad_alpha.numel() == 0:
+        return [grad_alpha, grad_beta]
+    lib = _native.lib()
+    code = _DTYPE_CODE[dtype]
+    cfg = _native.make_config(config)
+    with torch.cuda.device(alpha_saved.device):
+        stream = torch.cuda.current_stream()
+        ws = _workspace(alpha_saved.device, stream, lib.fss_cm_workspace_bytes(bs, d, seq, code, _native.FSS_BWD, cfg))
+        _native.check(
+            lib.fss_scan_bwd_cm(
+                code, alpha_saved.data_ptr(), h_saved.data_ptr(), grad_out.data_ptr(),
+                grad_alpha.data_ptr(), grad_beta.data_ptr(), bs, d, seq,
+                ws.data_ptr(), ws.numel(), stream.cuda_stream, cfg,
+            )
+        )
+    return [grad_alpha, grad_beta]

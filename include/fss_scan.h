@@ -215,6 +215,28 @@ int fss_gated_scan_bwd(int dtype, const void *gate, const void *x, const void *h
                        int64_t seq, int64_t d, void *workspace, size_t workspace_bytes,
                        void *stream, const fss_config *cfg);
 
+/*
+ * Channel-major layout: tensors are (bs, d, seq) row-major, i.e. every (batch, channel)
+ * pair is a contiguous run of seq timesteps - the layout of the `accelerated-scan`
+ * package the reference benchmarks against after a permute().contiguous() of its own
+ * (bs, seq, d) tensors (benchmark.py:67-72).  Same recurrences and gradients as
+ * fss_scan_fwd_ex / fss_scan_bwd_ex, per run; alpha[..., 0] is never read.  Note the
+ * argument order bs, d, seq.  Of `cfg` only vec (timesteps per lane: 1, 2 or 8 for the
+ * 16-bit types, 1 or 4 for fp32; seq % vec == 0 and tensors aligned to vec elements),
+ * waves and max_groups are used; steps must be 0.  A workgroup of 8 waves covers
+ * 4096 (16-bit) / 2048 (fp32) timesteps, and only longer sequences use the workspace:
+ * size it with fss_cm_workspace_bytes (an upper bound over alignments).
+ */
+size_t fss_cm_workspace_bytes(int64_t bs, int64_t d, int64_t seq, int dtype, int dir,
+                              const fss_config *cfg);
+int fss_scan_fwd_cm(int dtype, const void *alpha, const void *beta, void *h, int64_t bs,
+                    int64_t d, int64_t seq, void *workspace, size_t workspace_bytes,
+                    void *stream, const fss_config *cfg);
+int fss_scan_bwd_cm(int dtype, const void *alpha, const void *h, const void *dout,
+                    void *grad_alpha, void *grad_beta, int64_t bs, int64_t d, int64_t seq,
+                    void *workspace, size_t workspace_bytes, void *stream,
+                    const fss_config *cfg);
+
 /* Plain device-to-device copy kernel of `bytes` bytes (a multiple of 16; both
  * pointers 16-byte aligned).  Exists so that hardware counters read for the
  * scan kernels can be scaled by what the same counters read for a transfer of
