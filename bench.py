@@ -344,12 +344,13 @@ def main() -> int:
     try:
         with open(os.path.join(ROOT, "profiles", "hbm_traffic_bs8_seq4096_d1024.json")) as f:
             prof = json.load(f)
-        if prof["case"] == args.case and args.dtype == "bf16" and args.op == "scan":
-            scale_r = prof["copy"]["bytes_read"] / (prof["copy"]["fetch_kib"] * 1024.0)
-            scale_w = prof["copy"]["bytes_written"] / (prof["copy"]["write_kib"] * 1024.0)
+        if prof["case"] == args.case and args.dtype == "bf16":
+            part = prof if args.op == "scan" else prof[args.op]
+            scale_r = part["copy"]["bytes_read"] / (part["copy"]["fetch_kib"] * 1024.0)
+            scale_w = part["copy"]["bytes_written"] / (part["copy"]["write_kib"] * 1024.0)
             for name in ("fwd", "bwd"):
-                if prof[name]["config"] == chosen[name]:
-                    traffic[name] = int(prof[name]["fetch_kib"] * 1024 * scale_r + prof[name]["write_kib"] * 1024 * scale_w)
+                if part[name]["config"] == chosen[name]:
+                    traffic[name] = int(part[name]["fetch_kib"] * 1024 * scale_r + part[name]["write_kib"] * 1024 * scale_w)
     except (OSError, KeyError, ValueError):
         pass
 
