@@ -55,6 +55,13 @@
 //
 // The backward runs the same machine over reversed time r = seq-1-t with
 // a'[r] = alpha[t+1], b'[r] = dout[t], plus the elementwise g[t]*h[t-1].
+//
+// Variants built on the same machine (none of them in the reference): scans with a
+// state entering and leaving the sequence (STATE), the gated scan that computes
+// alpha = sigmoid(gate) and beta = x*sqrt(1-alpha^2) in phase 1 (GATED, gated_tile),
+// IEEE half next to bf16 and fp32, and the channel-major (bs, d, seq) layout with
+// time across the lanes (cm_tile, cm_scan_kernel), whose rows are chained exactly
+// as the channels are here.
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 #include <string.h>

@@ -157,3 +157,42 @@ def test_missing_library_is_an_error(monkeypatch, tmp_path):
     monkeypatch.setattr(_native, "LIB_PATH", str(tmp_path / "nope.so"))
     with pytest.raises(_native.NativeLibraryMissing):
         _native.lib()
+
+
+def test_planning_of_the_gated_fp16_and_channel_major_entry_points():
+    lib = _native.lib()
+    cfg = _native.FssConfig()
+
+    def choose(dtype, direction, shape=(8, 4096, 1024)):
+        assert lib.fss_choose_config(*shape, dtype, direction, 16, ctypes.byref(cfg)) == 0
+        return cfg.vec, cfg.steps, cfg.waves
+
+    # gated: 4 bytes per lane; the backward holds four tensors, so never more than 16 steps
+    assert choose(_native.FSS_BF16, _native.FSS_GATED_FWD) == (2, 16, 8)
+    assert choose(_native.FSS_BF16, _native.FSS_GATED_BWD) == (2, 16, 8)
+    assert choose(_native.FSS_F32, _native.FSS_GATED_FWD) == (1, 32, 8)
+    assert choose(_native.FSS_F32, _native.FSS_GATED_BWD)[1] <= 16
+    assert choose(_native.FSS_BF16, _native.FSS_GATED_BWD, (1, 65521, 256))[1] <= 16
+    # fp16 plans like bf16
+    for direction in (_native.FSS_FWD, _native.FSS_BWD):
+        assert choose(_native.FSS_F16, direction) == choose(_native.FSS_BF16, direction)
+    assert lib.fss_choose_config(8, 4096, 1024, 3, 0, 16, ctypes.byref(cfg)) == 5
+    assert lib.fss_choose_config(8, 4096, 1024, 0, 4, 16, ctypes.byref(cfg)) == 5
+    # every direction's workspace fits the documented upper bound
+    for shape in [(8, 4096, 1024), (1, 65521, 256), (3, 1, 7)]:
+        top = lib.fss_workspace_bytes_max(*shape)
+        for dtype in (_native.FSS_BF16, _native.FSS_F32, _native.FSS_F16):
+            for direction in range(4):
+                assert lib.fss_workspace_bytes(*shape, dtype, direction, None) <= top
+    # channel-major: one workgroup of 8 waves reaches 512 timesteps even at one timestep per lane
+    assert lib.fss_cm_workspace_bytes(8, 1024, 512, _native.FSS_BF16, _native.FSS_FWD, None) == 4096
+    assert lib.fss_cm_workspace_bytes(8, 1024, 8192, _native.FSS_BF16, _native.FSS_BWD, None) > 4096
+    assert lib.fss_cm_workspace_bytes(-1, 4, 4, _native.FSS_BF16, _native.FSS_FWD, None) == 4096
+    # bad arguments are rejected before any device call
+    one = ctypes.c_void_p(256)
+    assert lib.fss_gated_scan_fwd(0, None, one, one, 1, 8, 8, None, 0, None, None) == 1
+    assert lib.fss_gated_scan_bwd(0, one, None, one, one, one, one, 1, 8, 8, None, 0, None, None) == 1
+    assert lib.fss_scan_fwd_cm(0, one, one, None, 1, 8, 8, None, 0, None, None) == 1
+    assert lib.fss_scan_bwd_cm(0, one, one, one, None, one, 1, 8, 8, None, 0, None, None) == 1
+    assert lib.fss_scan_fwd_cm(0, one, one, one, 1, -8, 8, None, 0, None, None) == 2
+    assert lib.fss_scan_fwd_cm(0, ctypes.c_void_p(257), one, one, 1, 8, 8, None, 0, None, None) == 3
