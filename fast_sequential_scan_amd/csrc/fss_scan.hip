@@ -1,7 +1,7 @@
 // Linear-recurrence scan for MI355X (gfx950, wave64): kernels and the C ABI of
 // include/fss_scan.h.
 //
-//   forward    h[t] = alpha[t]*h[t-1] + beta[t],  h[-1] = 0, alpha[0] never read
+//   forward    h[t] = alpha[t]*h[t-1] + beta[t],  h[-1] = 0, alpha[0] never used
 //   backward   g[t] = alpha[t+1]*g[t+1] + dout[t];  grad_beta = g;  grad_alpha[t] = g[t]*h[t-1]
 //
 // Semantics follow the reference's kernels
@@ -638,7 +638,11 @@ __device__ __forceinline__ void scan_tile(const ScanArgs &p, const StateArgs<STA
 #pragma unroll
   for (int s = 0; s < STEPS; ++s) {
     if (FULL) {
-      a[s].template load<kNtA>(uniform_ptr(pa + s * step_bytes) + lane_off);
+      // The scan's very first step (r = 0) has no predecessor: its coefficient is replaced
+      // below, whatever is loaded here.  The backward would find it one row past the end
+      // of the sequence, so it loads the row before instead.
+      const int row = (BWD && s == 0 && r0 == 0) ? 1 : s;
+      a[s].template load<kNtA>(uniform_ptr(pa + row * step_bytes) + lane_off);
       b[s].template load<kNtB>(uniform_ptr(pb + s * step_bytes) + lane_off);
     } else {
       const int64_t r = r0 + s;
@@ -653,6 +657,15 @@ __device__ __forceinline__ void scan_tile(const ScanArgs &p, const StateArgs<STA
         b[s].template load<kNtB>(uniform_ptr(pb + s * step_bytes) + lane_off);
       }
     }
+  }
+
+  if (FULL && r0 == 0) {
+    // no predecessor: coefficient 0 - or, with a state coming in, alpha[0] as loaded
+    // (forward) resp. 1, since the incoming gradient is added (backward)
+    if (BWD)
+      a[0].fill((STATE && st.state_in) ? 1.0f : 0.0f);
+    else if (!(STATE && st.state_in))
+      a[0].fill(0.0f);
   }
 
   // The backward's third stream, h[t-1], only feeds phase 3.  Its first kHEarly rows go
@@ -1017,10 +1030,9 @@ __global__ __launch_bounds__(1024) void scan_kernel(const ScanArgs p, const Stat
     c.chan_row = static_cast<int64_t>(batch) * p.d + col0;
     c.r0 = (static_cast<int64_t>(chunk) * c.n_waves + c.wave) * STEPS;
 
-    // Forward touches rows r0..r0+STEPS-1 and must not be at r = 0 (alpha[0] is never
-    // read); the backward additionally reads row t+1 and row t-1.
-    // (the gated forward does read row 0 of its first input)
-    const bool full = (col0 + kLaneSlots <= p.d) && (c.r0 >= ((GATED && !BWD) ? 0 : 1)) &&
+    // Forward touches rows r0..r0+STEPS-1; the backward additionally reads row t+1 (the
+    // unpredicated variant handles r = 0 itself, except in the gated backward) and row t-1.
+    const bool full = (col0 + kLaneSlots <= p.d) && (c.r0 >= ((GATED && BWD) ? 1 : 0)) &&
                       (BWD ? (c.r0 + STEPS <= c.seq - 1) : (c.r0 + STEPS <= c.seq));
     // wave-uniform, but waves of one workgroup may differ: both variants execute the
     // same barriers, so they meet

@@ -8,7 +8,8 @@
  *   backward   g[seq-1] = dout[seq-1];  g[t] = alpha[t+1]*g[t+1] + dout[t]
  *              grad_beta[t] = g[t];  grad_alpha[t] = g[t]*h[t-1] (t >= 1);  grad_alpha[0] = 0
  *
- * with fp32 carries in both directions.  alpha[:,0,:] is never read.
+ * with fp32 carries in both directions.  The values in alpha[:,0,:] are never used
+ * (they may be NaN).
  *
  * This header replaces, for a host written in any language, the pybind11 module
  * `sequential_scan_cuda` of the reference (csrc/sequential_scan.cpp:13-22) and
@@ -220,7 +221,7 @@ int fss_gated_scan_bwd(int dtype, const void *gate, const void *x, const void *h
  * pair is a contiguous run of seq timesteps - the layout of the `accelerated-scan`
  * package the reference benchmarks against after a permute().contiguous() of its own
  * (bs, seq, d) tensors (benchmark.py:67-72).  Same recurrences and gradients as
- * fss_scan_fwd_ex / fss_scan_bwd_ex, per run; alpha[..., 0] is never read.  Note the
+ * fss_scan_fwd_ex / fss_scan_bwd_ex, per run; the values in alpha[..., 0] are never used.  Note the
  * argument order bs, d, seq.  Of `cfg` only vec (timesteps per lane: 1, 2 or 8 for the
  * 16-bit types, 1 or 4 for fp32; seq % vec == 0 and tensors aligned to vec elements),
  * waves and max_groups are used; steps must be 0.  A workgroup of 8 waves covers
