@@ -196,3 +196,18 @@ def test_planning_of_the_gated_fp16_and_channel_major_entry_points():
     assert lib.fss_scan_bwd_cm(0, one, one, one, None, one, 1, 8, 8, None, 0, None, None) == 1
     assert lib.fss_scan_fwd_cm(0, one, one, one, 1, -8, 8, None, 0, None, None) == 2
     assert lib.fss_scan_fwd_cm(0, ctypes.c_void_p(257), one, one, 1, 8, 8, None, 0, None, None) == 3
+
+
+def test_shipped_package_never_touches_the_oracle():
+    """The oracle is test infrastructure: nothing under the package (or the drop-in shim) may
+    import it, name its directory, or fall back to a CPU computation of the scan."""
+    offenders = []
+    for top in ("fast_sequential_scan_amd", "sequential_scan"):
+        for base, _dirs, files in os.walk(os.path.join(ROOT, top)):
+            for name in files:
+                if not name.endswith((".py", ".hip", ".h")):
+                    continue
+                text = open(os.path.join(base, name)).read()
+                if re.search(r"^\s*(from|import)\s+oracle\b", text, flags=re.M) or "oracle/" in text:
+                    offenders.append(os.path.join(base, name))
+    assert not offenders, offenders
