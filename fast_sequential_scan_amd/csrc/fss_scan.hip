@@ -901,6 +901,10 @@ __device__ __forceinline__ void gated_tile(const ScanArgs &p, const TileCtx &c) 
         }
         b[s].pack(be);  // rows outside the sequence hold x = 0, so beta = 0 there
       }
+      // one step at a time: left to itself the compiler interleaves the gating of many steps
+      // (for the latency of exp2/rcp/sqrt) and runs out of registers at 32 steps per lane
+      keep_packed(a[s]);
+      keep_packed(b[s]);
       const bool ident = !FULL && BWD && r >= seq;  // backward: a[s] with r == seq is alpha[0], not a coefficient
 #pragma unroll
       for (int v = 0; v < VEC; ++v) {
@@ -1351,8 +1355,6 @@ void complete_config(fss_config &c, int64_t bs, int64_t seq, int64_t d, int dtyp
     // traffic); that only pays where the chain of chunks is long.  Elsewhere 16 steps are
     // as fast in bf16 and 6 % faster in fp32 (forward and backward alternating).
     if (dir == FSS_BWD && s == 32 && (gated || ceil_div(seq, static_cast<int64_t>(8) * 32) <= 16)) s = 16;
-    // gated forward in bf16: 32 steps spill (the gating needs temporaries), 16 measured faster
-    if (gated && dir == FSS_FWD && dtype != FSS_F32 && s == 32) s = 16;
     // small problems: shorter slices until there are two 8-wave tiles per CU (512), as
     // long as the machine still gets a few waves per SIMD out of it
     const int64_t ctiles = bs * ceil_div(d, 64 * c.vec);

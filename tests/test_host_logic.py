@@ -168,7 +168,7 @@ def test_planning_of_the_gated_fp16_and_channel_major_entry_points():
         return cfg.vec, cfg.steps, cfg.waves
 
     # gated: 4 bytes per lane; the backward holds four tensors, so never more than 16 steps
-    assert choose(_native.FSS_BF16, _native.FSS_GATED_FWD) == (2, 16, 8)
+    assert choose(_native.FSS_BF16, _native.FSS_GATED_FWD) == (2, 32, 8)
     assert choose(_native.FSS_BF16, _native.FSS_GATED_BWD) == (2, 16, 8)
     assert choose(_native.FSS_F32, _native.FSS_GATED_FWD) == (1, 32, 8)
     assert choose(_native.FSS_F32, _native.FSS_GATED_BWD)[1] <= 16
