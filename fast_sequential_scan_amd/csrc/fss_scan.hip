@@ -67,6 +67,7 @@
 #include <string.h>
 
 #include <initializer_list>
+#include <mutex>
 
 #include "../../include/fss_scan.h"
 
@@ -1442,6 +1443,63 @@ int check_device() {
   return state == 1 ? FSS_OK : FSS_ERR_UNSUPPORTED_DEVICE;
 }
 
+// Scans of one process never overlap on a device.  A scan's workgroups wait for each
+// other and its grid is sized to fill the device, so two scans sharing the device
+// could each hold the compute units the other's unscheduled workgroups need, and
+// both would sit there until their waits give up.  Launches on one stream are
+// ordered anyway; when the stream changes, the new launch is made to wait for
+// everything queued on the previous stream.  The lock is held across the launch, so
+// that the event recorded by the next caller lands behind this one's kernel.
+// Streams under graph capture are left alone (a captured scan is ordered by its
+// graph; do not replay two graphs holding scans concurrently).
+struct ScanOrder {
+  std::mutex lock;
+  hipStream_t last = nullptr;
+  bool any = false;
+  hipEvent_t event = nullptr;
+};
+ScanOrder g_scan_order[64];
+
+inline bool stream_is_capturing(hipStream_t s) {
+  hipStreamCaptureStatus status = hipStreamCaptureStatusNone;
+  if (hipStreamIsCapturing(s, &status) != hipSuccess) {
+    (void)hipGetLastError();
+    return true;  // unknown: do not touch it
+  }
+  return status != hipStreamCaptureStatusNone;
+}
+
+class ScanOrderGuard {
+ public:
+  explicit ScanOrderGuard(hipStream_t s) {
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return;
+    order_ = &g_scan_order[dev];
+    order_->lock.lock();
+    if (stream_is_capturing(s)) return;
+    if (order_->any && order_->last != s && !stream_is_capturing(order_->last)) {
+      if (!order_->event && hipEventCreateWithFlags(&order_->event, hipEventDisableTiming) != hipSuccess) {
+        order_->event = nullptr;
+        (void)hipGetLastError();
+      }
+      // a stream the caller has destroyed since makes the record fail: nothing to wait for then
+      if (order_->event && hipEventRecord(order_->event, order_->last) == hipSuccess)
+        (void)hipStreamWaitEvent(s, order_->event, 0);
+      (void)hipGetLastError();
+    }
+    order_->last = s;
+    order_->any = true;
+  }
+  ~ScanOrderGuard() {
+    if (order_) order_->lock.unlock();
+  }
+  ScanOrderGuard(const ScanOrderGuard &) = delete;
+  ScanOrderGuard &operator=(const ScanOrderGuard &) = delete;
+
+ private:
+  ScanOrder *order_ = nullptr;
+};
+
 // Workgroups of `kernel` that are certainly resident together on the device (0 on
 // error).  Deliberately not the runtime's occupancy query: the kernel's waits
 // need a lower bound, and that query bounds by vector registers and LDS only.
@@ -1625,6 +1683,7 @@ int run_scan(int dtype, int dir, const void *alpha, const void *in_b, const void
   hipStream_t s = static_cast<hipStream_t>(stream);
   const bool st = state_in || state_out || h_before;
   const bool bwd = dir == FSS_BWD;
+  const ScanOrderGuard ordered(s);
 #define FSS_DISPATCH(E)                                                                        \
   do {                                                                                         \
     if (gated) return bwd ? launch_gated<E, true>(args, pl, s) : launch_gated<E, false>(args, pl, s); \
@@ -1768,6 +1827,7 @@ int run_cm_scan(int dtype, int dir, const void *alpha, const void *in_b, const v
   hipStream_t s = static_cast<hipStream_t>(stream);
   const int max_groups = cfg ? cfg->max_groups : 0;
   const bool bwd = dir == FSS_BWD;
+  const ScanOrderGuard ordered(s);
   if (dtype == FSS_BF16) return bwd ? launch_cm<BF16, true>(args, pl, max_groups, s) : launch_cm<BF16, false>(args, pl, max_groups, s);
   if (dtype == FSS_F16) return bwd ? launch_cm<F16, true>(args, pl, max_groups, s) : launch_cm<F16, false>(args, pl, max_groups, s);
   return bwd ? launch_cm<F32, true>(args, pl, max_groups, s) : launch_cm<F32, false>(args, pl, max_groups, s);

@@ -22,6 +22,13 @@
  *     workspace are the caller's.
  *   - Calls are asynchronous on `stream` (a hipStream_t passed as void*; NULL is
  *     the null stream).  No entry point synchronises except fss_workspace_status.
+ *   - Scans launched by one process on different streams of a device do not overlap:
+ *     a scan fills the device with workgroups that wait for each other, so the library
+ *     makes a launch on a new stream wait (hipStreamWaitEvent) for the work queued on
+ *     the stream of the previous scan.  Streams under graph capture are exempt: do not
+ *     replay two graphs containing scans concurrently, and do not share the device
+ *     between processes that scan at the same time - co-scheduled scans can stall each
+ *     other until their bounded waits give up (FSS_ERR_CHAIN_TIMEOUT).
  *   - Every entry point returns an fss_status (0 = ok); nothing throws.
  *   - Any seq >= 1 and any d >= 1 are accepted (the reference needs seq >= 2/3 and
  *     d in {512,768,1024,1536,2048}: csrc/sequential_scan_kernel.cu:136-184).

@@ -425,3 +425,33 @@ def test_tensors_larger_than_4_GiB():
     ext.workspace_status()
     del alpha, beta, h, ga, gb
     torch.cuda.empty_cache()
+
+
+def test_scans_on_two_streams_do_not_overlap(oracle):
+    """A scan fills the device with workgroups that wait for each other; the library chains launches
+    that arrive on different streams, so interleaved launches stay correct and never time out."""
+    shape = (8, 2048, 1024)
+    sets = []
+    for seed in (41, 42):
+        alpha, beta, dout = make_inputs("sigmoid", *shape, seed=seed)
+        sets.append(tuple(t.to(DEV) for t in (alpha, beta, dout)))
+    want = []
+    for a, b, do in sets:
+        h = ext.scan_forward_half(a, b)
+        want.append((h, *ext.scan_backward_half(a, h, do)))
+    torch.cuda.synchronize()
+    streams = [torch.cuda.Stream(), torch.cuda.Stream()]
+    got = [None, None]
+    for _ in range(8):  # no host synchronisation between the launches
+        for i, s in enumerate(streams):
+            with torch.cuda.stream(s):
+                a, b, do = sets[i]
+                h = ext.scan_forward_half(a, b)
+                got[i] = (h, *ext.scan_backward_half(a, h, do))
+    for i, s in enumerate(streams):
+        with torch.cuda.stream(s):
+            ext.workspace_status()  # synchronises the stream; raises on a chain time-out
+    torch.cuda.synchronize()
+    for i in range(2):
+        for g, w in zip(got[i], want[i]):
+            assert torch.equal(g, w)
