@@ -5,6 +5,11 @@
 hipcc cross-compiles without a GPU, so this runs anywhere ROCm is installed.
 The result, ``fast_sequential_scan_amd/_lib/libfss_scan.so``, is a plain C-ABI
 shared library (include/fss_scan.h): no torch headers, no pybind.
+
+Translation units (compiled in parallel, then linked):
+  csrc/fss_api.hip       the C ABI, planning, small kernels
+  csrc/fss_scan_rm.hip   the row-major scan kernels, once per storage type
+  csrc/fss_scan_cm.hip   the channel-major scan kernels
 """
 from __future__ import annotations
 
@@ -12,10 +17,12 @@ import os
 import shutil
 import subprocess
 import sys
-from typing import List
+import tempfile
+from concurrent.futures import ThreadPoolExecutor
+from typing import List, Sequence, Tuple
 
 PKG_DIR = os.path.dirname(os.path.abspath(__file__))
-SRC = os.path.join(PKG_DIR, "csrc", "fss_scan.hip")
+SRC_DIR = os.path.join(PKG_DIR, "csrc")
 LIB_DIR = os.path.join(PKG_DIR, "_lib")
 LIB_PATH = os.path.join(LIB_DIR, "libfss_scan.so")
 
@@ -25,10 +32,18 @@ HIPCC_FLAGS: List[str] = [
     "--offload-arch=gfx950",
     "-O3",
     "-std=c++17",
-    "-shared",
     "-fPIC",
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
 ]
+
+# (object name, source, extra defines)
+UNITS: Sequence[Tuple[str, str, Tuple[str, ...]]] = (
+    ("api", "fss_api.hip", ()),
+    ("rm_bf16", "fss_scan_rm.hip", ("-DFSS_RM_ELEM=BF16", "-DFSS_RM_LAUNCH=launch_rm_bf16")),
+    ("rm_f16", "fss_scan_rm.hip", ("-DFSS_RM_ELEM=F16", "-DFSS_RM_LAUNCH=launch_rm_f16")),
+    ("rm_f32", "fss_scan_rm.hip", ("-DFSS_RM_ELEM=F32", "-DFSS_RM_LAUNCH=launch_rm_f32")),
+    ("cm", "fss_scan_cm.hip", ()),
+)
 
 
 def hipcc_path() -> str:
@@ -38,18 +53,33 @@ def hipcc_path() -> str:
     raise FileNotFoundError("hipcc not found (set HIPCC or install ROCm)")
 
 
-def build(verbose: bool = False, extra_flags: List[str] = ()) -> str:
-    os.makedirs(LIB_DIR, exist_ok=True)
-    tmp = LIB_PATH + ".tmp"
-    cmd = [hipcc_path(), *HIPCC_FLAGS, *extra_flags, "-o", tmp, SRC]
+def _run(cmd: List[str], verbose: bool) -> None:
     if verbose:
         print(" ".join(cmd), flush=True)
     proc = subprocess.run(cmd, capture_output=True, text=True)
     if proc.returncode != 0:
         sys.stderr.write(proc.stdout + proc.stderr)
-        raise RuntimeError(f"hipcc failed with exit code {proc.returncode}")
-    os.replace(tmp, LIB_PATH)
-    return LIB_PATH
+        raise RuntimeError(f"hipcc failed with exit code {proc.returncode}: {' '.join(cmd)}")
+    if verbose and proc.stderr and "-Rpass" in " ".join(cmd):
+        sys.stderr.write(proc.stderr)
+
+
+def build(verbose: bool = False, extra_flags: Sequence[str] = (), output: str = LIB_PATH) -> str:
+    """Compiles every translation unit (always: nothing is cached) and links `output`."""
+    os.makedirs(os.path.dirname(output), exist_ok=True)
+    hipcc = hipcc_path()
+    with tempfile.TemporaryDirectory(prefix="fss_build_") as tmp:
+        objects = [os.path.join(tmp, name + ".o") for name, _src, _defs in UNITS]
+        commands = [
+            [hipcc, *HIPCC_FLAGS, *extra_flags, *defs, "-c", os.path.join(SRC_DIR, src), "-o", obj]
+            for (name, src, defs), obj in zip(UNITS, objects)
+        ]
+        with ThreadPoolExecutor(max_workers=min(len(commands), os.cpu_count() or 1, 8)) as pool:
+            list(pool.map(lambda c: _run(c, verbose), commands))
+        linked = output + ".tmp"
+        _run([hipcc, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", linked, *objects], verbose)
+        os.replace(linked, output)
+    return output
 
 
 if __name__ == "__main__":

@@ -1,0 +1,290 @@
+// The C ABI of include/fss_scan.h: argument checking, planning, and the hand-off to the
+// kernels' translation units (fss_scan_rm.hip per storage type, fss_scan_cm.hip).
+#include "fss_device.h"
+#include "fss_host.h"
+
+namespace fss {
+
+thread_local int tls_hip_error = 0;
+#ifdef FSS_TRACE
+uint64_t *g_trace = nullptr;
+#endif
+ScanOrder g_scan_order[64];
+
+// Zero everywhere (tag 0 = "never written"), launch counter starting at 1.
+__global__ void workspace_init_kernel(uint32_t *p, size_t n_words) {
+  const size_t stride = static_cast<size_t>(gridDim.x) * blockDim.x;
+  for (size_t i = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x; i < n_words; i += stride)
+    p[i] = (i == HDR_EPOCH) ? 1u : 0u;
+}
+
+__global__ void copy_kernel(const u32x4 *__restrict__ src, u32x4 *__restrict__ dst, size_t n_vec) {
+  const size_t stride = static_cast<size_t>(gridDim.x) * blockDim.x;
+  for (size_t i = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x; i < n_vec; i += stride)
+    dst[i] = src[i];
+}
+
+int run_scan(int dtype, int dir, const void *alpha, const void *in_b, const void *in_h, void *out0,
+             void *out1, int64_t bs, int64_t seq, int64_t d, void *workspace, size_t workspace_bytes,
+             void *stream, const fss_config *cfg, const float *state_in = nullptr,
+             float *state_out = nullptr, const float *h_before = nullptr, const void *in_x = nullptr) {
+  const bool gated = dir >= FSS_GATED_FWD;
+  const int plan_dir = dir;
+  dir &= 1;
+  if (bs < 0 || seq < 0 || d < 0) return FSS_ERR_BAD_SHAPE;
+  if (dtype != FSS_BF16 && dtype != FSS_F32 && dtype != FSS_F16) return FSS_ERR_BAD_CONFIG;
+  if (bs == 0 || seq == 0 || d == 0) return FSS_OK;
+  if (!alpha || !in_b || !out0) return FSS_ERR_NULL_POINTER;
+  if (dir == FSS_BWD && (!in_h || !out1)) return FSS_ERR_NULL_POINTER;
+  if (gated && dir == FSS_BWD && !in_x) return FSS_ERR_NULL_POINTER;
+  const size_t esize = dtype != FSS_F32 ? 2 : 4;
+  const size_t align = dir == FSS_BWD ? common_alignment({alpha, in_b, in_h, out0, out1, in_x})
+                                      : common_alignment({alpha, in_b, out0});
+  if (align < esize) return FSS_ERR_MISALIGNED;
+  if ((reinterpret_cast<uintptr_t>(state_in) | reinterpret_cast<uintptr_t>(state_out) |
+       reinterpret_cast<uintptr_t>(h_before)) % 4 != 0)
+    return FSS_ERR_MISALIGNED;
+  Plan pl;
+  int rc = make_plan(pl, bs, seq, d, dtype, plan_dir, align, cfg);
+  if (rc != FSS_OK) return rc;
+  if (pl.n_chunks > 1) {
+    if (!workspace || workspace_bytes < pl.ws_bytes) return FSS_ERR_WORKSPACE_SMALL;
+    if (reinterpret_cast<uintptr_t>(workspace) % 256 != 0) return FSS_ERR_MISALIGNED;
+  }
+  rc = check_device();
+  if (rc != FSS_OK) return rc;
+
+  ScanArgs args;
+  args.in_a = static_cast<const char *>(alpha);
+  args.in_b = static_cast<const char *>(in_b);
+  args.in_h = static_cast<const char *>(in_h);
+  args.out0 = static_cast<char *>(out0);
+  args.out1 = static_cast<char *>(out1);
+  args.in_x = static_cast<const char *>(in_x);
+  args.seq = seq;
+  args.d = d;
+  args.tiles_per_row = static_cast<int32_t>(pl.tiles_per_row);
+  args.n_ctiles = static_cast<int32_t>(pl.n_ctiles);
+  args.n_chunks = static_cast<int32_t>(pl.n_chunks);
+  args.n_tiles = static_cast<int32_t>(pl.n_tiles);
+  args.look_waves = look_waves(pl.cfg.waves, pl.cfg.vec);
+  const StateArgs<true> state = {state_in, state_out, h_before};
+  args.hdr = static_cast<uint32_t *>(workspace);
+  args.words = workspace ? reinterpret_cast<uint64_t *>(static_cast<char *>(workspace) + kHeaderBytes) : nullptr;
+#ifdef FSS_TRACE
+  args.trace = g_trace;
+#endif
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  const bool st = state_in || state_out || h_before;
+  const bool bwd = dir == FSS_BWD;
+  const ScanOrderGuard ordered(s);
+  if (dtype == FSS_BF16) return launch_rm_bf16(args, state, pl, bwd, gated, st, s);
+  if (dtype == FSS_F16) return launch_rm_f16(args, state, pl, bwd, gated, st, s);
+  return launch_rm_f32(args, state, pl, bwd, gated, st, s);
+}
+
+}  // namespace fss
+
+// ---- C ABI -------------------------------------------------------------------------
+
+extern "C" {
+
+#ifdef FSS_TRACE
+void fss_debug_set_trace(void *p) { fss::g_trace = static_cast<uint64_t *>(p); }
+#endif
+
+int fss_abi_version(void) { return FSS_ABI_VERSION; }
+
+const char *fss_strerror(int status) {
+  switch (status) {
+    case FSS_OK: return "ok";
+    case FSS_ERR_NULL_POINTER: return "a required pointer is NULL";
+    case FSS_ERR_BAD_SHAPE: return "bs, seq or d is negative or too large";
+    case FSS_ERR_MISALIGNED: return "a tensor (or the workspace) is not sufficiently aligned";
+    case FSS_ERR_WORKSPACE_SMALL: return "workspace missing or smaller than fss_workspace_bytes";
+    case FSS_ERR_BAD_CONFIG: return "unsupported dtype, direction or launch configuration";
+    case FSS_ERR_LAUNCH: return "HIP reported an error (see fss_last_hip_error)";
+    case FSS_ERR_CHAIN_TIMEOUT: return "a chunk gave up waiting for the state of its predecessor";
+    case FSS_ERR_UNSUPPORTED_DEVICE: return "the current device is not gfx950";
+    default: return "unknown status";
+  }
+}
+
+int fss_last_hip_error(void) { return fss::tls_hip_error; }
+
+size_t fss_workspace_bytes(int64_t bs, int64_t seq, int64_t d, int dtype, int dir, const fss_config *cfg) {
+  fss::Plan pl;
+  // alignment unknown here: assume the best the shape allows (the widest vector,
+  // hence the most words per tile, is what a less aligned call can only shrink)
+  if (fss::make_plan(pl, bs, seq, d, dtype, dir, 16, cfg) != FSS_OK) return fss::kHeaderBytes;
+  return pl.ws_bytes;
+}
+
+size_t fss_workspace_bytes_max(int64_t bs, int64_t seq, int64_t d) {
+  size_t best = fss::kHeaderBytes;
+  for (int dtype = FSS_BF16; dtype <= FSS_F16; ++dtype)
+    for (int dir = FSS_FWD; dir <= FSS_GATED_BWD; ++dir)
+      for (size_t align = 2; align <= 16; align <<= 1) {
+        fss::Plan pl;
+        if (fss::make_plan(pl, bs, seq, d, dtype, dir, align, nullptr) == FSS_OK && pl.ws_bytes > best)
+          best = pl.ws_bytes;
+      }
+  return best;
+}
+
+int fss_choose_config(int64_t bs, int64_t seq, int64_t d, int dtype, int dir, size_t align_bytes,
+                      fss_config *out) {
+  if (!out) return FSS_ERR_NULL_POINTER;
+  fss::Plan pl;
+  const int rc = fss::make_plan(pl, bs, seq, d, dtype, dir, align_bytes ? align_bytes : 16, nullptr);
+  if (rc == FSS_OK) *out = pl.cfg;
+  return rc;
+}
+
+int fss_workspace_init(void *workspace, size_t bytes, void *stream) {
+  if (!workspace) return FSS_ERR_NULL_POINTER;
+  if (bytes < fss::kHeaderBytes) return FSS_ERR_WORKSPACE_SMALL;
+  if (reinterpret_cast<uintptr_t>(workspace) % 256 != 0 || bytes % 4 != 0) return FSS_ERR_MISALIGNED;
+  const size_t n_words = bytes / 4;
+  size_t blocks = (n_words + 255) / 256;
+  if (blocks > 4096) blocks = 4096;
+  hipLaunchKernelGGL(fss::workspace_init_kernel, dim3(static_cast<uint32_t>(blocks)), dim3(256), 0,
+                     static_cast<hipStream_t>(stream), static_cast<uint32_t *>(workspace), n_words);
+  const hipError_t e = hipGetLastError();
+  if (e != hipSuccess) {
+    fss::tls_hip_error = static_cast<int>(e);
+    return FSS_ERR_LAUNCH;
+  }
+  return FSS_OK;
+}
+
+int fss_workspace_status(void *workspace, void *stream) {
+  if (!workspace) return FSS_ERR_NULL_POINTER;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  uint32_t hdr[4] = {0, 0, 0, 0};
+  hipError_t e = hipMemcpyAsync(hdr, workspace, sizeof(hdr), hipMemcpyDeviceToHost, s);
+  if (e == hipSuccess) e = hipStreamSynchronize(s);
+  if (e != hipSuccess) {
+    fss::tls_hip_error = static_cast<int>(e);
+    return FSS_ERR_LAUNCH;
+  }
+  if (hdr[fss::HDR_ERROR] != 0) {
+    const uint32_t zero = 0;
+    e = hipMemcpyAsync(static_cast<uint32_t *>(workspace) + fss::HDR_ERROR, &zero, 4, hipMemcpyHostToDevice, s);
+    if (e == hipSuccess) e = hipStreamSynchronize(s);
+    return FSS_ERR_CHAIN_TIMEOUT;
+  }
+  return FSS_OK;
+}
+
+int fss_scan_fwd_ex(int dtype, const void *alpha, const void *beta, void *h, int64_t bs, int64_t seq,
+                    int64_t d, void *workspace, size_t workspace_bytes, void *stream,
+                    const fss_config *cfg) {
+  return fss::run_scan(dtype, FSS_FWD, alpha, beta, nullptr, h, nullptr, bs, seq, d, workspace,
+                       workspace_bytes, stream, cfg);
+}
+
+int fss_scan_bwd_ex(int dtype, const void *alpha, const void *h, const void *dout, void *grad_alpha,
+                    void *grad_beta, int64_t bs, int64_t seq, int64_t d, void *workspace,
+                    size_t workspace_bytes, void *stream, const fss_config *cfg) {
+  return fss::run_scan(dtype, FSS_BWD, alpha, dout, h, grad_beta, grad_alpha, bs, seq, d, workspace,
+                       workspace_bytes, stream, cfg);
+}
+
+int fss_scan_fwd_state(int dtype, const void *alpha, const void *beta, void *h, const float *h_before,
+                       float *h_last, int64_t bs, int64_t seq, int64_t d, void *workspace,
+                       size_t workspace_bytes, void *stream, const fss_config *cfg) {
+  return fss::run_scan(dtype, FSS_FWD, alpha, beta, nullptr, h, nullptr, bs, seq, d, workspace,
+                       workspace_bytes, stream, cfg, h_before, h_last, nullptr);
+}
+
+int fss_scan_bwd_state(int dtype, const void *alpha, const void *h, const void *dout, const float *h_before,
+                       const float *grad_h_last, void *grad_alpha, void *grad_beta, float *grad_h_before,
+                       int64_t bs, int64_t seq, int64_t d, void *workspace, size_t workspace_bytes,
+                       void *stream, const fss_config *cfg) {
+  if (grad_h_before && !h_before) return FSS_ERR_NULL_POINTER;
+  return fss::run_scan(dtype, FSS_BWD, alpha, dout, h, grad_beta, grad_alpha, bs, seq, d, workspace,
+                       workspace_bytes, stream, cfg, grad_h_last, grad_h_before, h_before);
+}
+
+int fss_gated_scan_fwd(int dtype, const void *gate, const void *x, void *h, int64_t bs, int64_t seq,
+                       int64_t d, void *workspace, size_t workspace_bytes, void *stream,
+                       const fss_config *cfg) {
+  return fss::run_scan(dtype, FSS_GATED_FWD, gate, x, nullptr, h, nullptr, bs, seq, d, workspace,
+                       workspace_bytes, stream, cfg);
+}
+
+int fss_gated_scan_bwd(int dtype, const void *gate, const void *x, const void *h, const void *dout,
+                       void *grad_gate, void *grad_x, int64_t bs, int64_t seq, int64_t d,
+                       void *workspace, size_t workspace_bytes, void *stream, const fss_config *cfg) {
+  return fss::run_scan(dtype, FSS_GATED_BWD, gate, dout, h, grad_x, grad_gate, bs, seq, d, workspace,
+                       workspace_bytes, stream, cfg, nullptr, nullptr, nullptr, x);
+}
+
+int fss_scan_fwd_bf16(const void *alpha, const void *beta, void *h, int64_t bs, int64_t seq, int64_t d,
+                      void *workspace, size_t workspace_bytes, void *stream) {
+  return fss_scan_fwd_ex(FSS_BF16, alpha, beta, h, bs, seq, d, workspace, workspace_bytes, stream, nullptr);
+}
+
+int fss_scan_bwd_bf16(const void *alpha, const void *h, const void *dout, void *grad_alpha,
+                      void *grad_beta, int64_t bs, int64_t seq, int64_t d, void *workspace,
+                      size_t workspace_bytes, void *stream) {
+  return fss_scan_bwd_ex(FSS_BF16, alpha, h, dout, grad_alpha, grad_beta, bs, seq, d, workspace,
+                         workspace_bytes, stream, nullptr);
+}
+
+int fss_scan_fwd_f32(const void *alpha, const void *beta, void *h, int64_t bs, int64_t seq, int64_t d,
+                     void *workspace, size_t workspace_bytes, void *stream) {
+  return fss_scan_fwd_ex(FSS_F32, alpha, beta, h, bs, seq, d, workspace, workspace_bytes, stream, nullptr);
+}
+
+int fss_scan_bwd_f32(const void *alpha, const void *h, const void *dout, void *grad_alpha,
+                     void *grad_beta, int64_t bs, int64_t seq, int64_t d, void *workspace,
+                     size_t workspace_bytes, void *stream) {
+  return fss_scan_bwd_ex(FSS_F32, alpha, h, dout, grad_alpha, grad_beta, bs, seq, d, workspace,
+                         workspace_bytes, stream, nullptr);
+}
+
+size_t fss_cm_workspace_bytes(int64_t bs, int64_t d, int64_t seq, int dtype, int dir, const fss_config *cfg) {
+  fss::CmPlan pl;
+  if (bs < 0 || d < 0 || (d > 0 && bs > INT64_MAX / d)) return fss::kHeaderBytes;
+  // alignment unknown here: the narrowest vector gives the most chunks, hence the upper bound
+  size_t best = fss::kHeaderBytes;
+  for (size_t align = 2; align <= 16; align <<= 1)
+    if (fss::make_cm_plan(pl, bs * d, seq, dtype, dir, align, cfg) == FSS_OK && pl.ws_bytes > best) best = pl.ws_bytes;
+  return best;
+}
+
+int fss_scan_fwd_cm(int dtype, const void *alpha, const void *beta, void *h, int64_t bs, int64_t d, int64_t seq,
+                    void *workspace, size_t workspace_bytes, void *stream, const fss_config *cfg) {
+  return fss::run_cm_scan(dtype, FSS_FWD, alpha, beta, nullptr, h, nullptr, bs, d, seq, workspace, workspace_bytes,
+                          stream, cfg);
+}
+
+int fss_scan_bwd_cm(int dtype, const void *alpha, const void *h, const void *dout, void *grad_alpha,
+                    void *grad_beta, int64_t bs, int64_t d, int64_t seq, void *workspace, size_t workspace_bytes,
+                    void *stream, const fss_config *cfg) {
+  return fss::run_cm_scan(dtype, FSS_BWD, alpha, dout, h, grad_beta, grad_alpha, bs, d, seq, workspace,
+                          workspace_bytes, stream, cfg);
+}
+
+int fss_copy_bytes(const void *src, void *dst, size_t bytes, void *stream) {
+  if (!src || !dst) return FSS_ERR_NULL_POINTER;
+  if (bytes % 16 != 0 || reinterpret_cast<uintptr_t>(src) % 16 != 0 || reinterpret_cast<uintptr_t>(dst) % 16 != 0)
+    return FSS_ERR_MISALIGNED;
+  if (bytes == 0) return FSS_OK;
+  const size_t n_vec = bytes / 16;
+  size_t blocks = (n_vec + 255) / 256;
+  if (blocks > 8192) blocks = 8192;
+  hipLaunchKernelGGL(fss::copy_kernel, dim3(static_cast<uint32_t>(blocks)), dim3(256), 0,
+                     static_cast<hipStream_t>(stream), static_cast<const fss::u32x4 *>(src),
+                     static_cast<fss::u32x4 *>(dst), n_vec);
+  const hipError_t e = hipGetLastError();
+  if (e != hipSuccess) {
+    fss::tls_hip_error = static_cast<int>(e);
+    return FSS_ERR_LAUNCH;
+  }
+  return FSS_OK;
+}
+
+}  // extern "C"

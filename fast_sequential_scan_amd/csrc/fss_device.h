@@ -1,0 +1,578 @@
+// Device-side building blocks shared by the scan kernels: packed rows, the workspace
+// words, and the chain phase that carries state from chunk to chunk.  See the
+// comment at the top of fss_scan_rm.hip for how the kernels use them.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "../../include/fss_scan.h"
+
+#if defined(FSS_TRACE) && !defined(FSS_TRACE_WAVE)
+#define FSS_TRACE_WAVE 0
+#endif
+
+namespace fss {
+
+// Device pointers are kept in the global address space explicitly: the generic
+// ("flat") form costs a 64-bit vector address per access and a slower instruction.
+#define FSS_GLOBAL __attribute__((address_space(1)))
+typedef const FSS_GLOBAL char *gcptr_t;
+typedef FSS_GLOBAL char *gptr_t;
+
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef float f32x2 __attribute__((ext_vector_type(2)));
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+
+typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
+
+__device__ __forceinline__ float as_f32(uint32_t u) { return __builtin_bit_cast(float, u); }
+__device__ __forceinline__ uint32_t as_u32(float f) { return __builtin_bit_cast(uint32_t, f); }
+
+// Storage types.  The 16-bit ones say how the two halves of a packed dword become
+// fp32 and back (round to nearest even both ways).
+struct BF16 {
+  static constexpr int kBytes = 2;
+  static __device__ __forceinline__ float lo(uint32_t w) { return as_f32(w << 16); }
+  static __device__ __forceinline__ float hi(uint32_t w) { return as_f32(w & 0xffff0000u); }
+  // as __float2bfloat16 of the reference (csrc/include/sequential_scan_kernel_bf16.cuh:54)
+  static __device__ __forceinline__ uint32_t pack2(float a, float b) {
+    f32x2 v = {a, b};
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, bf16x2));
+  }
+  static __device__ __forceinline__ uint32_t bits(float x) { return as_u32(x) >> 16; }  // x exactly representable
+};
+struct F16 {
+  static constexpr int kBytes = 2;
+  static __device__ __forceinline__ float lo(uint32_t w) {
+    return static_cast<float>(__builtin_bit_cast(_Float16, static_cast<uint16_t>(w)));
+  }
+  static __device__ __forceinline__ float hi(uint32_t w) {
+    return static_cast<float>(__builtin_bit_cast(_Float16, static_cast<uint16_t>(w >> 16)));
+  }
+  static __device__ __forceinline__ uint32_t pack2(float a, float b) {
+    f32x2 v = {a, b};
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, f16x2));
+  }
+  static __device__ __forceinline__ uint32_t bits(float x) {
+    return __builtin_bit_cast(uint16_t, static_cast<_Float16>(x));
+  }
+};
+struct F32 {
+  static constexpr int kBytes = 4;
+};
+
+// Pins a wave-uniform pointer into scalar registers, so that `p + lane_offset`
+// becomes the scalar-base + 32-bit-vector-offset form of a global access and
+// costs no vector registers or 64-bit vector adds per row.
+template <typename Ptr>
+__device__ __forceinline__ Ptr uniform_ptr(Ptr ptr) {
+  const uint64_t u = reinterpret_cast<uint64_t>(ptr);
+  const uint32_t lo = __builtin_amdgcn_readfirstlane(static_cast<uint32_t>(u));
+  const uint32_t hi = __builtin_amdgcn_readfirstlane(static_cast<uint32_t>(u >> 32));
+  return reinterpret_cast<Ptr>((static_cast<uint64_t>(hi) << 32) | lo);
+}
+
+// Loads/stores of N dwords per lane.  NT marks the access non-temporal: the data
+// is touched once, so the caches should not keep it in preference to other lines.
+template <int N, bool NT>
+struct DwordIO;
+template <bool NT>
+struct DwordIO<1, NT> {
+  static __device__ __forceinline__ void load(uint32_t *dst, gcptr_t p) {
+    const FSS_GLOBAL uint32_t *q = reinterpret_cast<const FSS_GLOBAL uint32_t *>(p);
+    dst[0] = NT ? __builtin_nontemporal_load(q) : *q;
+  }
+  static __device__ __forceinline__ void store(gptr_t p, const uint32_t *src) {
+    FSS_GLOBAL uint32_t *q = reinterpret_cast<FSS_GLOBAL uint32_t *>(p);
+    if (NT)
+      __builtin_nontemporal_store(src[0], q);
+    else
+      *q = src[0];
+  }
+};
+template <bool NT>
+struct DwordIO<2, NT> {
+  static __device__ __forceinline__ void load(uint32_t *dst, gcptr_t p) {
+    const FSS_GLOBAL u32x2 *q = reinterpret_cast<const FSS_GLOBAL u32x2 *>(p);
+    const u32x2 v = NT ? __builtin_nontemporal_load(q) : *q;
+    dst[0] = v.x;
+    dst[1] = v.y;
+  }
+  static __device__ __forceinline__ void store(gptr_t p, const uint32_t *src) {
+    const u32x2 v = {src[0], src[1]};
+    FSS_GLOBAL u32x2 *q = reinterpret_cast<FSS_GLOBAL u32x2 *>(p);
+    if (NT)
+      __builtin_nontemporal_store(v, q);
+    else
+      *q = v;
+  }
+};
+template <bool NT>
+struct DwordIO<4, NT> {
+  static __device__ __forceinline__ void load(uint32_t *dst, gcptr_t p) {
+    const FSS_GLOBAL u32x4 *q = reinterpret_cast<const FSS_GLOBAL u32x4 *>(p);
+    const u32x4 v = NT ? __builtin_nontemporal_load(q) : *q;
+    dst[0] = v.x;
+    dst[1] = v.y;
+    dst[2] = v.z;
+    dst[3] = v.w;
+  }
+  static __device__ __forceinline__ void store(gptr_t p, const uint32_t *src) {
+    const u32x4 v = {src[0], src[1], src[2], src[3]};
+    FSS_GLOBAL u32x4 *q = reinterpret_cast<FSS_GLOBAL u32x4 *>(p);
+    if (NT)
+      __builtin_nontemporal_store(v, q);
+    else
+      *q = v;
+  }
+};
+
+// One row segment owned by a lane: VEC channels of element type E, kept packed.
+template <typename E, int VEC, int BYTES = E::kBytes>
+struct Row;
+
+template <typename E, int VEC>
+struct Row<E, VEC, 2> {
+  static_assert(VEC == 2 || VEC == 4 || VEC == 8, "16-bit vector width");
+  static constexpr int kDwords = VEC / 2;
+  static constexpr int kBytes = VEC * 2;
+  uint32_t dw[kDwords];
+  template <bool NT = false>
+  __device__ __forceinline__ void load(gcptr_t p) {
+    DwordIO<kDwords, NT>::load(dw, p);
+  }
+  template <bool NT = false>
+  __device__ __forceinline__ void store(gptr_t p) const {
+    DwordIO<kDwords, NT>::store(p, dw);
+  }
+  __device__ __forceinline__ float get(int i) const { return (i & 1) ? E::hi(dw[i >> 1]) : E::lo(dw[i >> 1]); }
+  __device__ __forceinline__ void fill(float x) {  // x exactly representable in E
+    const uint32_t b = E::bits(x);
+#pragma unroll
+    for (int i = 0; i < kDwords; ++i) dw[i] = b | (b << 16);
+  }
+  __device__ __forceinline__ void pack(const float *f) {
+#pragma unroll
+    for (int i = 0; i < kDwords; ++i) dw[i] = E::pack2(f[2 * i], f[2 * i + 1]);
+  }
+};
+
+template <typename E>
+struct Row<E, 1, 2> {
+  static constexpr int kDwords = 1;
+  static constexpr int kBytes = 2;
+  uint32_t dw[1];
+  template <bool NT = false>
+  __device__ __forceinline__ void load(gcptr_t p) {
+    const FSS_GLOBAL uint16_t *q = reinterpret_cast<const FSS_GLOBAL uint16_t *>(p);
+    dw[0] = NT ? __builtin_nontemporal_load(q) : *q;
+  }
+  template <bool NT = false>
+  __device__ __forceinline__ void store(gptr_t p) const {
+    FSS_GLOBAL uint16_t *q = reinterpret_cast<FSS_GLOBAL uint16_t *>(p);
+    if (NT)
+      __builtin_nontemporal_store(static_cast<uint16_t>(dw[0]), q);
+    else
+      *q = static_cast<uint16_t>(dw[0]);
+  }
+  __device__ __forceinline__ float get(int) const { return E::lo(dw[0]); }
+  __device__ __forceinline__ void fill(float x) { dw[0] = E::bits(x); }
+  __device__ __forceinline__ void pack(const float *f) { dw[0] = E::pack2(f[0], 0.0f) & 0xffffu; }
+};
+
+template <typename E, int VEC>
+struct Row<E, VEC, 4> {
+  static_assert(VEC == 1 || VEC == 2 || VEC == 4, "fp32 vector width");
+  static constexpr int kDwords = VEC;
+  static constexpr int kBytes = VEC * 4;
+  uint32_t dw[kDwords];
+  template <bool NT = false>
+  __device__ __forceinline__ void load(gcptr_t p) {
+    DwordIO<kDwords, NT>::load(dw, p);
+  }
+  template <bool NT = false>
+  __device__ __forceinline__ void store(gptr_t p) const {
+    DwordIO<kDwords, NT>::store(p, dw);
+  }
+  __device__ __forceinline__ float get(int i) const { return as_f32(dw[i]); }
+  __device__ __forceinline__ void fill(float x) {
+#pragma unroll
+    for (int i = 0; i < kDwords; ++i) dw[i] = as_u32(x);
+  }
+  __device__ __forceinline__ void pack(const float *f) {
+#pragma unroll
+    for (int i = 0; i < kDwords; ++i) dw[i] = as_u32(f[i]);
+  }
+};
+
+// Makes the compiler forget what it derived from a packed row: the rows stay
+// packed in registers across the chaining phase and are unpacked again after
+// it, instead of keeping an fp32 copy of every element alive next to them.
+template <typename RowT>
+__device__ __forceinline__ void keep_packed(RowT &r) {
+#pragma unroll
+  for (int i = 0; i < RowT::kDwords; ++i) asm volatile("" : "+v"(r.dw[i]));
+}
+
+// ---- workspace ----------------------------------------------------------------
+//
+// Header (kHeaderBytes): word 1 = top-level completion counter, word 2 = epoch,
+// word 3 = sticky error flag, words 64+32*i (i < 16, one 128-byte line each) =
+// first-level completion counters.  Then the tagged words,
+// [chunk][column tile][kind: map A, map B, outgoing state][VEC][64 lanes].
+
+enum : int { HDR_DONE = 1, HDR_EPOCH = 2, HDR_ERROR = 3, HDR_SLOT0 = 64, HDR_SLOT_STRIDE = 32 };
+constexpr int kDoneSlots = 16;
+constexpr size_t kHeaderBytes = 4096;
+// Polls a wave makes before it gives up on an earlier chunk (each poll is a memory
+// round trip plus a sleep: seconds in total, far beyond any healthy wait).
+constexpr uint32_t kSpinLimit = 1u << 20;
+// Most waves of a workgroup that look back in parallel, one earlier chunk each.
+constexpr int kMaxLookWaves = 16;
+enum : uint32_t { kPredNone = 0, kPredMap = 1, kPredState = 2 };
+
+__device__ __forceinline__ uint32_t ld_u32(const uint32_t *p) {
+  return __hip_atomic_load((const FSS_GLOBAL uint32_t *)p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ void st_u32(uint32_t *p, uint32_t v) {
+  __hip_atomic_store((FSS_GLOBAL uint32_t *)p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ uint32_t add_u32(uint32_t *p, uint32_t v) {
+  return __hip_atomic_fetch_add((FSS_GLOBAL uint32_t *)p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ uint64_t ld_word(const uint64_t *p) {
+  return __hip_atomic_load((const FSS_GLOBAL uint64_t *)p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ void st_word(uint64_t *p, uint32_t tag, float v) {
+  __hip_atomic_store((FSS_GLOBAL uint64_t *)p, (static_cast<uint64_t>(tag) << 32) | as_u32(v), __ATOMIC_RELAXED,
+                     __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ uint32_t word_tag(uint64_t w) { return static_cast<uint32_t>(w >> 32); }
+__device__ __forceinline__ float word_val(uint64_t w) { return as_f32(static_cast<uint32_t>(w)); }
+
+struct ScanArgs {
+  const char *in_a;  // alpha
+  const char *in_b;  // beta (forward) / dout (backward)
+  const char *in_h;  // stored forward output (backward only)
+  char *out0;        // h (forward) / grad_beta (backward)
+  char *out1;        // grad_alpha (backward only)
+  int64_t seq;
+  int64_t d;
+  int32_t tiles_per_row;  // ceil(d / (64*VEC))
+  int32_t n_ctiles;       // bs * tiles_per_row
+  int32_t n_chunks;       // ceil(seq / (WAVES*STEPS))
+  int32_t n_tiles;        // n_ctiles * n_chunks
+  int32_t look_waves;     // waves that look back in parallel (1..min(WAVES, kMaxLookWaves))
+  uint32_t *hdr;          // workspace header
+  uint64_t *words;        // tagged words
+  const char *in_x;       // gated backward only: the scan's input x (in_a is the gate there)
+#ifdef FSS_TRACE
+  uint64_t *trace;        // debug build: 8 timestamps per tile, written by lane 0 of every wave 0
+#endif
+};
+
+// Optional (bs, d) fp32 rows of the scans with a state entering/leaving the sequence.
+// The plain scan is compiled against the empty variant, whose members are constant
+// nulls: it carries no kernel arguments for them and every use folds away.
+template <bool STATE>
+struct StateArgs {
+  const float *state_in;  // forward: h[-1]; backward: gradient reaching the state after the last step
+  float *state_out;       // forward: un-rounded state after the last step; backward: gradient w.r.t. h[-1]
+  const float *h_before;  // backward only: h[-1] of the forward (grad_alpha[0] = g[0] * h[-1])
+};
+template <>
+struct StateArgs<false> {
+  static constexpr const float *state_in = nullptr;
+  static constexpr float *state_out = nullptr;
+  static constexpr const float *h_before = nullptr;
+};
+
+// ---- the kernel ----------------------------------------------------------------
+
+// Which streams are accessed non-temporally (bit 0: alpha, 1: beta/dout, 2: saved h,
+// 3: h output of the forward, 4: gradient outputs of the backward).  Measured on
+// MI355X at bs8 seq4096 d1024, forward and backward alternating: marking the
+// three output streams and the backward's reads of h non-temporal takes the step
+// from 134 us to 113 us; marking the reads of alpha, beta or dout as well is slower.
+#ifndef FSS_NT_MASK
+#define FSS_NT_MASK 28
+#endif
+constexpr bool kNtA = (FSS_NT_MASK & 1) != 0;
+constexpr bool kNtB = (FSS_NT_MASK & 2) != 0;
+constexpr bool kNtH = (FSS_NT_MASK & 4) != 0;
+constexpr bool kNtOutFwd = (FSS_NT_MASK & 8) != 0;
+constexpr bool kNtOutBwd = (FSS_NT_MASK & 16) != 0;
+
+#ifdef FSS_TRACE
+#define FSS_STAMP(c, p, slot)                                                                   \
+  do {                                                                                          \
+    if ((p).trace && (c).lane == 0 && (c).wave == (c).trace_wave)                                \
+      (p).trace[(static_cast<size_t>((c).chunk) * (p).n_ctiles + (c).ctile) * 8 + (slot)] =       \
+          __builtin_amdgcn_s_memrealtime();                                                         \
+  } while (0)
+#else
+#define FSS_STAMP(c, p, slot) \
+  do {                        \
+  } while (0)
+#endif
+
+// What is fixed for a wave while it works on one tile.
+struct TileCtx {
+  int lane, wave, n_waves, look;
+  int chunk, ctile;      // position of the tile: chunk of the sequence, column tile
+  bool chained, last;    // more than one chunk in the sequence; this is the last one
+  uint32_t tag;          // epoch of this launch
+  int64_t tile_base;     // byte offset of (batch, row 0, first channel of the tile)
+  int64_t chan_row;      // index of (batch, first channel of the tile) in a (bs, d) array; wave-uniform
+  int64_t r0;            // first scan-order index of this wave's slice
+  int64_t seq, row_bytes;
+  uint32_t lane_off;     // byte offset of the lane's channels inside the tile's row segment
+  bool col_ok;           // the lane's channels exist (d % VEC == 0, so all or none)
+  float2 *lds_map;       // [wave][v][lane] = (A, B) of this tile
+  float2 *lds_pred;      // [look wave][v][lane] = what an earlier chunk offers
+  float *lds_hin;        // [v][lane] = the chunk's incoming state, for every wave to read
+  uint32_t *s_kind;      // [look wave] kind of that offer
+  uint32_t *s_resolved;  // look-back finished (one word per workgroup)
+#ifdef FSS_TRACE
+  int trace_wave;
+#endif
+};
+
+// One look at what chunk `j` of this column tile offers: its outgoing state if it
+// has published one, else (j > 0) its map.  Split in two so that other work can be
+// placed between the loads and the use of what they return.
+template <int VEC>
+struct ChunkWords {
+  uint64_t a[VEC], b[VEC], s[VEC];
+};
+
+template <int VEC>
+__device__ __forceinline__ void poll_issue(const ScanArgs &p, const TileCtx &c, int j, ChunkWords<VEC> &w) {
+  const uint64_t *theirs = p.words + (static_cast<size_t>(j) * p.n_ctiles + c.ctile) * 3 * (64 * VEC) + c.lane;
+#pragma unroll
+  for (int v = 0; v < VEC; ++v) {
+    w.s[v] = ld_word(theirs + (2 * VEC + v) * 64);
+    w.a[v] = ld_word(theirs + (0 * VEC + v) * 64);
+    w.b[v] = ld_word(theirs + (1 * VEC + v) * 64);
+  }
+}
+
+// The answer is taken for the whole wave, so that one word per wave can describe
+// it.  Returns kPredNone when neither a state nor a map is there yet.
+template <int VEC>
+__device__ __forceinline__ uint32_t poll_eval(const TileCtx &c, int j, const ChunkWords<VEC> &w, float *qA,
+                                              float *qB) {
+  bool have_state = true, have_map = true;
+#pragma unroll
+  for (int v = 0; v < VEC; ++v) {
+    have_state = have_state && word_tag(w.s[v]) == c.tag;
+    have_map = have_map && word_tag(w.a[v]) == c.tag && word_tag(w.b[v]) == c.tag;
+  }
+  if (__builtin_amdgcn_ballot_w64(have_state) == ~0ull) {
+#pragma unroll
+    for (int v = 0; v < VEC; ++v) {
+      qA[v] = 0.0f;
+      qB[v] = word_val(w.s[v]);
+    }
+    return kPredState;
+  }
+  if (j > 0 && __builtin_amdgcn_ballot_w64(have_map) == ~0ull) {
+#pragma unroll
+    for (int v = 0; v < VEC; ++v) {
+      qA[v] = word_val(w.a[v]);
+      qB[v] = word_val(w.b[v]);
+    }
+    return kPredMap;
+  }
+  return kPredNone;
+}
+
+template <int VEC>
+__device__ __forceinline__ uint32_t poll_chunk(const ScanArgs &p, const TileCtx &c, int j, float *qA,
+                                               float *qB) {
+  ChunkWords<VEC> w;
+  poll_issue<VEC>(p, c, j, w);
+  return poll_eval<VEC>(c, j, w, qA, qB);
+}
+
+// (A, B) <- map[count-1] o ... o map[0] for this lane's channels: the maps of the
+// first `count` waves of the workgroup composed in scan order.  Reads go out in
+// small batches so that their LDS latencies overlap.
+template <int VEC>
+__device__ __forceinline__ void fold_wave_maps(const float2 *lds_map, int lane, int count, float *A,
+                                               float *B) {
+  constexpr int kBatch = 4;
+#pragma unroll
+  for (int v = 0; v < VEC; ++v) {
+    A[v] = 1.0f;
+    B[v] = 0.0f;
+  }
+  for (int w0 = 0; w0 < count; w0 += kBatch) {
+    float2 m[kBatch][VEC];
+#pragma unroll
+    for (int i = 0; i < kBatch; ++i) {
+      const int w = w0 + i < count ? w0 + i : count - 1;  // clamped: the read stays in bounds
+#pragma unroll
+      for (int v = 0; v < VEC; ++v) m[i][v] = lds_map[(w * VEC + v) * 64 + lane];
+    }
+#pragma unroll
+    for (int i = 0; i < kBatch; ++i) {
+      if (w0 + i < count) {
+#pragma unroll
+        for (int v = 0; v < VEC; ++v) {
+          B[v] = __builtin_fmaf(m[i][v].x, B[v], m[i][v].y);
+          A[v] *= m[i][v].x;
+        }
+      }
+    }
+  }
+}
+
+// Phase 2.  In: this wave's slice as the map x -> mA*x + mB.  Out: the state
+// entering the slice.  Every wave of the workgroup must call it (barriers).
+//
+// After one barrier every wave composes the maps of the waves before it (its state
+// is then one multiply-add away from the chunk's incoming state), and wave 0 composes
+// all of them into the chunk's map and publishes it.  Meanwhile wave w (w < look)
+// fetches what chunk-1-w offers - its outgoing state if it has one, else its map -
+// so a look-back over `look` chunks costs one memory round trip instead of one per
+// chunk; wave 0 folds what they found and hands the chunk's incoming state to all
+// waves through LDS.  Chains longer than `look` repeat the fetch.
+template <int VEC>
+__device__ __forceinline__ void chain_chunks(const ScanArgs &p, const TileCtx &c, const float *mA,
+                                             const float *mB, const float *seq_in, float *state) {
+  constexpr int kLaneSlots = 64 * VEC;
+  const int lane = c.lane, wave = c.wave;
+#pragma unroll
+  for (int v = 0; v < VEC; ++v) c.lds_map[(wave * VEC + v) * 64 + lane] = make_float2(mA[v], mB[v]);
+  __syncthreads();
+  FSS_STAMP(c, p, 2);
+
+  const bool look_back = c.chained && c.chunk > 0;
+  uint64_t *mine = nullptr;
+  float cA[VEC], cB[VEC];
+  if (wave == 0 && c.chained && !c.last) {
+    // the chunk's own map, needed by later chunks: out as early as possible
+    fold_wave_maps<VEC>(c.lds_map, lane, c.n_waves, cA, cB);
+    mine = p.words + (static_cast<size_t>(c.chunk) * p.n_ctiles + c.ctile) * 3 * kLaneSlots + lane;
+    if (c.chunk > 0) {
+#pragma unroll
+      for (int v = 0; v < VEC; ++v) {
+        st_word(mine + (0 * VEC + v) * 64, c.tag, cA[v]);
+        st_word(mine + (1 * VEC + v) * 64, c.tag, cB[v]);
+      }
+    }
+  }
+  FSS_STAMP(c, p, 3);
+
+  // (pA, pB): what the waves before this one do to the chunk's incoming state
+  float pA[VEC], pB[VEC];
+  if (!look_back) fold_wave_maps<VEC>(c.lds_map, lane, wave, pA, pB);
+
+  if (!look_back) {
+    // first chunk of the sequence (or the only one): the incoming state is the
+    // sequence's own (0 in the plain scan)
+    if (wave == 0 && c.chained && !c.last) {
+#pragma unroll
+      for (int v = 0; v < VEC; ++v)
+        st_word(mine + (2 * VEC + v) * 64, c.tag, seq_in ? __builtin_fmaf(cA[v], seq_in[v], cB[v]) : cB[v]);
+    }
+#pragma unroll
+    for (int v = 0; v < VEC; ++v) state[v] = seq_in ? __builtin_fmaf(pA[v], seq_in[v], pB[v]) : pB[v];
+    FSS_STAMP(c, p, 5);
+    return;
+  }
+
+  float hin[VEC], accA[VEC], accB[VEC];
+#pragma unroll
+  for (int v = 0; v < VEC; ++v) {
+    accA[v] = 1.0f;
+    accB[v] = hin[v] = 0.0f;
+  }
+  int nearest = c.chunk - 1;  // nearest earlier chunk not folded yet
+  for (;;) {
+    const int j = nearest - wave;
+    if (wave < c.look && j >= 0) {
+      float qA[VEC], qB[VEC];
+      uint32_t kind = kPredNone;
+      uint32_t polls = 0;
+      while ((kind = poll_chunk<VEC>(p, c, j, qA, qB)) == kPredNone) {
+        if (++polls > kSpinLimit) {
+          if (lane == 0) st_u32(p.hdr + HDR_ERROR, 1u);
+          kind = kPredState;  // give up: zero state, so that the grid still drains
+#pragma unroll
+          for (int v = 0; v < VEC; ++v) qA[v] = qB[v] = 0.0f;
+          break;
+        }
+        __builtin_amdgcn_s_sleep(2);
+      }
+#pragma unroll
+      for (int v = 0; v < VEC; ++v) c.lds_pred[(wave * VEC + v) * 64 + lane] = make_float2(qA[v], qB[v]);
+      if (lane == 0) c.s_kind[wave] = kind;
+    }
+    __syncthreads();
+    if (wave == 0) {
+      bool resolved = false;
+      for (int w = 0; w < c.look && nearest - w >= 0 && !resolved; ++w) {
+        const bool is_state = c.s_kind[w] == kPredState;
+#pragma unroll
+        for (int v = 0; v < VEC; ++v) {
+          const float2 m = c.lds_pred[(w * VEC + v) * 64 + lane];
+          if (is_state) {
+            hin[v] = __builtin_fmaf(accA[v], m.y, accB[v]);
+          } else {
+            accB[v] = __builtin_fmaf(accA[v], m.y, accB[v]);
+            accA[v] *= m.x;
+          }
+        }
+        resolved = is_state;
+      }
+      if (resolved) {
+#pragma unroll
+        for (int v = 0; v < VEC; ++v) c.lds_hin[v * 64 + lane] = hin[v];
+        if (!c.last) {
+#pragma unroll
+          for (int v = 0; v < VEC; ++v)
+            st_word(mine + (2 * VEC + v) * 64, c.tag, __builtin_fmaf(cA[v], hin[v], cB[v]));
+        }
+      }
+      if (lane == 0) *c.s_resolved = resolved ? 1u : 0u;
+    }
+    __syncthreads();
+    if (*c.s_resolved != 0u) break;  // chunk 0 always offers a state, so this is reached
+    nearest -= c.look;
+    if (nearest < 0) {  // cannot happen; never spin on a logic error
+      if (threadIdx.x == 0) st_u32(p.hdr + HDR_ERROR, 1u);
+      break;
+    }
+  }
+  FSS_STAMP(c, p, 4);
+  fold_wave_maps<VEC>(c.lds_map, lane, wave, pA, pB);  // after the polls: those are what is waited for
+#pragma unroll
+  for (int v = 0; v < VEC; ++v) state[v] = __builtin_fmaf(pA[v], c.lds_hin[v * 64 + lane], pB[v]);
+  FSS_STAMP(c, p, 5);
+}
+
+// Two-level completion count (16 first-level counters on separate lines keep the
+// atomics off one hot address).  Whoever counts last knows that no workgroup will
+// read the workspace again and advances the epoch for the next launch.
+__device__ __forceinline__ void count_out(const ScanArgs &p, const TileCtx &c) {
+  if (c.chained && threadIdx.x == 0) {
+    const uint32_t slot = blockIdx.x % kDoneSlots;
+    const uint32_t in_slot = (gridDim.x - slot + kDoneSlots - 1) / kDoneSlots;
+    uint32_t *counter = p.hdr + HDR_SLOT0 + slot * HDR_SLOT_STRIDE;
+    if (add_u32(counter, 1u) == in_slot - 1) {
+      st_u32(counter, 0u);
+      const uint32_t slots_used = gridDim.x < kDoneSlots ? gridDim.x : kDoneSlots;
+      if (add_u32(p.hdr + HDR_DONE, 1u) == slots_used - 1) {
+        st_u32(p.hdr + HDR_DONE, 0u);
+        // 0 is the tag of never-written words: skip it when the counter wraps
+        st_u32(p.hdr + HDR_EPOCH, c.tag + 1u == 0u ? 1u : c.tag + 1u);
+      }
+    }
+  }
+}
+
+}  // namespace fss

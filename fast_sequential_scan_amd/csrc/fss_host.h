@@ -1,0 +1,343 @@
+// Host-side pieces shared by the translation units of the library: launch planning,
+// device checks, the ordering of scans across streams, residency of a kernel.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include <string.h>
+
+#include <initializer_list>
+#include <mutex>
+
+#include "../../include/fss_scan.h"
+#include "fss_device.h"
+
+namespace fss {
+
+extern thread_local int tls_hip_error;  // hipError_t of this thread's last failed HIP call
+#ifdef FSS_TRACE
+extern uint64_t *g_trace;
+#endif
+
+inline int64_t ceil_div(int64_t a, int64_t b) { return (a + b - 1) / b; }
+
+// Register budget: packed dwords a lane may hold per input tensor.
+inline int max_vec_steps(int dtype) { return dtype != FSS_F32 ? 64 : 32; }  // vec*steps
+
+// LDS: one (A,B) slot per lane and vector element for every wave, twice (tiles
+// alternate between two sets), the same for every wave that looks back, and two
+// rows of incoming states.
+constexpr size_t kLdsBudget = 60 * 1024;
+inline int look_waves(int waves, int vec) {
+  int look = waves < kMaxLookWaves ? waves : kMaxLookWaves;
+  while (look > 1 && static_cast<size_t>(2 * waves + look + 1) * vec * 512 > kLdsBudget) --look;
+  return look;
+}
+inline size_t lds_bytes(int waves, int vec) {
+  return static_cast<size_t>(2 * waves + look_waves(waves, vec) + 1) * vec * 512;
+}
+
+inline bool config_valid(const fss_config &c, int dtype, bool gated = false, int dir = FSS_FWD) {
+  // the gated kernels exist for 4 bytes (or one element) per lane; their backward holds
+  // four tensors, so at most 16 timesteps per lane
+  if (gated && (c.vec > (dtype != FSS_F32 ? 2 : 1) || (dir == FSS_BWD && c.steps > 16))) return false;
+  const bool vec_ok = dtype != FSS_F32 ? (c.vec == 1 || c.vec == 2 || c.vec == 4 || c.vec == 8)
+                                        : (c.vec == 1 || c.vec == 2 || c.vec == 4);
+  const bool steps_ok = c.steps == 8 || c.steps == 16 || c.steps == 32;
+  if (!vec_ok || !steps_ok) return false;
+  if (c.vec * c.steps > max_vec_steps(dtype)) return false;
+  if (dtype != FSS_F32 && c.vec == 1 && c.steps > 32) return false;
+  if (c.waves < 1 || c.waves > 16) return false;
+  if (lds_bytes(c.waves, c.vec) > kLdsBudget) return false;
+  return true;
+}
+
+// Fills the zero fields of `c`.  `align` is the common alignment in bytes of all
+// tensors of the call.
+inline void complete_config(fss_config &c, int64_t bs, int64_t seq, int64_t d, int dtype, int dir,
+                     size_t align, bool gated = false) {
+  // Choices below come from sweeps on MI355X over the five measured workloads
+  // (bs8 d1024 seq512..8192, bs16 d512 seq2048, bs4 d2048 seq8192, bs2 d768
+  // seq1024, bs1 d256 seq65521).  What they showed: 4 bytes per lane per load
+  // (bf16 x2) with as many timesteps in registers as fit beats wider vectors;
+  // 8 waves per workgroup (two workgroups per CU, one loading while the other
+  // chains and stores) beats 16 unless the chain of chunks is long; with few
+  // channels, one channel per lane (twice the column tiles) and shorter slices
+  // put more waves in flight.
+  const int esize = dtype != FSS_F32 ? 2 : 4;
+  const int64_t channels = bs * d;
+  if (c.vec == 0) {
+    // 4 bytes per lane and load either way: two bf16 channels or one fp32 channel
+    const bool can2 = dtype != FSS_F32 && d % 2 == 0 && align % (2 * static_cast<size_t>(esize)) == 0;
+    int v = can2 ? 2 : 1;
+    // few channels: more, narrower column tiles; also never pad a row to twice its width
+    if (v == 2 && (channels < 8192 || ceil_div(d, 128) * 128 >= 2 * ceil_div(d, 64) * 64)) v = 1;
+    // forward: if two channels per lane leave at most one tile per resident workgroup, the whole
+    // scan is a single round of load - chain - store with nothing overlapping; one channel per
+    // lane gives twice the tiles (measured 8-9 % faster at bs16 seq2048 d512 and bs8 seq2048 d1024)
+    if (v == 2 && dir == FSS_FWD && bs * ceil_div(d, 128) * ceil_div(seq, 256) <= 512) v = 1;
+    c.vec = v;
+  }
+  // packed dwords one lane holds per timestep and tensor
+  const int dwords = dtype != FSS_F32 ? (c.vec + 1) / 2 : c.vec;
+  if (c.steps == 0) {
+    int s = 32 / dwords;  // 32 packed dwords per lane and tensor (the backward loads half of its third one late)
+    if (s > 32) s = 32;
+    if (s < 8) s = 8;
+    // backward: 32-step slices cost it a dozen spilled registers per lane (5 % more HBM
+    // traffic); that only pays where the chain of chunks is long.  Elsewhere 16 steps are
+    // as fast in bf16 and 6 % faster in fp32 (forward and backward alternating).
+    if (dir == FSS_BWD && s == 32 && (gated || ceil_div(seq, static_cast<int64_t>(8) * 32) <= 16)) s = 16;
+    // small problems: shorter slices until there are two 8-wave tiles per CU (512), as
+    // long as the machine still gets a few waves per SIMD out of it
+    const int64_t ctiles = bs * ceil_div(d, 64 * c.vec);
+    while (s > 16 && ctiles * ceil_div(seq, static_cast<int64_t>(8) * s) < 512) s >>= 1;
+    while (s > 8 && ctiles * ceil_div(seq, s) < 1024) s >>= 1;
+    // never longer than the sequence needs
+    while (s > 8 && seq <= s / 2) s >>= 1;
+    c.steps = s;
+  }
+  if (c.waves == 0) {
+    int64_t w = ceil_div(seq, c.steps);
+    // long chains of chunks (few channels, long sequence): the largest tile
+    const int64_t cap = ceil_div(seq, static_cast<int64_t>(8) * c.steps) > 64 ? 16 : 8;
+    if (w > cap) w = cap;
+    // many channels but a short sequence: half-size workgroups to reach 512 tiles
+    if (w == 8 && bs * ceil_div(d, 64 * c.vec) >= 64 &&
+        bs * ceil_div(d, 64 * c.vec) * ceil_div(seq, static_cast<int64_t>(8) * c.steps) < 512)
+      w = 4;
+    while (w > 1 && lds_bytes(static_cast<int>(w), c.vec) > kLdsBudget) --w;
+    c.waves = static_cast<int32_t>(w);
+  }
+}
+
+struct Plan {
+  fss_config cfg;
+  int64_t tiles_per_row, n_ctiles, n_chunks, n_tiles;
+  size_t ws_bytes;
+};
+
+inline int make_plan(Plan &pl, int64_t bs, int64_t seq, int64_t d, int dtype, int dir, size_t align,
+              const fss_config *user) {
+  if (bs < 0 || seq < 0 || d < 0) return FSS_ERR_BAD_SHAPE;
+  if (dtype != FSS_BF16 && dtype != FSS_F32 && dtype != FSS_F16) return FSS_ERR_BAD_CONFIG;
+  if (dir < FSS_FWD || dir > FSS_GATED_BWD) return FSS_ERR_BAD_CONFIG;
+  const bool gated = dir >= FSS_GATED_FWD;
+  dir &= 1;
+  const int esize = dtype != FSS_F32 ? 2 : 4;
+  // bs*seq*d*esize must fit int64
+  if (bs > 0 && seq > 0 && d > 0) {
+    const __int128 total = static_cast<__int128>(bs) * seq * d * esize;
+    if (total > (static_cast<__int128>(1) << 62)) return FSS_ERR_BAD_SHAPE;
+  }
+  fss_config c = {0, 0, 0, 0};
+  if (user) c = *user;
+  if (c.max_groups < 0) return FSS_ERR_BAD_CONFIG;
+  const int64_t dd = d > 0 ? d : 1, ss = seq > 0 ? seq : 1, bb = bs > 0 ? bs : 1;
+  complete_config(c, bb, ss, dd, dtype, dir, align, gated);
+  if (!config_valid(c, dtype, gated, dir)) return FSS_ERR_BAD_CONFIG;
+  if (dd % c.vec != 0) return FSS_ERR_BAD_CONFIG;
+  if (align % (static_cast<size_t>(c.vec) * esize) != 0) return FSS_ERR_MISALIGNED;
+  pl.cfg = c;
+  pl.tiles_per_row = ceil_div(dd, 64 * c.vec);
+  pl.n_ctiles = bb * pl.tiles_per_row;
+  pl.n_chunks = ceil_div(ss, static_cast<int64_t>(c.waves) * c.steps);
+  pl.n_tiles = pl.n_ctiles * pl.n_chunks;
+  if (pl.n_ctiles > INT32_MAX || pl.n_chunks > INT32_MAX || pl.n_tiles > INT32_MAX) return FSS_ERR_BAD_SHAPE;
+  pl.ws_bytes = kHeaderBytes;
+  if (pl.n_chunks > 1) pl.ws_bytes += static_cast<size_t>(pl.n_tiles) * 3 * 64 * c.vec * sizeof(uint64_t);
+  return FSS_OK;
+}
+
+inline size_t common_alignment(std::initializer_list<const void *> ptrs) {
+  uintptr_t bits = 0;
+  for (const void *p : ptrs) bits |= reinterpret_cast<uintptr_t>(p);
+  bits |= 16;  // 16 bytes is all any path needs
+  return static_cast<size_t>(bits & (~bits + 1));
+}
+
+inline int check_device() {
+  static int cached[64];  // 0 unknown, 1 ok, 2 unsupported
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess) return FSS_ERR_LAUNCH;
+  if (dev < 0 || dev >= 64) return FSS_OK;
+  int state = __atomic_load_n(&cached[dev], __ATOMIC_RELAXED);
+  if (state == 0) {
+    hipDeviceProp_t prop;
+    hipError_t e = hipGetDeviceProperties(&prop, dev);
+    if (e != hipSuccess) {
+      tls_hip_error = static_cast<int>(e);
+      return FSS_ERR_LAUNCH;
+    }
+    state = strncmp(prop.gcnArchName, "gfx950", 6) == 0 ? 1 : 2;
+    __atomic_store_n(&cached[dev], state, __ATOMIC_RELAXED);
+  }
+  return state == 1 ? FSS_OK : FSS_ERR_UNSUPPORTED_DEVICE;
+}
+
+// Scans of one process never overlap on a device.  A scan's workgroups wait for each
+// other and its grid is sized to fill the device, so two scans sharing the device
+// could each hold the compute units the other's unscheduled workgroups need, and
+// both would sit there until their waits give up.  Launches on one stream are
+// ordered anyway; when the stream changes, the new launch is made to wait for
+// everything queued on the previous stream.  The lock is held across the launch, so
+// that the event recorded by the next caller lands behind this one's kernel.
+// Streams under graph capture are left alone (a captured scan is ordered by its
+// graph; do not replay two graphs holding scans concurrently).
+struct ScanOrder {
+  std::mutex lock;
+  hipStream_t last = nullptr;
+  bool any = false;
+  hipEvent_t event = nullptr;
+};
+extern ScanOrder g_scan_order[64];
+
+inline bool stream_is_capturing(hipStream_t s) {
+  hipStreamCaptureStatus status = hipStreamCaptureStatusNone;
+  if (hipStreamIsCapturing(s, &status) != hipSuccess) {
+    (void)hipGetLastError();
+    return true;  // unknown: do not touch it
+  }
+  return status != hipStreamCaptureStatusNone;
+}
+
+class ScanOrderGuard {
+ public:
+  explicit ScanOrderGuard(hipStream_t s) {
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return;
+    order_ = &g_scan_order[dev];
+    order_->lock.lock();
+    if (stream_is_capturing(s)) return;
+    if (order_->any && order_->last != s && !stream_is_capturing(order_->last)) {
+      if (!order_->event && hipEventCreateWithFlags(&order_->event, hipEventDisableTiming) != hipSuccess) {
+        order_->event = nullptr;
+        (void)hipGetLastError();
+      }
+      // a stream the caller has destroyed since makes the record fail: nothing to wait for then
+      if (order_->event && hipEventRecord(order_->event, order_->last) == hipSuccess)
+        (void)hipStreamWaitEvent(s, order_->event, 0);
+      (void)hipGetLastError();
+    }
+    order_->last = s;
+    order_->any = true;
+  }
+  ~ScanOrderGuard() {
+    if (order_) order_->lock.unlock();
+  }
+  ScanOrderGuard(const ScanOrderGuard &) = delete;
+  ScanOrderGuard &operator=(const ScanOrderGuard &) = delete;
+
+ private:
+  ScanOrder *order_ = nullptr;
+};
+
+// Workgroups of `kernel` that are certainly resident together on the device (0 on
+// error).  Deliberately not the runtime's occupancy query: the kernel's waits
+// need a lower bound, and that query bounds by vector registers and LDS only.
+// These kernels hold many scalar registers as well (a row pointer per load); a
+// wave may be allocated 128 of the 800 a SIMD has, which caps a SIMD at 6 waves -
+// the residency measured on MI355X for the scalar-heaviest variants.
+template <typename Kernel>
+int resident_workgroups(Kernel kernel, int waves, size_t lds) {
+  static int cu_count = 0;
+  if (cu_count == 0) {
+    int dev = 0, n = 0;
+    if (hipGetDevice(&dev) != hipSuccess ||
+        hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0)
+      return 0;
+    cu_count = n;
+  }
+  hipFuncAttributes attr;
+  const hipError_t e = hipFuncGetAttributes(&attr, reinterpret_cast<const void *>(kernel));
+  if (e != hipSuccess) {
+    tls_hip_error = static_cast<int>(e);
+    return 0;
+  }
+  int vgprs = attr.numRegs > 0 ? attr.numRegs : 128;
+  vgprs = (vgprs + 7) / 8 * 8;                    // allocation granule
+  int per_simd = 512 / vgprs;                      // 512 vector registers per lane per SIMD
+  if (per_simd > 6) per_simd = 6;                  // scalar-register bound, see above
+  if (per_simd < 1) return 0;
+  int per_cu;
+  if (waves >= 4)
+    per_cu = per_simd / ((waves + 3) / 4);         // a workgroup puts ceil(waves/4) waves on a SIMD
+  else
+    per_cu = per_simd * (waves == 1 ? 4 : waves == 2 ? 2 : 1);
+  const size_t lds_alloc = (lds + attr.sharedSizeBytes + 1023) / 1024 * 1024;
+  const int by_lds = static_cast<int>((160 * 1024) / (lds_alloc ? lds_alloc : 1024));
+  if (per_cu > by_lds) per_cu = by_lds;
+  if (per_cu > 32) per_cu = 32;
+  return per_cu * cu_count;
+}
+
+// ---- channel-major planning -------------------------------------------------------------
+
+// rows per wave: 4 bytes-per-lane budgets as in the row-major kernels (two tensors of
+// 8 rows x 16 bytes forward, three of 4 rows backward)
+constexpr int kCmRowsFwd = 8, kCmRowsBwd = 4;
+
+struct CmPlan {
+  int vec, waves;
+  int64_t n_rowtiles, n_chunks, n_tiles;
+  size_t ws_bytes;
+};
+
+inline int make_cm_plan(CmPlan &pl, int64_t rows, int64_t seq, int dtype, int dir, size_t align, const fss_config *user) {
+  if (rows < 0 || seq < 0) return FSS_ERR_BAD_SHAPE;
+  if (dtype != FSS_BF16 && dtype != FSS_F32 && dtype != FSS_F16) return FSS_ERR_BAD_CONFIG;
+  if (dir != FSS_FWD && dir != FSS_BWD) return FSS_ERR_BAD_CONFIG;
+  const int esize = dtype != FSS_F32 ? 2 : 4;
+  const int64_t rr = rows > 0 ? rows : 1, ss = seq > 0 ? seq : 1;
+  if (static_cast<__int128>(rr) * ss * esize > (static_cast<__int128>(1) << 62)) return FSS_ERR_BAD_SHAPE;
+  const int widest = 16 / esize;  // 16 bytes per lane and load
+  int vec = user ? user->vec : 0, waves = user ? user->waves : 0;
+  if (user && (user->max_groups < 0 || user->steps != 0)) return FSS_ERR_BAD_CONFIG;
+  if (vec == 0) {
+    vec = widest;
+    // rows start at multiples of seq elements: every row must keep the vectors aligned
+    while (vec > 2 || (vec == 2 && esize == 4)) {
+      if (ss % vec == 0 && align % (static_cast<size_t>(vec) * esize) == 0) break;
+      vec = 2;  // only 1, 2 and the widest are compiled (fp32: 1 and 4)
+      if (esize == 4) vec = 1;
+    }
+    if (vec == 2 && (ss % 2 != 0 || align % (2 * static_cast<size_t>(esize)) != 0)) vec = 1;
+  }
+  const bool vec_ok = vec == 1 || vec == widest || (vec == 2 && esize == 2);
+  if (!vec_ok) return FSS_ERR_BAD_CONFIG;
+  if (ss % vec != 0) return FSS_ERR_BAD_CONFIG;
+  if (align % (static_cast<size_t>(vec) * esize) != 0) return FSS_ERR_MISALIGNED;
+  if (waves == 0) {
+    const int64_t w = ceil_div(ss, static_cast<int64_t>(64) * vec);
+    waves = static_cast<int>(w < 8 ? w : 8);
+  }
+  if (waves < 1 || waves > 16) return FSS_ERR_BAD_CONFIG;
+  pl.vec = vec;
+  pl.waves = waves;
+  pl.n_rowtiles = ceil_div(rr, dir == FSS_BWD ? kCmRowsBwd : kCmRowsFwd);
+  pl.n_chunks = ceil_div(ss, static_cast<int64_t>(waves) * 64 * vec);
+  pl.n_tiles = pl.n_rowtiles * pl.n_chunks;
+  if (pl.n_rowtiles > INT32_MAX || pl.n_chunks > INT32_MAX || pl.n_tiles > INT32_MAX) return FSS_ERR_BAD_SHAPE;
+  pl.ws_bytes = kHeaderBytes;
+  if (pl.n_chunks > 1) pl.ws_bytes += static_cast<size_t>(pl.n_tiles) * 3 * 64 * sizeof(uint64_t);
+  return FSS_OK;
+}
+
+
+// ---- what each translation unit provides --------------------------------------------------
+
+// fss_scan_rm.hip, compiled once per storage type: launches the row-major kernel (plain,
+// with states, or gated) the plan asks for.
+int launch_rm_bf16(const ScanArgs &args, const StateArgs<true> &state, const Plan &pl, bool bwd, bool gated,
+                   bool with_state, hipStream_t stream);
+int launch_rm_f16(const ScanArgs &args, const StateArgs<true> &state, const Plan &pl, bool bwd, bool gated,
+                  bool with_state, hipStream_t stream);
+int launch_rm_f32(const ScanArgs &args, const StateArgs<true> &state, const Plan &pl, bool bwd, bool gated,
+                  bool with_state, hipStream_t stream);
+
+// fss_scan_cm.hip
+int run_cm_scan(int dtype, int dir, const void *alpha, const void *in_b, const void *in_h, void *out0, void *out1,
+                int64_t bs, int64_t d, int64_t seq, void *workspace, size_t workspace_bytes, void *stream,
+                const fss_config *cfg);
+
+}  // namespace fss
