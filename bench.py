@@ -15,6 +15,9 @@ tensors already resident in HBM.  Prints ONE JSON line:
                    timed region (less what an empty pair of events reads, calibrated
                    in the same run); `traffic` is the counter-measured HBM bytes per
                    launch from profiles/, when that summary covers the configuration
+  rotating_sets    the same step over eight sets of tensors in rotation, so that no step finds its
+                   inputs in the memory-side cache (`value` reuses one set, as the reference's
+                   benchmark does); `--rotate 8` makes that the timed region itself
   cpu_baseline     the reference's PyTorch sequential loop (oracle/torch_loop.py) on the
                    host cores, same inputs, fp32; also the parity check of this run
 """
@@ -259,6 +262,32 @@ def main() -> int:
     bwd_gbps = bwd_bytes_per_elem * n_elem / (bwd_mean * 1e-3) / 1e9
     fwd_gbps = fwd_bytes_per_elem * n_elem / (fwd_mean * 1e-3) / 1e9
 
+    # ---- the same step over eight tensor sets in rotation (nothing reused between steps), unless
+    # the timed region above already rotated; reported next to `value`, never as `value` ----
+    rotating = {}
+    if len(pointer_sets) == 1 and args.flush_mb > 0:
+        extra = [(alpha.clone(), beta.clone(), dout.clone(), torch.empty_like(h), torch.empty_like(h),
+                  torch.empty_like(h)) for _ in range(7)]
+        pointer_sets.extend(tuple(t.data_ptr() for t in ts) for ts in extra)
+        n_rot = max(16, K // 2)
+        for _ in range(8):
+            fwd()
+            bwd()
+            next_set()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(n_rot):
+            fwd()
+            bwd()
+            next_set()
+        torch.cuda.synchronize()
+        rot_ms = (time.perf_counter() - t0) * 1e3 / n_rot
+        rotating = {"tensor_sets": len(pointer_sets), "steps": n_rot, "ms_per_step": round(rot_ms, 5),
+                    "GBps": round(step_bytes / (rot_ms * 1e-3) / 1e9, 1)}
+        del pointer_sets[1:]
+        del extra
+        first_set()
+
     # ---- cold timings: reading a large buffer between launches evicts L2 and the memory-side
     # cache and leaves them clean (a large write would leave dirty lines whose write-back is then
     # charged to the kernel under test) ----
@@ -434,6 +463,7 @@ def main() -> int:
             "avg_launch_ms": round(fwd_mean, 5),
         },
         "cold_cache": cold,
+        "rotating_sets": rotating,
         "autograd_path_ms_per_step": round(autograd_ms, 5),
         "parity": parity,
         "cpu_baseline": cpu,
