@@ -70,12 +70,19 @@ inline void complete_config(fss_config &c, int64_t bs, int64_t seq, int64_t d, i
     // 4 bytes per lane and load either way: two bf16 channels or one fp32 channel
     const bool can2 = dtype != FSS_F32 && d % 2 == 0 && align % (2 * static_cast<size_t>(esize)) == 0;
     int v = can2 ? 2 : 1;
-    // few channels: more, narrower column tiles; also never pad a row to twice its width
-    if (v == 2 && (channels < 8192 || ceil_div(d, 128) * 128 >= 2 * ceil_div(d, 64) * 64)) v = 1;
-    // forward: if two channels per lane leave at most one tile per resident workgroup, the whole
-    // scan is a single round of load - chain - store with nothing overlapping; one channel per
-    // lane gives twice the tiles (measured 8-9 % faster at bs16 seq2048 d512 and bs8 seq2048 d1024)
-    if (v == 2 && dir == FSS_FWD && bs * ceil_div(d, 128) * ceil_div(seq, 256) <= 512) v = 1;
+    // never pad a row to twice its width
+    if (v == 2 && ceil_div(d, 128) * 128 >= 2 * ceil_div(d, 64) * 64) v = 1;
+    // Few channels: more, narrower column tiles.  From a sweep over bs 1..64, seq 256..16384,
+    // d 256..4096: the forward prefers one channel per lane below 8192 channels unless the
+    // sequence is long, the backward only below 2048 (1024 for long sequences).
+    if (v == 2 && dir == FSS_FWD && (channels < 1024 || (channels < 8192 && seq < 8192))) v = 1;
+    if (v == 2 && dir == FSS_BWD && (channels < 1024 || (channels < 2048 && seq < 8192))) v = 1;
+    // Two channels per lane halve the number of tiles.  With fewer tiles than resident
+    // workgroups (512) one channel per lane is 25-30 % faster; in the forward also with exactly
+    // one tile per workgroup when the sequence has several chunks (the whole scan is then a single
+    // round of load - chain - store with nothing overlapping: 8-9 % at bs16 seq2048 d512).
+    const int64_t tiles2 = bs * ceil_div(d, 128) * ceil_div(seq, dir == FSS_FWD ? 256 : 128);
+    if (v == 2 && (tiles2 < 512 || (dir == FSS_FWD && tiles2 == 512 && seq > 256))) v = 1;
     c.vec = v;
   }
   // packed dwords one lane holds per timestep and tensor
@@ -88,11 +95,14 @@ inline void complete_config(fss_config &c, int64_t bs, int64_t seq, int64_t d, i
     // traffic); that only pays where the chain of chunks is long.  Elsewhere 16 steps are
     // as fast in bf16 and 6 % faster in fp32 (forward and backward alternating).
     if (dir == FSS_BWD && s == 32 && (gated || ceil_div(seq, static_cast<int64_t>(8) * 32) <= 16)) s = 16;
-    // small problems: shorter slices until there are two 8-wave tiles per CU (512), as
-    // long as the machine still gets a few waves per SIMD out of it
+    // small problems, backward: shorter slices until there are two 8-wave tiles per CU (512),
+    // as long as the machine still gets a few waves per SIMD out of it.  (The forward is
+    // fastest with 32 steps per lane down to the smallest sizes measured.)
     const int64_t ctiles = bs * ceil_div(d, 64 * c.vec);
-    while (s > 16 && ctiles * ceil_div(seq, static_cast<int64_t>(8) * s) < 512) s >>= 1;
-    while (s > 8 && ctiles * ceil_div(seq, s) < 1024) s >>= 1;
+    if (dir == FSS_BWD) {
+      while (s > 16 && ctiles * ceil_div(seq, static_cast<int64_t>(8) * s) < 512) s >>= 1;
+      while (s > 8 && ctiles * ceil_div(seq, s) < 1024) s >>= 1;
+    }
     // never longer than the sequence needs
     while (s > 8 && seq <= s / 2) s >>= 1;
     c.steps = s;
