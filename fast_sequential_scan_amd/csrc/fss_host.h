@@ -83,6 +83,11 @@ inline void complete_config(fss_config &c, int64_t bs, int64_t seq, int64_t d, i
     // round of load - chain - store with nothing overlapping: 8-9 % at bs16 seq2048 d512).
     const int64_t tiles2 = bs * ceil_div(d, 128) * ceil_div(seq, dir == FSS_FWD ? 256 : 128);
     if (v == 2 && (tiles2 < 512 || (dir == FSS_FWD && tiles2 == 512 && seq > 256))) v = 1;
+    // fp32, very large tensors (from 2^26 elements) with wide rows and sequences of a few
+    // thousand steps: 8 bytes per lane measured 5-15 % faster than 4 (below that size, slower)
+    if (dtype == FSS_F32 && d % 2 == 0 && align % 8 == 0 && d >= 512 && seq <= 4096 &&
+        bs * seq * d >= (static_cast<int64_t>(1) << 26))
+      v = 2;
     c.vec = v;
   }
   // packed dwords one lane holds per timestep and tensor
@@ -91,6 +96,7 @@ inline void complete_config(fss_config &c, int64_t bs, int64_t seq, int64_t d, i
     int s = 32 / dwords;  // 32 packed dwords per lane and tensor (the backward loads half of its third one late)
     if (s > 32) s = 32;
     if (s < 8) s = 8;
+    if (dtype == FSS_F32 && c.vec == 2 && dir == FSS_BWD) s = 8;  // three tensors of 8-byte rows
     // backward: 32-step slices cost it a dozen spilled registers per lane (5 % more HBM
     // traffic); that only pays where the chain of chunks is long.  Elsewhere 16 steps are
     // as fast in bf16 and 6 % faster in fp32 (forward and backward alternating).
@@ -112,10 +118,13 @@ inline void complete_config(fss_config &c, int64_t bs, int64_t seq, int64_t d, i
     // long chains of chunks (few channels, long sequence): the largest tile
     const int64_t cap = ceil_div(seq, static_cast<int64_t>(8) * c.steps) > 64 ? 16 : 8;
     if (w > cap) w = cap;
-    // many channels but a short sequence: half-size workgroups to reach 512 tiles
-    if (w == 8 && bs * ceil_div(d, 64 * c.vec) >= 64 &&
+    // many channels but a short sequence: half-size workgroups to reach 512 tiles (not where
+    // that would split a sequence that one workgroup covers, and so start a chain)
+    if (w == 8 && ceil_div(seq, static_cast<int64_t>(8) * c.steps) > 1 && bs * ceil_div(d, 64 * c.vec) >= 64 &&
         bs * ceil_div(d, 64 * c.vec) * ceil_div(seq, static_cast<int64_t>(8) * c.steps) < 512)
       w = 4;
+    // fp32 backward: a sequence that fits one workgroup of up to 16 waves is not chained at all
+    if (dtype == FSS_F32 && dir == FSS_BWD && w == 8 && ceil_div(seq, c.steps) <= 16) w = ceil_div(seq, c.steps);
     while (w > 1 && lds_bytes(static_cast<int>(w), c.vec) > kLdsBudget) --w;
     c.waves = static_cast<int32_t>(w);
   }
