@@ -66,6 +66,44 @@ inline void complete_config(fss_config &c, int64_t bs, int64_t seq, int64_t d, i
   // put more waves in flight.
   const int esize = dtype != FSS_F32 ? 2 : 4;
   const int64_t channels = bs * d;
+  if (gated) {
+    // The gated kernels spend as much time on arithmetic as on memory, and their sweep (same 75
+    // shapes, bf16) came out differently: two channels per lane from 2048 channels on in the
+    // backward (one channel per lane with 8 steps below), 16 steps there, and 4-wave workgroups
+    // while there are few tiles.
+    const bool wide = dtype != FSS_F32 && d % 2 == 0 && align % (2 * static_cast<size_t>(esize)) == 0 &&
+                      ceil_div(d, 128) * 128 < 2 * ceil_div(d, 64) * 64;
+    if (c.vec == 0) {
+      int v = wide ? 2 : 1;
+      // tiles with two channels per lane (forward 256, backward 128 timesteps long)
+      const int64_t tiles2 = bs * ceil_div(d, 128) * ceil_div(seq, dir == FSS_FWD ? 256 : 128);
+      if (dir == FSS_FWD && (channels < 1024 || (channels < 8192 && seq < 8192) || tiles2 < 512)) v = 1;
+      if (dir == FSS_BWD && (tiles2 < 128 || (channels < 2048 && seq < 4096) || (channels < 1024 && seq < 8192))) v = 1;
+      c.vec = v;
+    }
+    if (c.steps == 0) {
+      int s = dir == FSS_FWD ? 32 : (dtype != FSS_F32 && c.vec == 1) ? 8 : 16;
+      // forward, few tiles of a sequence of a thousand steps or more: half-length slices
+      if (dir == FSS_FWD && c.vec == 1 && seq >= 1024 && bs * ceil_div(d, 64) * ceil_div(seq, 256) <= 128) s = 16;
+      if (dtype == FSS_F32 && dir == FSS_BWD) {  // as the plain fp32 backward: shorter for small problems
+        const int64_t ct = bs * ceil_div(d, 64);
+        while (s > 8 && ct * ceil_div(seq, s) < 1024) s >>= 1;
+      }
+      while (s > 8 && seq <= s / 2) s >>= 1;
+      c.steps = s;
+    }
+    if (c.waves == 0) {
+      int64_t w = ceil_div(seq, c.steps);
+      const int64_t chunks8 = ceil_div(seq, static_cast<int64_t>(8) * c.steps);
+      const int64_t cap = chunks8 > 128 ? 16 : 8;
+      if (w > cap) w = cap;
+      const int64_t tiles = bs * ceil_div(d, 64 * c.vec) * chunks8;
+      if (w == 8 && chunks8 > 1 && chunks8 <= 16 && c.vec == 2 && tiles < (dir == FSS_FWD ? 1025 : 512)) w = 4;
+      while (w > 1 && lds_bytes(static_cast<int>(w), c.vec) > kLdsBudget) --w;
+      c.waves = static_cast<int32_t>(w);
+    }
+    return;
+  }
   if (c.vec == 0) {
     // 4 bytes per lane and load either way: two bf16 channels or one fp32 channel
     const bool can2 = dtype != FSS_F32 && d % 2 == 0 && align % (2 * static_cast<size_t>(esize)) == 0;
@@ -100,7 +138,7 @@ inline void complete_config(fss_config &c, int64_t bs, int64_t seq, int64_t d, i
     // backward: 32-step slices cost it a dozen spilled registers per lane (5 % more HBM
     // traffic); that only pays where the chain of chunks is long.  Elsewhere 16 steps are
     // as fast in bf16 and 6 % faster in fp32 (forward and backward alternating).
-    if (dir == FSS_BWD && s == 32 && (gated || ceil_div(seq, static_cast<int64_t>(8) * 32) <= 16)) s = 16;
+    if (dir == FSS_BWD && s == 32 && ceil_div(seq, static_cast<int64_t>(8) * 32) <= 16) s = 16;
     // small problems, backward: shorter slices until there are two 8-wave tiles per CU (512),
     // as long as the machine still gets a few waves per SIMD out of it.  (The forward is
     // fastest with 32 steps per lane down to the smallest sizes measured.)
