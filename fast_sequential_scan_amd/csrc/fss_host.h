@@ -367,6 +367,10 @@ inline int make_cm_plan(CmPlan &pl, int64_t rows, int64_t seq, int dtype, int di
   if (waves == 0) {
     const int64_t w = ceil_div(ss, static_cast<int64_t>(64) * vec);
     waves = static_cast<int>(w < 8 ? w : 8);
+    // forward, a chained sequence with few rows: half-size workgroups double the tiles in
+    // flight (10-15 % at bs1 d256 seq16384)
+    const int64_t chunks8 = ceil_div(ss, static_cast<int64_t>(8) * 64 * vec);
+    if (dir == FSS_FWD && waves == 8 && chunks8 >= 2 && ceil_div(rr, kCmRowsFwd) * chunks8 < 1024) waves = 4;
   }
   if (waves < 1 || waves > 16) return FSS_ERR_BAD_CONFIG;
   pl.vec = vec;
