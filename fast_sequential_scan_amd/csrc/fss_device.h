@@ -513,45 +513,42 @@ __device__ __forceinline__ void chain_chunks(const ScanArgs &p, const TileCtx &c
       if (lane == 0) c.s_kind[wave] = kind;
     }
     __syncthreads();
-    if (wave == 0) {
-      bool resolved = false;
-      for (int w = 0; w < c.look && nearest - w >= 0 && !resolved; ++w) {
-        const bool is_state = c.s_kind[w] == kPredState;
+    // every wave folds what the look-back waves found (the same few LDS reads in each wave
+    // cost less than a second barrier and a broadcast by wave 0)
+    bool resolved = false;
+    for (int w = 0; w < c.look && nearest - w >= 0 && !resolved; ++w) {
+      const bool is_state = c.s_kind[w] == kPredState;
 #pragma unroll
-        for (int v = 0; v < VEC; ++v) {
-          const float2 m = c.lds_pred[(w * VEC + v) * 64 + lane];
-          if (is_state) {
-            hin[v] = __builtin_fmaf(accA[v], m.y, accB[v]);
-          } else {
-            accB[v] = __builtin_fmaf(accA[v], m.y, accB[v]);
-            accA[v] *= m.x;
-          }
-        }
-        resolved = is_state;
-      }
-      if (resolved) {
-#pragma unroll
-        for (int v = 0; v < VEC; ++v) c.lds_hin[v * 64 + lane] = hin[v];
-        if (!c.last) {
-#pragma unroll
-          for (int v = 0; v < VEC; ++v)
-            st_word(mine + (2 * VEC + v) * 64, c.tag, __builtin_fmaf(cA[v], hin[v], cB[v]));
+      for (int v = 0; v < VEC; ++v) {
+        const float2 m = c.lds_pred[(w * VEC + v) * 64 + lane];
+        if (is_state) {
+          hin[v] = __builtin_fmaf(accA[v], m.y, accB[v]);
+        } else {
+          accB[v] = __builtin_fmaf(accA[v], m.y, accB[v]);
+          accA[v] *= m.x;
         }
       }
-      if (lane == 0) *c.s_resolved = resolved ? 1u : 0u;
+      resolved = is_state;
     }
-    __syncthreads();
-    if (*c.s_resolved != 0u) break;  // chunk 0 always offers a state, so this is reached
+    if (resolved) {  // chunk 0 always offers a state, so this is reached
+      if (wave == 0 && !c.last) {
+#pragma unroll
+        for (int v = 0; v < VEC; ++v)
+          st_word(mine + (2 * VEC + v) * 64, c.tag, __builtin_fmaf(cA[v], hin[v], cB[v]));
+      }
+      break;
+    }
     nearest -= c.look;
     if (nearest < 0) {  // cannot happen; never spin on a logic error
       if (threadIdx.x == 0) st_u32(p.hdr + HDR_ERROR, 1u);
       break;
     }
+    __syncthreads();  // the slots are about to be overwritten: wait until every wave has read them
   }
   FSS_STAMP(c, p, 4);
   fold_wave_maps<VEC>(c.lds_map, lane, wave, pA, pB);  // after the polls: those are what is waited for
 #pragma unroll
-  for (int v = 0; v < VEC; ++v) state[v] = __builtin_fmaf(pA[v], c.lds_hin[v * 64 + lane], pB[v]);
+  for (int v = 0; v < VEC; ++v) state[v] = __builtin_fmaf(pA[v], hin[v], pB[v]);
   FSS_STAMP(c, p, 5);
 }
 
