@@ -440,9 +440,9 @@ __device__ __forceinline__ void fold_wave_maps(const float2 *lds_map, int lane, 
 // so a look-back over `look` chunks costs one memory round trip instead of one per
 // chunk; wave 0 folds what they found and hands the chunk's incoming state to all
 // waves through LDS.  Chains longer than `look` repeat the fetch.
-template <int VEC>
+template <int VEC, typename Mid>
 __device__ __forceinline__ void chain_chunks(const ScanArgs &p, const TileCtx &c, const float *mA,
-                                             const float *mB, const float *seq_in, float *state) {
+                                             const float *mB, const float *seq_in, float *state, Mid &&mid) {
   constexpr int kLaneSlots = 64 * VEC;
   const int lane = c.lane, wave = c.wave;
 #pragma unroll
@@ -469,7 +469,10 @@ __device__ __forceinline__ void chain_chunks(const ScanArgs &p, const TileCtx &c
 
   // (pA, pB): what the waves before this one do to the chunk's incoming state
   float pA[VEC], pB[VEC];
-  if (!look_back) fold_wave_maps<VEC>(c.lds_map, lane, wave, pA, pB);
+  if (!look_back) {
+    mid();
+    fold_wave_maps<VEC>(c.lds_map, lane, wave, pA, pB);
+  }
 
   if (!look_back) {
     // first chunk of the sequence (or the only one): the incoming state is the
@@ -492,13 +495,17 @@ __device__ __forceinline__ void chain_chunks(const ScanArgs &p, const TileCtx &c
     accB[v] = hin[v] = 0.0f;
   }
   int nearest = c.chunk - 1;  // nearest earlier chunk not folded yet
+  bool first = true;
   for (;;) {
     const int j = nearest - wave;
     if (wave < c.look && j >= 0) {
       float qA[VEC], qB[VEC];
-      uint32_t kind = kPredNone;
       uint32_t polls = 0;
-      while ((kind = poll_chunk<VEC>(p, c, j, qA, qB)) == kPredNone) {
+      ChunkWords<VEC> w;
+      poll_issue<VEC>(p, c, j, w);
+      if (first) mid();  // behind the look's loads, so that those return first
+      uint32_t kind = poll_eval<VEC>(c, j, w, qA, qB);
+      while (kind == kPredNone && (kind = poll_chunk<VEC>(p, c, j, qA, qB)) == kPredNone) {
         if (++polls > kSpinLimit) {
           if (lane == 0) st_u32(p.hdr + HDR_ERROR, 1u);
           kind = kPredState;  // give up: zero state, so that the grid still drains
@@ -511,7 +518,10 @@ __device__ __forceinline__ void chain_chunks(const ScanArgs &p, const TileCtx &c
 #pragma unroll
       for (int v = 0; v < VEC; ++v) c.lds_pred[(wave * VEC + v) * 64 + lane] = make_float2(qA[v], qB[v]);
       if (lane == 0) c.s_kind[wave] = kind;
+    } else if (first) {
+      mid();
     }
+    first = false;
     __syncthreads();
     // every wave folds what the look-back waves found (the same few LDS reads in each wave
     // cost less than a second barrier and a broadcast by wave 0)

@@ -52,120 +52,104 @@ inline bool config_valid(const fss_config &c, int dtype, bool gated = false, int
   return true;
 }
 
+// One candidate launch configuration: taken when it yields at least `need` tiles.
+struct Rung {
+  int vec, steps, waves;
+  int64_t need;
+};
+
 // Fills the zero fields of `c`.  `align` is the common alignment in bytes of all
 // tensors of the call.
+//
+// From sweeps over bs 1..64, seq 256..16384, d 256..4096 per storage type and kernel
+// family (every shape against 8-11 configurations), which all show the same thing: the
+// largest tile that still leaves one tile per CU wins.  Large tiles mean few chunks per
+// sequence (a short chain) and long uninterrupted streams per wave; 16 waves of 32
+// (backward 16) timesteps with 4 bytes per lane is the largest that fits the register
+// file.  So the choice walks down a ladder of tile sizes, each half the one before, and
+// takes the first with at least 256 tiles; which of time, channels per lane and waves
+// is halved at each rung is what the sweeps decided.  Below the last rung the problem
+// is latency-bound and the smallest tile is as good as any.
 inline void complete_config(fss_config &c, int64_t bs, int64_t seq, int64_t d, int dtype, int dir,
                      size_t align, bool gated = false) {
-  // Choices below come from sweeps on MI355X over the five measured workloads
-  // (bs8 d1024 seq512..8192, bs16 d512 seq2048, bs4 d2048 seq8192, bs2 d768
-  // seq1024, bs1 d256 seq65521).  What they showed: 4 bytes per lane per load
-  // (bf16 x2) with as many timesteps in registers as fit beats wider vectors;
-  // 8 waves per workgroup (two workgroups per CU, one loading while the other
-  // chains and stores) beats 16 unless the chain of chunks is long; with few
-  // channels, one channel per lane (twice the column tiles) and shorter slices
-  // put more waves in flight.
-  const int esize = dtype != FSS_F32 ? 2 : 4;
-  const int64_t channels = bs * d;
-  if (gated) {
-    // The gated kernels spend as much time on arithmetic as on memory, and their sweep (same 75
-    // shapes, bf16) came out differently: two channels per lane from 2048 channels on in the
-    // backward (one channel per lane with 8 steps below), 16 steps there, and 4-wave workgroups
-    // while there are few tiles.
-    const bool wide = dtype != FSS_F32 && d % 2 == 0 && align % (2 * static_cast<size_t>(esize)) == 0 &&
-                      ceil_div(d, 128) * 128 < 2 * ceil_div(d, 64) * 64;
-    if (c.vec == 0) {
-      int v = wide ? 2 : 1;
-      // tiles with two channels per lane (forward 256, backward 128 timesteps long)
-      const int64_t tiles2 = bs * ceil_div(d, 128) * ceil_div(seq, dir == FSS_FWD ? 256 : 128);
-      if (dir == FSS_FWD && (channels < 1024 || (channels < 8192 && seq < 8192) || tiles2 < 512)) v = 1;
-      if (dir == FSS_BWD && (tiles2 < 128 || (channels < 2048 && seq < 4096) || (channels < 1024 && seq < 8192))) v = 1;
-      c.vec = v;
+  const bool narrow = dtype != FSS_F32;  // 16-bit storage
+  const int esize = narrow ? 2 : 4;
+  // two channels per lane: even d, 2-element alignment, and never pad a row to twice its width
+  const bool can2 = d % 2 == 0 && align % (2 * static_cast<size_t>(esize)) == 0 &&
+                    ceil_div(d, 128) * 128 < 2 * ceil_div(d, 64) * 64;
+  // fp32, very large tensors (from 2^26 elements) with wide rows and sequences of a few
+  // thousand steps: 8 bytes per lane measured 5-15 % faster than 4 (below that size, slower)
+  const bool wide32 = !narrow && !gated && can2 && d >= 512 && seq <= 4096 &&
+                      bs * seq * d >= (static_cast<int64_t>(1) << 26);
+  Rung ladder[6];
+  int n = 0;
+  auto rung = [&](int v, int s, int w, int64_t need = 256) { ladder[n++] = Rung{v, s, w, need}; };
+  const bool fwd = dir == FSS_FWD;
+  if (!gated && fwd) {
+    // (very long sequences: one channel per lane, i.e. twice the independent chains, is 5-16 % faster)
+    if (narrow && seq < 32768) rung(2, 32, 16);
+    if (wide32) rung(2, 16, 16);
+    rung(1, 32, 16);
+    if (seq <= 2048) rung(1, 16, 16);
+    rung(1, 32, 8, 0);
+  } else if (!gated) {
+    // 32-step slices would cost the backward a dozen spilled registers per lane
+    if (narrow) {
+      // one or two column tiles and hundreds of chunks: here the spills of 32-step slices are
+      // the lesser evil (bs1 seq65521 d256: 42 against 49 us)
+      if (seq > 49152 && bs * d <= 256) rung(1, 32, 8, 0);
+      rung(2, 16, 16);
+      if (seq >= 4096) rung(1, 16, 16); else rung(2, 16, 8);
+      if (seq > 256) rung(1, 16, 8); else rung(2, 8, 8);
+    } else {
+      if (wide32) rung(2, 8, 16);
+      rung(1, 16, 16);
+      rung(1, 16, 8);
     }
-    if (c.steps == 0) {
-      int s = dir == FSS_FWD ? 32 : (dtype != FSS_F32 && c.vec == 1) ? 8 : 16;
-      // forward, few tiles of a sequence of a thousand steps or more: half-length slices
-      if (dir == FSS_FWD && c.vec == 1 && seq >= 1024 && bs * ceil_div(d, 64) * ceil_div(seq, 256) <= 128) s = 16;
-      if (dtype == FSS_F32 && dir == FSS_BWD) {  // as the plain fp32 backward: shorter for small problems
-        const int64_t ct = bs * ceil_div(d, 64);
-        while (s > 8 && ct * ceil_div(seq, s) < 1024) s >>= 1;
-      }
-      while (s > 8 && seq <= s / 2) s >>= 1;
-      c.steps = s;
+    if (seq >= 2048) rung(1, 16, 8, 0); else rung(1, 8, 8, 0);
+  } else if (fwd) {
+    // The gated kernels spend as much time on arithmetic as on memory and like more, smaller
+    // waves; a sequence that 8 waves cover wants two workgroups per CU before it takes them.
+    if (narrow) {
+      if (seq > 256) rung(2, 32, 16); else rung(2, 32, 8, 512);
+      if (seq >= 4096) rung(1, 32, 16); else rung(2, 16, 16);
+      if (seq >= 16384) rung(1, 32, 8);
+      rung(1, 16, 16);
+      if (seq >= 1024) rung(1, 16, 8, 0); else rung(1, 16, 16, 0);
+    } else {
+      if (seq > 256) rung(1, 32, 16); else rung(1, 32, 8, 512);
+      rung(1, 16, 16, 0);
     }
-    if (c.waves == 0) {
-      int64_t w = ceil_div(seq, c.steps);
-      const int64_t chunks8 = ceil_div(seq, static_cast<int64_t>(8) * c.steps);
-      const int64_t cap = chunks8 > 128 ? 16 : 8;
-      if (w > cap) w = cap;
-      const int64_t tiles = bs * ceil_div(d, 64 * c.vec) * chunks8;
-      if (w == 8 && chunks8 > 1 && chunks8 <= 16 && c.vec == 2 && tiles < (dir == FSS_FWD ? 1025 : 512)) w = 4;
-      while (w > 1 && lds_bytes(static_cast<int>(w), c.vec) > kLdsBudget) --w;
-      c.waves = static_cast<int32_t>(w);
+  } else {
+    // gated backward: four tensors per timestep, at most 16 steps per lane (fp32: 8 are faster)
+    if (narrow) {
+      if (seq > 256) rung(2, 16, 16); else rung(2, 16, 8, 1024);
+      rung(2, 8, 16);
+      if (seq < 2048) rung(2, 8, 8); else rung(1, 8, 16);
+      if (seq <= 256) rung(2, 8, 8, 1);
+      rung(1, 8, 8, 0);
+    } else {
+      if (seq > 256) rung(1, 8, 16);
+      rung(1, 8, 8, 0);
     }
-    return;
   }
-  if (c.vec == 0) {
-    // 4 bytes per lane and load either way: two bf16 channels or one fp32 channel
-    const bool can2 = dtype != FSS_F32 && d % 2 == 0 && align % (2 * static_cast<size_t>(esize)) == 0;
-    int v = can2 ? 2 : 1;
-    // never pad a row to twice its width
-    if (v == 2 && ceil_div(d, 128) * 128 >= 2 * ceil_div(d, 64) * 64) v = 1;
-    // Few channels: more, narrower column tiles.  From a sweep over bs 1..64, seq 256..16384,
-    // d 256..4096: the forward prefers one channel per lane below 8192 channels unless the
-    // sequence is long, the backward only below 2048 (1024 for long sequences).
-    if (v == 2 && dir == FSS_FWD && (channels < 1024 || (channels < 8192 && seq < 8192))) v = 1;
-    if (v == 2 && dir == FSS_BWD && (channels < 1024 || (channels < 2048 && seq < 8192))) v = 1;
-    // Two channels per lane halve the number of tiles.  With fewer tiles than resident
-    // workgroups (512) one channel per lane is 25-30 % faster; in the forward also with exactly
-    // one tile per workgroup when the sequence has several chunks (the whole scan is then a single
-    // round of load - chain - store with nothing overlapping: 8-9 % at bs16 seq2048 d512).
-    const int64_t tiles2 = bs * ceil_div(d, 128) * ceil_div(seq, dir == FSS_FWD ? 256 : 128);
-    if (v == 2 && (tiles2 < 512 || (dir == FSS_FWD && tiles2 == 512 && seq > 256))) v = 1;
-    // fp32, very large tensors (from 2^26 elements) with wide rows and sequences of a few
-    // thousand steps: 8 bytes per lane measured 5-15 % faster than 4 (below that size, slower)
-    if (dtype == FSS_F32 && d % 2 == 0 && align % 8 == 0 && d >= 512 && seq <= 4096 &&
-        bs * seq * d >= (static_cast<int64_t>(1) << 26))
-      v = 2;
-    c.vec = v;
+  fss_config pick = {0, 0, 0, 0};
+  for (int i = 0; i < n; ++i) {
+    // what the caller fixed stays fixed
+    int v = c.vec ? c.vec : ladder[i].vec;
+    int s = c.steps ? c.steps : ladder[i].steps;
+    int w = c.waves ? c.waves : ladder[i].waves;
+    if (!c.vec && v == 2 && !can2) continue;
+    // never more waves or steps than the sequence needs
+    while (!c.waves && w > 1 && static_cast<int64_t>(s) * (w / 2) >= seq) w /= 2;
+    while (!c.steps && s > 8 && s / 2 >= seq) s /= 2;
+    while (!c.waves && w > 1 && lds_bytes(w, v) > kLdsBudget) --w;
+    pick = fss_config{v, s, w, 0};
+    if (bs * ceil_div(d, 64 * static_cast<int64_t>(v)) * ceil_div(seq, static_cast<int64_t>(s) * w) >= ladder[i].need) break;
   }
-  // packed dwords one lane holds per timestep and tensor
-  const int dwords = dtype != FSS_F32 ? (c.vec + 1) / 2 : c.vec;
-  if (c.steps == 0) {
-    int s = 32 / dwords;  // 32 packed dwords per lane and tensor (the backward loads half of its third one late)
-    if (s > 32) s = 32;
-    if (s < 8) s = 8;
-    if (dtype == FSS_F32 && c.vec == 2 && dir == FSS_BWD) s = 8;  // three tensors of 8-byte rows
-    // backward: 32-step slices cost it a dozen spilled registers per lane (5 % more HBM
-    // traffic); that only pays where the chain of chunks is long.  Elsewhere 16 steps are
-    // as fast in bf16 and 6 % faster in fp32 (forward and backward alternating).
-    if (dir == FSS_BWD && s == 32 && ceil_div(seq, static_cast<int64_t>(8) * 32) <= 16) s = 16;
-    // small problems, backward: shorter slices until there are two 8-wave tiles per CU (512),
-    // as long as the machine still gets a few waves per SIMD out of it.  (The forward is
-    // fastest with 32 steps per lane down to the smallest sizes measured.)
-    const int64_t ctiles = bs * ceil_div(d, 64 * c.vec);
-    if (dir == FSS_BWD) {
-      while (s > 16 && ctiles * ceil_div(seq, static_cast<int64_t>(8) * s) < 512) s >>= 1;
-      while (s > 8 && ctiles * ceil_div(seq, s) < 1024) s >>= 1;
-    }
-    // never longer than the sequence needs
-    while (s > 8 && seq <= s / 2) s >>= 1;
-    c.steps = s;
-  }
-  if (c.waves == 0) {
-    int64_t w = ceil_div(seq, c.steps);
-    // long chains of chunks (few channels, long sequence): the largest tile
-    const int64_t cap = ceil_div(seq, static_cast<int64_t>(8) * c.steps) > 64 ? 16 : 8;
-    if (w > cap) w = cap;
-    // many channels but a short sequence: half-size workgroups to reach 512 tiles (not where
-    // that would split a sequence that one workgroup covers, and so start a chain)
-    if (w == 8 && ceil_div(seq, static_cast<int64_t>(8) * c.steps) > 1 && bs * ceil_div(d, 64 * c.vec) >= 64 &&
-        bs * ceil_div(d, 64 * c.vec) * ceil_div(seq, static_cast<int64_t>(8) * c.steps) < 512)
-      w = 4;
-    // fp32 backward: a sequence that fits one workgroup of up to 16 waves is not chained at all
-    if (dtype == FSS_F32 && dir == FSS_BWD && w == 8 && ceil_div(seq, c.steps) <= 16) w = ceil_div(seq, c.steps);
-    while (w > 1 && lds_bytes(static_cast<int>(w), c.vec) > kLdsBudget) --w;
-    c.waves = static_cast<int32_t>(w);
-  }
+  c.vec = pick.vec;
+  c.steps = pick.steps;
+  c.waves = pick.waves;
 }
 
 struct Plan {

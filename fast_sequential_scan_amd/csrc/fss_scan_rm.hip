@@ -143,11 +143,12 @@ __device__ __forceinline__ void scan_tile(const ScanArgs &p, const StateArgs<STA
         hp[s].template load<kNtH>(uniform_ptr(ph + s * step_bytes) + lane_off);
     }
   };
-  if (BWD) {
+  auto load_h_early = [&] {
+    if (BWD) {
 #pragma unroll
-    for (int s = 0; s < kHEarly; ++s) load_h(s);
-  }
-
+      for (int s = 0; s < kHEarly; ++s) load_h(s);
+    }
+  };
 
   // the state the whole sequence starts from: only its first chunk needs it
   float seq_in[VEC];
@@ -163,6 +164,7 @@ __device__ __forceinline__ void scan_tile(const ScanArgs &p, const StateArgs<STA
     // the slice is the whole sequence: nothing to chain
 #pragma unroll
     for (int v = 0; v < VEC; ++v) state[v] = seq_in[v];
+    load_h_early();
   } else {
     // ---- phase 1b: the slice as an affine map ----------------------------------------
     float mA[VEC], mB[VEC];
@@ -181,7 +183,7 @@ __device__ __forceinline__ void scan_tile(const ScanArgs &p, const StateArgs<STA
       }
     }
     FSS_STAMP(c, p, 1);
-    chain_chunks<VEC>(p, c, mA, mB, STATE ? seq_in : nullptr, state);
+    chain_chunks<VEC>(p, c, mA, mB, STATE ? seq_in : nullptr, state, load_h_early);
   }
 
   // ---- phase 3: the recurrence from the true incoming state, in order ---------------
@@ -360,7 +362,7 @@ __device__ __forceinline__ void gated_tile(const ScanArgs &p, const TileCtx &c) 
 #pragma unroll
     for (int v = 0; v < VEC; ++v) state[v] = 0.0f;
   } else {
-    chain_chunks<VEC>(p, c, mA, mB, nullptr, state);
+    chain_chunks<VEC>(p, c, mA, mB, nullptr, state, [] {});
   }
 
   // ---- phase 3 -------------------------------------------------------------------------

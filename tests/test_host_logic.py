@@ -168,9 +168,9 @@ def test_planning_of_the_gated_fp16_and_channel_major_entry_points():
         return cfg.vec, cfg.steps, cfg.waves
 
     # gated: 4 bytes per lane; the backward holds four tensors, so never more than 16 steps
-    assert choose(_native.FSS_BF16, _native.FSS_GATED_FWD) == (2, 32, 4)
-    assert choose(_native.FSS_BF16, _native.FSS_GATED_BWD) == (2, 16, 8)
-    assert choose(_native.FSS_F32, _native.FSS_GATED_FWD) == (1, 32, 8)
+    assert choose(_native.FSS_BF16, _native.FSS_GATED_FWD) == (2, 32, 16)
+    assert choose(_native.FSS_BF16, _native.FSS_GATED_BWD) == (2, 16, 16)
+    assert choose(_native.FSS_F32, _native.FSS_GATED_FWD) == (1, 32, 16)
     assert choose(_native.FSS_F32, _native.FSS_GATED_BWD)[1] <= 16
     assert choose(_native.FSS_BF16, _native.FSS_GATED_BWD, (1, 65521, 256))[1] <= 16
     assert choose(_native.FSS_BF16, _native.FSS_GATED_BWD, (1, 1024, 1024)) == (1, 8, 8)
