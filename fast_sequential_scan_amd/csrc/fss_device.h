@@ -332,9 +332,7 @@ struct TileCtx {
   bool col_ok;           // the lane's channels exist (d % VEC == 0, so all or none)
   float2 *lds_map;       // [wave][v][lane] = (A, B) of this tile
   float2 *lds_pred;      // [look wave][v][lane] = what an earlier chunk offers
-  float *lds_hin;        // [v][lane] = the chunk's incoming state, for every wave to read
   uint32_t *s_kind;      // [look wave] kind of that offer
-  uint32_t *s_resolved;  // look-back finished (one word per workgroup)
 #ifdef FSS_TRACE
   int trace_wave;
 #endif
@@ -433,13 +431,18 @@ __device__ __forceinline__ void fold_wave_maps(const float2 *lds_map, int lane, 
 // Phase 2.  In: this wave's slice as the map x -> mA*x + mB.  Out: the state
 // entering the slice.  Every wave of the workgroup must call it (barriers).
 //
-// After one barrier every wave composes the maps of the waves before it (its state
-// is then one multiply-add away from the chunk's incoming state), and wave 0 composes
-// all of them into the chunk's map and publishes it.  Meanwhile wave w (w < look)
-// fetches what chunk-1-w offers - its outgoing state if it has one, else its map -
-// so a look-back over `look` chunks costs one memory round trip instead of one per
-// chunk; wave 0 folds what they found and hands the chunk's incoming state to all
-// waves through LDS.  Chains longer than `look` repeat the fetch.
+// After one barrier wave 0 composes all the waves' maps into the chunk's map and
+// publishes it.  Meanwhile wave w (w < look) fetches what chunk-1-w offers - its
+// outgoing state if it has one, else its map - so a look-back over `look` chunks
+// costs one memory round trip instead of one per chunk.  After a second barrier
+// every wave folds what the look-back waves found into the chunk's incoming state
+// itself (a few multiply-adds: cheaper than a third barrier and a broadcast), wave 0
+// also publishes the chunk's outgoing state, and every wave applies the composition
+// of the waves before it.  Chains longer than `look` repeat the fetch.
+//
+// `mid` is called once by every wave, by the look-back waves right after their first
+// fetch has been issued: loads it issues travel while the chain is resolved and
+// return after the fetch (loads return in issue order).
 template <int VEC, typename Mid>
 __device__ __forceinline__ void chain_chunks(const ScanArgs &p, const TileCtx &c, const float *mA,
                                              const float *mB, const float *seq_in, float *state, Mid &&mid) {

@@ -25,16 +25,15 @@ inline int64_t ceil_div(int64_t a, int64_t b) { return (a + b - 1) / b; }
 inline int max_vec_steps(int dtype) { return dtype != FSS_F32 ? 64 : 32; }  // vec*steps
 
 // LDS: one (A,B) slot per lane and vector element for every wave, twice (tiles
-// alternate between two sets), the same for every wave that looks back, and two
-// rows of incoming states.
+// alternate between two sets), and the same for every wave that looks back.
 constexpr size_t kLdsBudget = 60 * 1024;
 inline int look_waves(int waves, int vec) {
   int look = waves < kMaxLookWaves ? waves : kMaxLookWaves;
-  while (look > 1 && static_cast<size_t>(2 * waves + look + 1) * vec * 512 > kLdsBudget) --look;
+  while (look > 1 && static_cast<size_t>(2 * waves + look) * vec * 512 > kLdsBudget) --look;
   return look;
 }
 inline size_t lds_bytes(int waves, int vec) {
-  return static_cast<size_t>(2 * waves + look_waves(waves, vec) + 1) * vec * 512;
+  return static_cast<size_t>(2 * waves + look_waves(waves, vec)) * vec * 512;
 }
 
 inline bool config_valid(const fss_config &c, int dtype, bool gated = false, int dir = FSS_FWD) {

@@ -175,7 +175,6 @@ template <typename E, int VEC, int ROWS, bool BWD>
 __global__ __launch_bounds__(1024) void cm_scan_kernel(const ScanArgs p) {
   extern __shared__ float lds[];
   __shared__ uint32_t s_kind[kMaxLookWaves];
-  __shared__ uint32_t s_resolved;
 
   TileCtx c;
   c.lane = threadIdx.x & 63;
@@ -184,9 +183,7 @@ __global__ __launch_bounds__(1024) void cm_scan_kernel(const ScanArgs p) {
   c.look = p.look_waves;
   float2 *const lds_maps = reinterpret_cast<float2 *>(lds);  // laid out as in scan_kernel with one slot per lane
   c.lds_pred = lds_maps + 2 * c.n_waves * 64;
-  float *const lds_hins = reinterpret_cast<float *>(c.lds_pred + c.look * 64);
   c.s_kind = s_kind;
-  c.s_resolved = &s_resolved;
   c.seq = p.seq;
   c.row_bytes = 0;
   c.lane_off = 0;
@@ -201,7 +198,6 @@ __global__ __launch_bounds__(1024) void cm_scan_kernel(const ScanArgs p) {
   uint32_t parity = 0;
   for (uint32_t tile = blockIdx.x; tile < static_cast<uint32_t>(p.n_tiles); tile += gridDim.x, parity ^= 1u) {
     c.lds_map = lds_maps + parity * c.n_waves * 64;
-    c.lds_hin = lds_hins + parity * 64;
     const uint32_t chunk = __builtin_amdgcn_readfirstlane(tile / static_cast<uint32_t>(p.n_ctiles));
     const uint32_t ctile = tile - chunk * static_cast<uint32_t>(p.n_ctiles);
     c.chunk = static_cast<int>(chunk);

@@ -24,12 +24,14 @@
 //        the memory-level parallelism that fills HBM), then folds its slice into
 //        the affine map x -> A*x + B it applies to the incoming state;
 //     2. wave 0 composes the waves' maps through LDS and publishes the chunk's map;
-//        at the same time up to 8 waves each fetch what one earlier chunk of the
+//        at the same time up to 16 waves each fetch what one earlier chunk of the
 //        same channels offers (its outgoing state if it has one, else its map),
 //        so the look-back over the nearest chunks costs one memory round trip, not
 //        one per chunk (decoupled look-back over (A,B) pairs in global memory).
-//        Wave 0 folds what they found into the chunk's incoming state, publishes
-//        the outgoing state, and hands every wave its own incoming state via LDS;
+//        Every wave folds what they found into the chunk's incoming state and
+//        applies the maps of the waves before it; wave 0 publishes the outgoing
+//        state.  The backward issues the loads of its third tensor, which only
+//        phase 3 needs, inside this phase, behind the look-back's fetch;
 //     3. every lane re-runs the recurrence over its register-resident slice from
 //        its true incoming state, in sequential order, and stores the results.
 //   Because phase 3 restarts from the incoming state, only that state is
@@ -419,7 +421,6 @@ __global__ __launch_bounds__(1024) void scan_kernel(const ScanArgs p, const Stat
 
   extern __shared__ float lds[];
   __shared__ uint32_t s_kind[kMaxLookWaves];
-  __shared__ uint32_t s_resolved;
 
   TileCtx c;
   c.lane = threadIdx.x & 63;
@@ -428,12 +429,10 @@ __global__ __launch_bounds__(1024) void scan_kernel(const ScanArgs p, const Stat
   c.look = p.look_waves;
   // LDS: two sets of per-wave maps (tiles alternate between them, so a wave that runs
   // ahead into the next tile cannot overwrite a map a slower wave still reads), then
-  // the slots the look-back waves fill, then two rows for the chunk's incoming state
+  // the slots the look-back waves fill
   float2 *const lds_maps = reinterpret_cast<float2 *>(lds);
   c.lds_pred = lds_maps + 2 * c.n_waves * kLaneSlots;
-  float *const lds_hins = reinterpret_cast<float *>(c.lds_pred + c.look * kLaneSlots);
   c.s_kind = s_kind;
-  c.s_resolved = &s_resolved;
   c.seq = p.seq;
   c.row_bytes = p.d * E::kBytes;
   c.lane_off = static_cast<uint32_t>(c.lane * Row<E, VEC>::kBytes);
@@ -459,7 +458,6 @@ __global__ __launch_bounds__(1024) void scan_kernel(const ScanArgs p, const Stat
   uint32_t parity = 0;
   for (uint32_t tile = blockIdx.x; tile < static_cast<uint32_t>(p.n_tiles); tile += gridDim.x, parity ^= 1u) {
     c.lds_map = lds_maps + parity * c.n_waves * kLaneSlots;
-    c.lds_hin = lds_hins + parity * kLaneSlots;
     // unsigned, wave-uniform arithmetic: stays on the scalar unit
     // (the compiler divides through a vector-unit reciprocal: pin the quotients back)
     const uint32_t chunk = __builtin_amdgcn_readfirstlane(tile / static_cast<uint32_t>(p.n_ctiles));
