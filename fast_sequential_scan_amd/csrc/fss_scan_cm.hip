@@ -54,31 +54,41 @@ __device__ __forceinline__ void cm_tile(const ScanArgs &p, const TileCtx &c, int
     ok[r] = in_seq && row < n_rows;
     a[r].fill(1.0f);  // outside: identity steps
     b[r].fill(0.0f);
-    if (BWD) hp[r].fill(0.0f);
     if (ok[r]) {
       const int64_t off = (row * seq + t_base) * E::kBytes;
       a[r].template load<kNtA>(uniform_ptr((gcptr_t)p.in_a + off) + lane_off);
       b[r].template load<kNtB>(uniform_ptr((gcptr_t)p.in_b + off) + lane_off);
-      if (BWD) hp[r].template load<kNtH>(uniform_ptr((gcptr_t)p.in_h + off) + lane_off);
     }
   }
   if (BWD) {
-    // alpha[t_hi+1] for the first step and h[t_lo-1] for the last one: from the
-    // neighbouring lanes, except at the two ends of the wave's slice
+    // alpha[t_hi+1] for the first step: from the neighbouring lane, except at the end of
+    // the wave's slice
 #pragma unroll
     for (int r = 0; r < ROWS; ++r) {
-      const int64_t row = row0 + r;
-      OneT ea, eh;
+      OneT ea;
       ea.fill(0.0f);
-      eh.fill(0.0f);
-      if (lane == 0 && ok[r] && t_hi + 1 < seq) ea.load((gcptr_t)p.in_a + (row * seq + t_hi + 1) * E::kBytes);
-      if (lane == 63 && ok[r] && t_lo >= 1) eh.load((gcptr_t)p.in_h + (row * seq + t_lo - 1) * E::kBytes);
-      const float from_prev = __shfl_up(a[r].get(0), 1);        // lane-1 holds timesteps just above ours
-      const float from_next = __shfl_down(hp[r].get(VEC - 1), 1);  // lane+1 holds timesteps just below ours
+      if (lane == 0 && ok[r] && t_hi + 1 < seq) ea.load((gcptr_t)p.in_a + ((row0 + r) * seq + t_hi + 1) * E::kBytes);
+      const float from_prev = __shfl_up(a[r].get(0), 1);  // lane-1 holds timesteps just above ours
       edge_a[r] = lane == 0 ? ea.get(0) : from_prev;
-      edge_h[r] = lane == 63 ? eh.get(0) : from_next;
     }
   }
+  // The saved h only feeds phase 3: its loads go out inside the chain phase, behind the
+  // look-back's, and travel while the chain is resolved.
+  OneT eh[BWD ? ROWS : 1];
+  auto load_h = [&] {
+    if (BWD) {
+#pragma unroll
+      for (int r = 0; r < ROWS; ++r) {
+        eh[r].fill(0.0f);
+        hp[r].fill(0.0f);
+        if (ok[r]) {
+          const int64_t off = ((row0 + r) * seq + t_base) * E::kBytes;
+          hp[r].template load<kNtH>(uniform_ptr((gcptr_t)p.in_h + off) + lane_off);
+        }
+        if (lane == 63 && ok[r] && t_lo >= 1) eh[r].load((gcptr_t)p.in_h + ((row0 + r) * seq + t_lo - 1) * E::kBytes);
+      }
+    }
+  };
 
   // coefficient, addend and saved h of scan step j of row r
   auto coef = [&](int r, int j) -> float {
@@ -135,7 +145,18 @@ __device__ __forceinline__ void cm_tile(const ScanArgs &p, const TileCtx &c, int
   }
 
   float slice_in = 0.0f;
-  if (c.chained || c.n_waves > 1) chain_chunks<1>(p, c, &mA, &mB, nullptr, &slice_in, [] {});
+  if (c.chained || c.n_waves > 1)
+    chain_chunks<1>(p, c, &mA, &mB, nullptr, &slice_in, load_h);
+  else
+    load_h();
+  if (BWD) {
+    // h[t_lo-1] for the last step: from the neighbouring lane, except at the end of the slice
+#pragma unroll
+    for (int r = 0; r < ROWS; ++r) {
+      const float from_next = __shfl_down(hp[r].get(VEC - 1), 1);  // lane+1 holds timesteps just below ours
+      edge_h[r] = lane == 63 ? eh[r].get(0) : from_next;
+    }
+  }
 
   // ---- phase 3 ---------------------------------------------------------------------------
 #pragma unroll
