@@ -70,6 +70,14 @@ def parse_args():
     return ap.parse_args()
 
 
+def quantile_pair(samples):
+    """20th and 80th percentile, as the reference's benchmark reports them (benchmark.py:65)."""
+    if len(samples) < 2:
+        return [round(samples[0], 5)] * 2 if samples else None
+    q = statistics.quantiles(samples, n=5, method="inclusive")
+    return [round(q[0], 5), round(q[3], 5)]
+
+
 def main() -> int:
     args = parse_args()
     if args.gpus != 1:
@@ -435,6 +443,8 @@ def main() -> int:
         "bwd_ms": round(bwd_mean, 5),
         "fwd_ms_median": round(statistics.median(fwd_ms), 5),
         "bwd_ms_median": round(statistics.median(bwd_ms), 5),
+        "fwd_ms_p20_p80": quantile_pair(fwd_ms),
+        "bwd_ms_p20_p80": quantile_pair(bwd_ms),
         "algorithmic_bytes_per_step": step_bytes,
         "event_sampled_steps": len(sampled),
         "event_pair_overhead_ms": round(event_overhead, 5),
