@@ -291,19 +291,36 @@ struct StateArgs<false> {
 
 // ---- the kernel ----------------------------------------------------------------
 
-// Which streams are accessed non-temporally (bit 0: alpha, 1: beta/dout, 2: saved h,
-// 3: h output of the forward, 4: gradient outputs of the backward).  Measured on
-// MI355X at bs8 seq4096 d1024, forward and backward alternating: marking the
-// three output streams and the backward's reads of h non-temporal takes the step
-// from 134 us to 113 us; marking the reads of alpha, beta or dout as well is slower.
+// Which streams are accessed non-temporally (bit 0: alpha in the forward, 1: beta,
+// 2: the saved h in the backward, 3: the forward's output h, 4: the backward's two
+// gradient outputs, 5: alpha in the backward, 6: dout).  Measured on MI355X at bs8
+// seq4096 d1024 with 16-wave workgroups, forward and backward alternating on one set
+// of tensors (the way the reference benchmarks): no hints 115 us per step; hints on the
+// three output streams and on the backward's reads of h (their last use) 94 us; hints
+// on the reads of alpha, beta or dout as well 96-105 us.  With nothing cached between
+// launches (eight sets of tensors in rotation) the same settings read 114 / 113 /
+// 106-108 us: hints on the input reads would be worth 5 % there and cost up to 15 % in
+// the first setting.
 #ifndef FSS_NT_MASK
 #define FSS_NT_MASK 28
 #endif
-constexpr bool kNtA = (FSS_NT_MASK & 1) != 0;
-constexpr bool kNtB = (FSS_NT_MASK & 2) != 0;
+constexpr bool kNtAFwd = (FSS_NT_MASK & 1) != 0;
+constexpr bool kNtBFwd = (FSS_NT_MASK & 2) != 0;
+constexpr bool kNtABwd = (FSS_NT_MASK & 32) != 0;
+constexpr bool kNtBBwd = (FSS_NT_MASK & 64) != 0;
 constexpr bool kNtH = (FSS_NT_MASK & 4) != 0;
 constexpr bool kNtOutFwd = (FSS_NT_MASK & 8) != 0;
 constexpr bool kNtOutBwd = (FSS_NT_MASK & 16) != 0;
+
+// The forward's output is the one stream with a reader waiting: the next kernel of any
+// pipeline, or the backward in a benchmark loop.  A small h is therefore stored without
+// the hint and found in the 256 MiB memory-side cache by its reader (forward and backward
+// alternating, bf16: bs16 seq2048 d512 52.4 -> 49.0 us per step, bs8 seq3000 d1024
+// 74.0 -> 69.8 us).  "Small" means that h and the three inputs of such a step fill at
+// most three quarters of that cache; at bs8 seq4096 d1024 (4 x 64 MiB, all of it) the
+// same change read -4 us or +4 us depending on where the tensors happened to lie, and
+// a larger h only pushes the inputs out (bs8 seq8192: the forward on its own 69 -> 89 us).
+constexpr int64_t kKeepOutBytes = static_cast<int64_t>(48) << 20;
 
 #ifdef FSS_TRACE
 #define FSS_STAMP(c, p, slot)                                                                   \

@@ -56,8 +56,8 @@ __device__ __forceinline__ void cm_tile(const ScanArgs &p, const TileCtx &c, int
     b[r].fill(0.0f);
     if (ok[r]) {
       const int64_t off = (row * seq + t_base) * E::kBytes;
-      a[r].template load<kNtA>(uniform_ptr((gcptr_t)p.in_a + off) + lane_off);
-      b[r].template load<kNtB>(uniform_ptr((gcptr_t)p.in_b + off) + lane_off);
+      a[r].template load<(BWD ? kNtABwd : kNtAFwd)>(uniform_ptr((gcptr_t)p.in_a + off) + lane_off);
+      b[r].template load<(BWD ? kNtBBwd : kNtBFwd)>(uniform_ptr((gcptr_t)p.in_b + off) + lane_off);
     }
   }
   if (BWD) {

@@ -79,7 +79,7 @@ namespace fss {
 // interior and every lane has channels, so nothing is predicated; otherwise every
 // access is guarded.  The two variants share no registers, so the guarded one
 // costs the fast one nothing.
-template <typename E, int VEC, int STEPS, bool BWD, bool STATE, bool FULL>
+template <typename E, int VEC, int STEPS, bool BWD, bool STATE, bool FULL, bool KEEP>
 __device__ __forceinline__ void scan_tile(const ScanArgs &p, const StateArgs<STATE> &st, const TileCtx &c) {
   using RowT = Row<E, VEC>;
   const int64_t seq = c.seq, row_bytes = c.row_bytes, r0 = c.r0;
@@ -104,8 +104,8 @@ __device__ __forceinline__ void scan_tile(const ScanArgs &p, const StateArgs<STA
       // below, whatever is loaded here.  The backward would find it one row past the end
       // of the sequence, so it loads the row before instead.
       const int row = (BWD && s == 0 && r0 == 0) ? 1 : s;
-      a[s].template load<kNtA>(uniform_ptr(pa + row * step_bytes) + lane_off);
-      b[s].template load<kNtB>(uniform_ptr(pb + s * step_bytes) + lane_off);
+      a[s].template load<(BWD ? kNtABwd : kNtAFwd)>(uniform_ptr(pa + row * step_bytes) + lane_off);
+      b[s].template load<(BWD ? kNtBBwd : kNtBFwd)>(uniform_ptr(pb + s * step_bytes) + lane_off);
     } else {
       const int64_t r = r0 + s;
       // Outside the sequence the step is the identity map (a=1, b=0).  The first step
@@ -115,8 +115,8 @@ __device__ __forceinline__ void scan_tile(const ScanArgs &p, const StateArgs<STA
       b[s].fill(0.0f);
       if (c.col_ok && r < seq) {
         if (r >= 1 || (STATE && !BWD && st.state_in))
-          a[s].template load<kNtA>(uniform_ptr(pa + s * step_bytes) + lane_off);
-        b[s].template load<kNtB>(uniform_ptr(pb + s * step_bytes) + lane_off);
+          a[s].template load<(BWD ? kNtABwd : kNtAFwd)>(uniform_ptr(pa + s * step_bytes) + lane_off);
+        b[s].template load<(BWD ? kNtBBwd : kNtBFwd)>(uniform_ptr(pb + s * step_bytes) + lane_off);
       }
     }
   }
@@ -209,7 +209,7 @@ __device__ __forceinline__ void scan_tile(const ScanArgs &p, const StateArgs<STA
     if (FULL || (c.col_ok && r < seq)) {
       RowT o;
       o.pack(state);
-      o.template store<(BWD ? kNtOutBwd : kNtOutFwd)>(uniform_ptr(po0 + s * step_bytes) + lane_off);
+      o.template store<(BWD ? kNtOutBwd : (kNtOutFwd && !KEEP))>(uniform_ptr(po0 + s * step_bytes) + lane_off);
       if (BWD) {
         if (!FULL && r == seq - 1) {  // t = 0: grad_alpha[0] = g[0] * h[-1], 0 in the plain scan
 #pragma unroll
@@ -286,10 +286,10 @@ __device__ __forceinline__ void gated_tile(const ScanArgs &p, const TileCtx &c) 
     // the gate row of a[s] exists: forward r < seq; backward 1 <= r <= seq
     const bool a_ok = FULL || (c.col_ok && (BWD ? (r >= 1 && r <= seq) : (r < seq)));
     if (!FULL) a[s].fill(0.0f);
-    if (a_ok) a[s].template load<kNtA>(uniform_ptr(pa + s * step_bytes) + lane_off);
+    if (a_ok) a[s].template load<(BWD ? kNtABwd : kNtAFwd)>(uniform_ptr(pa + s * step_bytes) + lane_off);
     if (s < STEPS) {
       if (!FULL) b[s].fill(0.0f);
-      if (FULL || (c.col_ok && r < seq)) b[s].template load<kNtB>(uniform_ptr(pb + s * step_bytes) + lane_off);
+      if (FULL || (c.col_ok && r < seq)) b[s].template load<(BWD ? kNtBBwd : kNtBFwd)>(uniform_ptr(pb + s * step_bytes) + lane_off);
     }
   }
   // x and the saved h only feed phase 3 of the backward: half of their rows now, the
@@ -415,7 +415,8 @@ __device__ __forceinline__ void gated_tile(const ScanArgs &p, const TileCtx &c) 
 
 // STATE: the variant that honours the optional incoming/outgoing state rows of ScanArgs;
 // the plain scan is compiled without them.  GATED: the gated scan (never with STATE).
-template <typename E, int VEC, int STEPS, bool BWD, bool STATE, bool GATED = false>
+// KEEP: the plain forward for small outputs, which stores h without the non-temporal hint.
+template <typename E, int VEC, int STEPS, bool BWD, bool STATE, bool GATED = false, bool KEEP = false>
 __global__ __launch_bounds__(1024) void scan_kernel(const ScanArgs p, const StateArgs<STATE> st) {
   constexpr int kLaneSlots = 64 * VEC;  // channels per tile
 
@@ -487,9 +488,9 @@ __global__ __launch_bounds__(1024) void scan_kernel(const ScanArgs p, const Stat
         gated_tile<E, VEC, STEPS, BWD, false>(p, c);
     } else {
       if (full)
-        scan_tile<E, VEC, STEPS, BWD, STATE, true>(p, st, c);
+        scan_tile<E, VEC, STEPS, BWD, STATE, true, KEEP>(p, st, c);
       else
-        scan_tile<E, VEC, STEPS, BWD, STATE, false>(p, st, c);
+        scan_tile<E, VEC, STEPS, BWD, STATE, false, KEEP>(p, st, c);
     }
   }
 
@@ -501,7 +502,7 @@ __global__ __launch_bounds__(1024) void scan_kernel(const ScanArgs p, const Stat
 
 // ---- launching ---------------------------------------------------------------------
 
-template <typename E, int VEC, int STEPS, bool BWD, bool STATE, bool GATED = false>
+template <typename E, int VEC, int STEPS, bool BWD, bool STATE, bool GATED = false, bool KEEP = false>
 int launch_one(const ScanArgs &args, const StateArgs<true> &state, const Plan &pl, hipStream_t stream) {
   // The kernel's waits are only safe if every workgroup of the grid is resident,
   // so the grid never exceeds what the device holds at once; workgroups loop.
@@ -510,7 +511,7 @@ int launch_one(const ScanArgs &args, const StateArgs<true> &state, const Plan &p
   const size_t lds = lds_bytes(waves, VEC);
   int fit = __atomic_load_n(&resident[waves], __ATOMIC_RELAXED);
   if (fit == 0) {
-    fit = resident_workgroups(scan_kernel<E, VEC, STEPS, BWD, STATE, GATED>, waves, lds);
+    fit = resident_workgroups(scan_kernel<E, VEC, STEPS, BWD, STATE, GATED, KEEP>, waves, lds);
     if (fit <= 0) return FSS_ERR_LAUNCH;
     __atomic_store_n(&resident[waves], fit, __ATOMIC_RELAXED);
   }
@@ -520,7 +521,7 @@ int launch_one(const ScanArgs &args, const StateArgs<true> &state, const Plan &p
   const dim3 block(static_cast<uint32_t>(waves) * 64);
   StateArgs<STATE> st;
   if constexpr (STATE) st = state;
-  hipLaunchKernelGGL((scan_kernel<E, VEC, STEPS, BWD, STATE, GATED>), grid, block, lds, stream, args, st);
+  hipLaunchKernelGGL((scan_kernel<E, VEC, STEPS, BWD, STATE, GATED, KEEP>), grid, block, lds, stream, args, st);
   const hipError_t e = hipGetLastError();
   if (e != hipSuccess) {
     tls_hip_error = static_cast<int>(e);
@@ -534,8 +535,11 @@ int launch_typed(const ScanArgs &args, const StateArgs<true> &state, const Plan 
   constexpr bool is_16bit = E::kBytes == 2;
   const int key = pl.cfg.vec * 100 + pl.cfg.steps;
   switch (key) {
-#define FSS_CASE(V, S) \
-  case V * 100 + S:    \
+#define FSS_CASE(V, S)                                                                            \
+  case V * 100 + S:                                                                               \
+    if constexpr (!BWD && !STATE) {                                                               \
+      if (pl.keep_out) return launch_one<E, V, S, BWD, STATE, false, true>(args, state, pl, stream); \
+    }                                                                                             \
     return launch_one<E, V, S, BWD, STATE>(args, state, pl, stream);
     FSS_CASE(1, 8)
     FSS_CASE(1, 16)
