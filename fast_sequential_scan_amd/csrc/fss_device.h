@@ -350,6 +350,7 @@ struct TileCtx {
   float2 *lds_map;       // [wave][v][lane] = (A, B) of this tile
   float2 *lds_pred;      // [look wave][v][lane] = what an earlier chunk offers
   uint32_t *s_kind;      // [look wave] kind of that offer
+  int span;              // chunks one look-back wave covers: more than 1 when the sequence has more chunks than such waves
 #ifdef FSS_TRACE
   int trace_wave;
 #endif
@@ -517,7 +518,7 @@ __device__ __forceinline__ void chain_chunks(const ScanArgs &p, const TileCtx &c
   int nearest = c.chunk - 1;  // nearest earlier chunk not folded yet
   bool first = true;
   for (;;) {
-    const int j = nearest - wave;
+    const int j = nearest - wave * c.span;
     if (wave < c.look && j >= 0) {
       float qA[VEC], qB[VEC];
       uint32_t polls = 0;
@@ -535,6 +536,28 @@ __device__ __forceinline__ void chain_chunks(const ScanArgs &p, const TileCtx &c
         }
         __builtin_amdgcn_s_sleep(2);
       }
+      // long chains: the wave also takes the chunks before that one (by now they have nearly
+      // always published), so that one round of the look-back reaches `span` times as far
+      for (int k = 1; k < c.span && kind == kPredMap && j - k >= 0; ++k) {
+        float rA[VEC], rB[VEC];
+        polls = 0;
+        while ((kind = poll_chunk<VEC>(p, c, j - k, rA, rB)) == kPredNone) {
+          if (++polls > kSpinLimit) {
+            if (lane == 0) st_u32(p.hdr + HDR_ERROR, 1u);
+            kind = kPredState;
+#pragma unroll
+            for (int v = 0; v < VEC; ++v) rA[v] = rB[v] = 0.0f;
+            break;
+          }
+          __builtin_amdgcn_s_sleep(2);
+        }
+        // (a state is the map x -> 0*x + value)
+#pragma unroll
+        for (int v = 0; v < VEC; ++v) {
+          qB[v] = __builtin_fmaf(qA[v], rB[v], qB[v]);
+          qA[v] *= rA[v];
+        }
+      }
 #pragma unroll
       for (int v = 0; v < VEC; ++v) c.lds_pred[(wave * VEC + v) * 64 + lane] = make_float2(qA[v], qB[v]);
       if (lane == 0) c.s_kind[wave] = kind;
@@ -546,7 +569,7 @@ __device__ __forceinline__ void chain_chunks(const ScanArgs &p, const TileCtx &c
     // every wave folds what the look-back waves found (the same few LDS reads in each wave
     // cost less than a second barrier and a broadcast by wave 0)
     bool resolved = false;
-    for (int w = 0; w < c.look && nearest - w >= 0 && !resolved; ++w) {
+    for (int w = 0; w < c.look && nearest - w * c.span >= 0 && !resolved; ++w) {
       const bool is_state = c.s_kind[w] == kPredState;
 #pragma unroll
       for (int v = 0; v < VEC; ++v) {
@@ -568,7 +591,7 @@ __device__ __forceinline__ void chain_chunks(const ScanArgs &p, const TileCtx &c
       }
       break;
     }
-    nearest -= c.look;
+    nearest -= c.look * c.span;
     if (nearest < 0) {  // cannot happen; never spin on a logic error
       if (threadIdx.x == 0) st_u32(p.hdr + HDR_ERROR, 1u);
       break;

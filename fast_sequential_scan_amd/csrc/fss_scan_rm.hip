@@ -428,6 +428,11 @@ __global__ __launch_bounds__(1024) void scan_kernel(const ScanArgs p, const Stat
   c.wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   c.n_waves = blockDim.x >> 6;
   c.look = p.look_waves;
+#ifndef FSS_MAX_SPAN
+#define FSS_MAX_SPAN 4
+#endif
+  c.span = (p.n_chunks + p.look_waves - 1) / p.look_waves;
+  if (c.span > FSS_MAX_SPAN) c.span = FSS_MAX_SPAN;
   // LDS: two sets of per-wave maps (tiles alternate between them, so a wave that runs
   // ahead into the next tile cannot overwrite a map a slower wave still reads), then
   // the slots the look-back waves fill
