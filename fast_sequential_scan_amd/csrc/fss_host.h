@@ -94,11 +94,8 @@ inline void complete_config(fss_config &c, int64_t bs, int64_t seq, int64_t d, i
   } else if (!gated) {
     // 32-step slices would cost the backward a dozen spilled registers per lane
     if (narrow) {
-      // one or two column tiles and hundreds of chunks: here the spills of 32-step slices are
-      // the lesser evil (bs1 seq65521 d256: 42 against 49 us)
-      if (seq > 49152 && bs * d <= 256) rung(1, 32, 8, 0);
       rung(2, 16, 16);
-      if (seq >= 4096) rung(1, 16, 16); else rung(2, 16, 8);
+      if (seq >= 16384) rung(1, 16, 16); else rung(2, 16, 8);
       if (seq > 256) rung(1, 16, 8); else rung(2, 8, 8);
     } else {
       if (wide32) rung(2, 8, 16);
