@@ -121,7 +121,7 @@ inline void complete_config(fss_config &c, int64_t bs, int64_t seq, int64_t d, i
     if (narrow) {
       if (seq > 256) rung(2, 16, 16); else rung(2, 16, 8, 1024);
       rung(2, 8, 16);
-      if (seq < 2048) rung(2, 8, 8); else rung(1, 8, 16);
+      rung(2, 8, 8);
       if (seq <= 256) rung(2, 8, 8, 1);
       rung(1, 8, 8, 0);
     } else {
@@ -142,6 +142,15 @@ inline void complete_config(fss_config &c, int64_t bs, int64_t seq, int64_t d, i
     while (!c.waves && w > 1 && lds_bytes(w, v) > kLdsBudget) --w;
     pick = fss_config{v, s, w, 0};
     if (bs * ceil_div(d, 64 * static_cast<int64_t>(v)) * ceil_div(seq, static_cast<int64_t>(s) * w) >= ladder[i].need) break;
+  }
+  // Forward, 16-wave workgroups (one per CU) whose last round would leave CUs idle: the same
+  // tile shape as two 8-wave workgroups per CU spreads that round over all CUs (7-18 % on 59
+  // shapes with sequence lengths and widths that are no powers of two; the backward, already two
+  // tiles per CU and round at the sizes that matter, gains nothing).
+  if (fwd && !c.waves && pick.waves == 16) {
+    const int64_t tiles = bs * ceil_div(d, 64 * static_cast<int64_t>(pick.vec)) * ceil_div(seq, static_cast<int64_t>(pick.steps) * 16);
+    const int64_t rounds = ceil_div(tiles, 256);
+    if (rounds >= 2 && tiles * 10 < rounds * 256 * 9) pick.waves = 8;
   }
   c.vec = pick.vec;
   c.steps = pick.steps;
