@@ -68,7 +68,8 @@ int run_scan(int dtype, int dir, const void *alpha, const void *in_b, const void
   args.n_chunks = static_cast<int32_t>(pl.n_chunks);
   args.n_tiles = static_cast<int32_t>(pl.n_tiles);
   args.look_waves = look_waves(pl.cfg.waves, pl.cfg.vec);
-  pl.keep_out = !gated && dir == FSS_FWD && bs * seq * d * static_cast<int64_t>(esize) <= kKeepOutBytes;
+  const int64_t tensor_bytes = bs * seq * d * static_cast<int64_t>(esize);
+  pl.alt_policy = !gated && (dir == FSS_FWD ? tensor_bytes <= kKeepOutBytes : tensor_bytes > kStreamDoutBytes);
   const StateArgs<true> state = {state_in, state_out, h_before};
   args.hdr = static_cast<uint32_t *>(workspace);
   args.words = workspace ? reinterpret_cast<uint64_t *>(static_cast<char *>(workspace) + kHeaderBytes) : nullptr;

@@ -322,6 +322,15 @@ constexpr bool kNtOutBwd = (FSS_NT_MASK & 16) != 0;
 // a larger h only pushes the inputs out (bs8 seq8192: the forward on its own 69 -> 89 us).
 constexpr int64_t kKeepOutBytes = static_cast<int64_t>(48) << 20;
 
+// dout is read once per step.  While the three inputs of a step (alpha, h or beta, dout)
+// fit the memory-side cache together, a benchmark loop over one set of tensors finds it
+// there again and a hint on its reads costs 4 % (bs8 seq4096 d1024 bf16, 64 MiB per
+// tensor: 93.6 -> 97.3 us per step); beyond that the hint keeps dout from evicting alpha,
+// which the backward reads a second time (128 MiB per tensor: bs8 seq8192 d1024
+// 201.7 -> 192.6 us, fp32 at seq4096 194.4 -> 182.3 us).  With nothing cached between
+// launches the hint is worth 5 % at any size.
+constexpr int64_t kStreamDoutBytes = static_cast<int64_t>(80) << 20;
+
 #ifdef FSS_TRACE
 #define FSS_STAMP(c, p, slot)                                                                   \
   do {                                                                                          \

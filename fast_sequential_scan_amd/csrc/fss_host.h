@@ -159,7 +159,7 @@ inline void complete_config(fss_config &c, int64_t bs, int64_t seq, int64_t d, i
 
 struct Plan {
   fss_config cfg;
-  bool keep_out = false;  // plain forward: the output is small enough to be left in the memory-side cache
+  bool alt_policy = false;  // plain scan: the other cache policy (see kKeepOutBytes, kStreamDoutBytes)
   int64_t tiles_per_row, n_ctiles, n_chunks, n_tiles;
   size_t ws_bytes;
 };

@@ -79,7 +79,7 @@ namespace fss {
 // interior and every lane has channels, so nothing is predicated; otherwise every
 // access is guarded.  The two variants share no registers, so the guarded one
 // costs the fast one nothing.
-template <typename E, int VEC, int STEPS, bool BWD, bool STATE, bool FULL, bool KEEP>
+template <typename E, int VEC, int STEPS, bool BWD, bool STATE, bool FULL, bool ALT>
 __device__ __forceinline__ void scan_tile(const ScanArgs &p, const StateArgs<STATE> &st, const TileCtx &c) {
   using RowT = Row<E, VEC>;
   const int64_t seq = c.seq, row_bytes = c.row_bytes, r0 = c.r0;
@@ -105,7 +105,7 @@ __device__ __forceinline__ void scan_tile(const ScanArgs &p, const StateArgs<STA
       // of the sequence, so it loads the row before instead.
       const int row = (BWD && s == 0 && r0 == 0) ? 1 : s;
       a[s].template load<(BWD ? kNtABwd : kNtAFwd)>(uniform_ptr(pa + row * step_bytes) + lane_off);
-      b[s].template load<(BWD ? kNtBBwd : kNtBFwd)>(uniform_ptr(pb + s * step_bytes) + lane_off);
+      b[s].template load<(BWD ? (kNtBBwd || ALT) : kNtBFwd)>(uniform_ptr(pb + s * step_bytes) + lane_off);
     } else {
       const int64_t r = r0 + s;
       // Outside the sequence the step is the identity map (a=1, b=0).  The first step
@@ -116,7 +116,7 @@ __device__ __forceinline__ void scan_tile(const ScanArgs &p, const StateArgs<STA
       if (c.col_ok && r < seq) {
         if (r >= 1 || (STATE && !BWD && st.state_in))
           a[s].template load<(BWD ? kNtABwd : kNtAFwd)>(uniform_ptr(pa + s * step_bytes) + lane_off);
-        b[s].template load<(BWD ? kNtBBwd : kNtBFwd)>(uniform_ptr(pb + s * step_bytes) + lane_off);
+        b[s].template load<(BWD ? (kNtBBwd || ALT) : kNtBFwd)>(uniform_ptr(pb + s * step_bytes) + lane_off);
       }
     }
   }
@@ -209,7 +209,7 @@ __device__ __forceinline__ void scan_tile(const ScanArgs &p, const StateArgs<STA
     if (FULL || (c.col_ok && r < seq)) {
       RowT o;
       o.pack(state);
-      o.template store<(BWD ? kNtOutBwd : (kNtOutFwd && !KEEP))>(uniform_ptr(po0 + s * step_bytes) + lane_off);
+      o.template store<(BWD ? kNtOutBwd : (kNtOutFwd && !ALT))>(uniform_ptr(po0 + s * step_bytes) + lane_off);
       if (BWD) {
         if (!FULL && r == seq - 1) {  // t = 0: grad_alpha[0] = g[0] * h[-1], 0 in the plain scan
 #pragma unroll
@@ -415,8 +415,9 @@ __device__ __forceinline__ void gated_tile(const ScanArgs &p, const TileCtx &c) 
 
 // STATE: the variant that honours the optional incoming/outgoing state rows of ScanArgs;
 // the plain scan is compiled without them.  GATED: the gated scan (never with STATE).
-// KEEP: the plain forward for small outputs, which stores h without the non-temporal hint.
-template <typename E, int VEC, int STEPS, bool BWD, bool STATE, bool GATED = false, bool KEEP = false>
+// ALT: the other cache policy of the plain scan - the forward for small outputs, which stores h
+// without the non-temporal hint; the backward for large tensors, which reads dout with it.
+template <typename E, int VEC, int STEPS, bool BWD, bool STATE, bool GATED = false, bool ALT = false>
 __global__ __launch_bounds__(1024) void scan_kernel(const ScanArgs p, const StateArgs<STATE> st) {
   constexpr int kLaneSlots = 64 * VEC;  // channels per tile
 
@@ -493,9 +494,9 @@ __global__ __launch_bounds__(1024) void scan_kernel(const ScanArgs p, const Stat
         gated_tile<E, VEC, STEPS, BWD, false>(p, c);
     } else {
       if (full)
-        scan_tile<E, VEC, STEPS, BWD, STATE, true, KEEP>(p, st, c);
+        scan_tile<E, VEC, STEPS, BWD, STATE, true, ALT>(p, st, c);
       else
-        scan_tile<E, VEC, STEPS, BWD, STATE, false, KEEP>(p, st, c);
+        scan_tile<E, VEC, STEPS, BWD, STATE, false, ALT>(p, st, c);
     }
   }
 
@@ -507,7 +508,7 @@ __global__ __launch_bounds__(1024) void scan_kernel(const ScanArgs p, const Stat
 
 // ---- launching ---------------------------------------------------------------------
 
-template <typename E, int VEC, int STEPS, bool BWD, bool STATE, bool GATED = false, bool KEEP = false>
+template <typename E, int VEC, int STEPS, bool BWD, bool STATE, bool GATED = false, bool ALT = false>
 int launch_one(const ScanArgs &args, const StateArgs<true> &state, const Plan &pl, hipStream_t stream) {
   // The kernel's waits are only safe if every workgroup of the grid is resident,
   // so the grid never exceeds what the device holds at once; workgroups loop.
@@ -516,7 +517,7 @@ int launch_one(const ScanArgs &args, const StateArgs<true> &state, const Plan &p
   const size_t lds = lds_bytes(waves, VEC);
   int fit = __atomic_load_n(&resident[waves], __ATOMIC_RELAXED);
   if (fit == 0) {
-    fit = resident_workgroups(scan_kernel<E, VEC, STEPS, BWD, STATE, GATED, KEEP>, waves, lds);
+    fit = resident_workgroups(scan_kernel<E, VEC, STEPS, BWD, STATE, GATED, ALT>, waves, lds);
     if (fit <= 0) return FSS_ERR_LAUNCH;
     __atomic_store_n(&resident[waves], fit, __ATOMIC_RELAXED);
   }
@@ -526,7 +527,7 @@ int launch_one(const ScanArgs &args, const StateArgs<true> &state, const Plan &p
   const dim3 block(static_cast<uint32_t>(waves) * 64);
   StateArgs<STATE> st;
   if constexpr (STATE) st = state;
-  hipLaunchKernelGGL((scan_kernel<E, VEC, STEPS, BWD, STATE, GATED, KEEP>), grid, block, lds, stream, args, st);
+  hipLaunchKernelGGL((scan_kernel<E, VEC, STEPS, BWD, STATE, GATED, ALT>), grid, block, lds, stream, args, st);
   const hipError_t e = hipGetLastError();
   if (e != hipSuccess) {
     tls_hip_error = static_cast<int>(e);
@@ -542,8 +543,8 @@ int launch_typed(const ScanArgs &args, const StateArgs<true> &state, const Plan 
   switch (key) {
 #define FSS_CASE(V, S)                                                                            \
   case V * 100 + S:                                                                               \
-    if constexpr (!BWD && !STATE) {                                                               \
-      if (pl.keep_out) return launch_one<E, V, S, BWD, STATE, false, true>(args, state, pl, stream); \
+    if constexpr (!STATE) {                                                                       \
+      if (pl.alt_policy) return launch_one<E, V, S, BWD, STATE, false, true>(args, state, pl, stream); \
     }                                                                                             \
     return launch_one<E, V, S, BWD, STATE>(args, state, pl, stream);
     FSS_CASE(1, 8)
