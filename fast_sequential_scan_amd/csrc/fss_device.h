@@ -467,10 +467,10 @@ __device__ __forceinline__ void fold_wave_maps(const float2 *lds_map, int lane, 
 // also publishes the chunk's outgoing state, and every wave applies the composition
 // of the waves before it.  Chains longer than `look` repeat the fetch.
 //
-// `mid` is called once by every wave, by the look-back waves right after their first
-// fetch has been issued: loads it issues travel while the chain is resolved and
+// `mid` (only with HAS_MID) is called once by every wave, by the look-back waves right after their
+// first fetch has been issued: loads it issues travel while the chain is resolved and
 // return after the fetch (loads return in issue order).
-template <int VEC, typename Mid>
+template <int VEC, bool HAS_MID, typename Mid>
 __device__ __forceinline__ void chain_chunks(const ScanArgs &p, const TileCtx &c, const float *mA,
                                              const float *mB, const float *seq_in, float *state, Mid &&mid) {
   constexpr int kLaneSlots = 64 * VEC;
@@ -500,7 +500,7 @@ __device__ __forceinline__ void chain_chunks(const ScanArgs &p, const TileCtx &c
   // (pA, pB): what the waves before this one do to the chunk's incoming state
   float pA[VEC], pB[VEC];
   if (!look_back) {
-    mid();
+    if constexpr (HAS_MID) mid();
     fold_wave_maps<VEC>(c.lds_map, lane, wave, pA, pB);
   }
 
@@ -525,16 +525,35 @@ __device__ __forceinline__ void chain_chunks(const ScanArgs &p, const TileCtx &c
     accB[v] = hin[v] = 0.0f;
   }
   int nearest = c.chunk - 1;  // nearest earlier chunk not folded yet
-  bool first = true;
+  // The first look goes out ahead of the loop, with `mid` in a straight line between the
+  // issue of its loads and their use: only so does the compiler wait for exactly those
+  // loads and not for the ones `mid` has issued behind them.
+  uint32_t kind0 = kPredNone;
+  float q0A[VEC], q0B[VEC];
+#pragma unroll
+  for (int v = 0; v < VEC; ++v) q0A[v] = q0B[v] = 0.0f;
+  if constexpr (HAS_MID) {
+    if (wave < c.look && nearest - wave * c.span >= 0) {
+      ChunkWords<VEC> w;
+      poll_issue<VEC>(p, c, nearest - wave * c.span, w);
+      mid();
+      kind0 = poll_eval<VEC>(c, nearest - wave * c.span, w, q0A, q0B);
+    } else {
+      mid();
+    }
+  }
   for (;;) {
     const int j = nearest - wave * c.span;
     if (wave < c.look && j >= 0) {
       float qA[VEC], qB[VEC];
       uint32_t polls = 0;
-      ChunkWords<VEC> w;
-      poll_issue<VEC>(p, c, j, w);
-      if (first) mid();  // behind the look's loads, so that those return first
-      uint32_t kind = poll_eval<VEC>(c, j, w, qA, qB);
+      uint32_t kind = kind0;  // what the first look found (nothing, in later rounds)
+#pragma unroll
+      for (int v = 0; v < VEC; ++v) {
+        qA[v] = q0A[v];
+        qB[v] = q0B[v];
+      }
+      kind0 = kPredNone;
       while (kind == kPredNone && (kind = poll_chunk<VEC>(p, c, j, qA, qB)) == kPredNone) {
         if (++polls > kSpinLimit) {
           if (lane == 0) st_u32(p.hdr + HDR_ERROR, 1u);
@@ -570,10 +589,7 @@ __device__ __forceinline__ void chain_chunks(const ScanArgs &p, const TileCtx &c
 #pragma unroll
       for (int v = 0; v < VEC; ++v) c.lds_pred[(wave * VEC + v) * 64 + lane] = make_float2(qA[v], qB[v]);
       if (lane == 0) c.s_kind[wave] = kind;
-    } else if (first) {
-      mid();
     }
-    first = false;
     __syncthreads();
     // every wave folds what the look-back waves found (the same few LDS reads in each wave
     // cost less than a second barrier and a broadcast by wave 0)

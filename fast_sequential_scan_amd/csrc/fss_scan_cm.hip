@@ -146,7 +146,7 @@ __device__ __forceinline__ void cm_tile(const ScanArgs &p, const TileCtx &c, int
 
   float slice_in = 0.0f;
   if (c.chained || c.n_waves > 1)
-    chain_chunks<1>(p, c, &mA, &mB, nullptr, &slice_in, load_h);
+    chain_chunks<1, BWD>(p, c, &mA, &mB, nullptr, &slice_in, load_h);
   else
     load_h();
   if (BWD) {

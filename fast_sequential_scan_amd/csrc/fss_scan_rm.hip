@@ -185,7 +185,7 @@ __device__ __forceinline__ void scan_tile(const ScanArgs &p, const StateArgs<STA
       }
     }
     FSS_STAMP(c, p, 1);
-    chain_chunks<VEC>(p, c, mA, mB, STATE ? seq_in : nullptr, state, load_h_early);
+    chain_chunks<VEC, BWD>(p, c, mA, mB, STATE ? seq_in : nullptr, state, load_h_early);
   }
 
   // ---- phase 3: the recurrence from the true incoming state, in order ---------------
@@ -364,7 +364,7 @@ __device__ __forceinline__ void gated_tile(const ScanArgs &p, const TileCtx &c) 
 #pragma unroll
     for (int v = 0; v < VEC; ++v) state[v] = 0.0f;
   } else {
-    chain_chunks<VEC>(p, c, mA, mB, nullptr, state, [] {});
+    chain_chunks<VEC, false>(p, c, mA, mB, nullptr, state, [] {});
   }
 
   // ---- phase 3 -------------------------------------------------------------------------
