@@ -38,6 +38,8 @@ EXPORTED_SYMBOLS = (
     "fss_scan_bwd_state",
     "fss_gated_scan_fwd",
     "fss_gated_scan_bwd",
+    "fss_gated_scan_fwd_state",
+    "fss_gated_scan_bwd_state",
     "fss_cm_workspace_bytes",
     "fss_scan_fwd_cm",
     "fss_scan_bwd_cm",
@@ -107,6 +109,10 @@ def _declare(lib: ctypes.CDLL) -> None:
     lib.fss_copy_bytes.restype = _int
     lib.fss_gated_scan_fwd.restype = _int
     lib.fss_gated_scan_fwd.argtypes = [_int, _vp, _vp, _vp, _i64, _i64, _i64, _vp, _sz, _vp, _cfgp]
+    lib.fss_gated_scan_fwd_state.restype = _int
+    lib.fss_gated_scan_fwd_state.argtypes = [_int, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _vp, _sz, _vp, _cfgp]
+    lib.fss_gated_scan_bwd_state.restype = _int
+    lib.fss_gated_scan_bwd_state.argtypes = [_int, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _vp, _sz, _vp, _cfgp]
     lib.fss_gated_scan_bwd.restype = _int
     lib.fss_gated_scan_bwd.argtypes = [_int, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _vp, _sz, _vp, _cfgp]
     lib.fss_cm_workspace_bytes.restype = _sz

@@ -223,6 +223,22 @@ int fss_gated_scan_bwd(int dtype, const void *gate, const void *x, const void *h
                        workspace_bytes, stream, cfg, nullptr, nullptr, nullptr, x);
 }
 
+int fss_gated_scan_fwd_state(int dtype, const void *gate, const void *x, void *h, const float *h_before,
+                             float *h_last, int64_t bs, int64_t seq, int64_t d, void *workspace,
+                             size_t workspace_bytes, void *stream, const fss_config *cfg) {
+  return fss::run_scan(dtype, FSS_GATED_FWD, gate, x, nullptr, h, nullptr, bs, seq, d, workspace,
+                       workspace_bytes, stream, cfg, h_before, h_last, nullptr);
+}
+
+int fss_gated_scan_bwd_state(int dtype, const void *gate, const void *x, const void *h, const void *dout,
+                             const float *h_before, const float *grad_h_last, void *grad_gate, void *grad_x,
+                             float *grad_h_before, int64_t bs, int64_t seq, int64_t d, void *workspace,
+                             size_t workspace_bytes, void *stream, const fss_config *cfg) {
+  if (grad_h_before && !h_before) return FSS_ERR_NULL_POINTER;
+  return fss::run_scan(dtype, FSS_GATED_BWD, gate, dout, h, grad_x, grad_gate, bs, seq, d, workspace,
+                       workspace_bytes, stream, cfg, grad_h_last, grad_h_before, h_before, x);
+}
+
 int fss_scan_fwd_bf16(const void *alpha, const void *beta, void *h, int64_t bs, int64_t seq, int64_t d,
                       void *workspace, size_t workspace_bytes, void *stream) {
   return fss_scan_fwd_ex(FSS_BF16, alpha, beta, h, bs, seq, d, workspace, workspace_bytes, stream, nullptr);

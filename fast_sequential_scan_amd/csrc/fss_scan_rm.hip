@@ -261,10 +261,12 @@ __device__ __forceinline__ float sigmoid_f32(float z) {
 //   grad_x[t]    = g[t] * s[t]                                     s = sqrt(1 - alpha^2)
 //   grad_gate[t] = g[t] * (h[t-1] - x[t]*alpha[t]/s[t]) * alpha[t]*(1 - alpha[t])
 // (h[-1] = 0; the x term is dropped where alpha rounds to exactly 1, i.e. s = 0).
+// STATE: h[-1] and the gradient reaching the last state come in, the last state and the
+// gradient with respect to h[-1] go out, exactly as in the plain scan (scan_tile).
 // The backward needs alpha[t+1] as the coefficient of step t and alpha[t] for its
 // elementwise part: a slice of STEPS steps loads STEPS+1 rows of the gate.
-template <typename E, int VEC, int STEPS, bool BWD, bool FULL>
-__device__ __forceinline__ void gated_tile(const ScanArgs &p, const TileCtx &c) {
+template <typename E, int VEC, int STEPS, bool BWD, bool STATE, bool FULL>
+__device__ __forceinline__ void gated_tile(const ScanArgs &p, const StateArgs<STATE> &st, const TileCtx &c) {
   using RowT = Row<E, VEC>;
   const int64_t seq = c.seq, row_bytes = c.row_bytes, r0 = c.r0;
   const uint32_t lane_off = c.lane_off;
@@ -330,7 +332,8 @@ __device__ __forceinline__ void gated_tile(const ScanArgs &p, const TileCtx &c) 
     float al[VEC];
 #pragma unroll
     for (int v = 0; v < VEC; ++v) al[v] = sigmoid_f32(a[s].get(v));
-    if (!FULL && (r >= seq + (BWD ? 1 : 0) || !c.col_ok)) {
+    // (backward with a gradient coming in through the last state: it is added, coefficient 1)
+    if (!FULL && (r >= seq + (BWD ? 1 : 0) || !c.col_ok || (STATE && BWD && r == 0 && st.state_in))) {
 #pragma unroll
       for (int v = 0; v < VEC; ++v) al[v] = 1.0f;
     }
@@ -359,12 +362,20 @@ __device__ __forceinline__ void gated_tile(const ScanArgs &p, const TileCtx &c) 
     }
   }
 
+  // the state the whole sequence starts from: only its first chunk needs it
+  float seq_in[VEC];
+#pragma unroll
+  for (int v = 0; v < VEC; ++v) seq_in[v] = 0.0f;
+  if (STATE && st.state_in && c.chunk == 0 && c.col_ok) {
+#pragma unroll
+    for (int v = 0; v < VEC; ++v) seq_in[v] = st.state_in[c.chan_row + c.lane * VEC + v];
+  }
   float state[VEC];
   if (!c.chained && c.n_waves == 1) {
 #pragma unroll
-    for (int v = 0; v < VEC; ++v) state[v] = 0.0f;
+    for (int v = 0; v < VEC; ++v) state[v] = seq_in[v];
   } else {
-    chain_chunks<VEC, false>(p, c, mA, mB, nullptr, state, [] {});
+    chain_chunks<VEC, false>(p, c, mA, mB, STATE ? seq_in : nullptr, state, [] {});
   }
 
   // ---- phase 3 -------------------------------------------------------------------------
@@ -385,6 +396,8 @@ __device__ __forceinline__ void gated_tile(const ScanArgs &p, const TileCtx &c) 
     const int64_t r = r0 + s;
     const bool ident = !FULL && BWD && r >= seq;
     float o0[VEC], o1[VEC];
+    // t = 0 with a state coming in: h[-1] is that state, and alpha[0]*g[0] goes out
+    const bool t_zero = STATE && BWD && !FULL && r == seq - 1;
 #pragma unroll
     for (int v = 0; v < VEC; ++v) {
       state[v] = __builtin_fmaf(ident ? 1.0f : a[s].get(v), state[v], b[s].get(v));
@@ -393,7 +406,15 @@ __device__ __forceinline__ void gated_tile(const ScanArgs &p, const TileCtx &c) 
         const float om = __builtin_fmaf(-at, at, 1.0f);
         const float rs = om > 0.0f ? __builtin_amdgcn_rsqf(om) : 0.0f;
         o0[v] = state[v] * (om * rs);
-        const float inner = __builtin_fmaf(-xs[s].get(v) * at, rs, hp[s].get(v));
+        float h_prev = hp[s].get(v);
+        if constexpr (STATE) {
+          if (t_zero && c.col_ok) {
+            const int64_t ch = c.chan_row + c.lane * VEC + v;
+            if (st.h_before) h_prev = st.h_before[ch];
+            if (st.state_out) st.state_out[ch] = at * state[v];
+          }
+        }
+        const float inner = __builtin_fmaf(-xs[s].get(v) * at, rs, h_prev);
         o1[v] = state[v] * inner * (at - at * at);
       } else {
         o0[v] = state[v];
@@ -411,10 +432,16 @@ __device__ __forceinline__ void gated_tile(const ScanArgs &p, const TileCtx &c) 
     }
     if (BWD && s + kEarly < STEPS) load_hx(s + kEarly);
   }
+  // forward: the wave whose slice holds the last step hands out the final state (the steps
+  // past the end are identity maps)
+  if (STATE && !BWD && st.state_out && c.col_ok && r0 <= seq - 1 && seq - 1 < r0 + STEPS) {
+#pragma unroll
+    for (int v = 0; v < VEC; ++v) st.state_out[c.chan_row + c.lane * VEC + v] = state[v];
+  }
 }
 
 // STATE: the variant that honours the optional incoming/outgoing state rows of ScanArgs;
-// the plain scan is compiled without them.  GATED: the gated scan (never with STATE).
+// the plain and the gated scan are compiled without them.  GATED: the gated scan.
 // ALT: the other cache policy of the plain scan - the forward for small outputs, which stores h
 // without the non-temporal hint; the backward for large tensors, which reads dout with it.
 template <typename E, int VEC, int STEPS, bool BWD, bool STATE, bool GATED = false, bool ALT = false>
@@ -489,9 +516,9 @@ __global__ __launch_bounds__(1024) void scan_kernel(const ScanArgs p, const Stat
     // same barriers, so they meet
     if constexpr (GATED) {
       if (full)
-        gated_tile<E, VEC, STEPS, BWD, true>(p, c);
+        gated_tile<E, VEC, STEPS, BWD, STATE, true>(p, st, c);
       else
-        gated_tile<E, VEC, STEPS, BWD, false>(p, c);
+        gated_tile<E, VEC, STEPS, BWD, STATE, false>(p, st, c);
     } else {
       if (full)
         scan_tile<E, VEC, STEPS, BWD, STATE, true, ALT>(p, st, c);
@@ -570,22 +597,21 @@ int launch_typed(const ScanArgs &args, const StateArgs<true> &state, const Plan 
 }
 
 // The gated kernels: 4 bytes (bf16 x2, fp32 x1) or one bf16 element per lane.
-template <typename E, bool BWD>
-int launch_gated(const ScanArgs &args, const Plan &pl, hipStream_t stream) {
+template <typename E, bool BWD, bool STATE>
+int launch_gated(const ScanArgs &args, const StateArgs<true> &none, const Plan &pl, hipStream_t stream) {
   constexpr bool is_16bit = E::kBytes == 2;
-  const StateArgs<true> none = {nullptr, nullptr, nullptr};
   const int key = pl.cfg.vec * 100 + pl.cfg.steps;
   switch (key) {
 #define FSS_CASE(V, S) \
   case V * 100 + S:    \
-    return launch_one<E, V, S, BWD, false, true>(args, none, pl, stream);
+    return launch_one<E, V, S, BWD, STATE, true>(args, none, pl, stream);
     FSS_CASE(1, 8)
     FSS_CASE(1, 16)
     default:
       break;
   }
   if constexpr (!BWD) {
-    if (key == 132) return launch_one<E, 1, 32, BWD, false, true>(args, none, pl, stream);
+    if (key == 132) return launch_one<E, 1, 32, BWD, STATE, true>(args, none, pl, stream);
   }
   if constexpr (is_16bit) {
     switch (key) {
@@ -595,7 +621,7 @@ int launch_gated(const ScanArgs &args, const Plan &pl, hipStream_t stream) {
         break;
     }
     if constexpr (!BWD) {
-      if (key == 232) return launch_one<E, 2, 32, BWD, false, true>(args, none, pl, stream);
+      if (key == 232) return launch_one<E, 2, 32, BWD, STATE, true>(args, none, pl, stream);
     }
   }
 #undef FSS_CASE
@@ -605,7 +631,13 @@ int launch_gated(const ScanArgs &args, const Plan &pl, hipStream_t stream) {
 int FSS_RM_LAUNCH(const ScanArgs &args, const StateArgs<true> &state, const Plan &pl, bool bwd, bool gated,
                   bool with_state, hipStream_t stream) {
   using E = FSS_RM_ELEM;
-  if (gated) return bwd ? launch_gated<E, true>(args, pl, stream) : launch_gated<E, false>(args, pl, stream);
+  if (gated) {
+    if (bwd)
+      return with_state ? launch_gated<E, true, true>(args, state, pl, stream)
+                        : launch_gated<E, true, false>(args, state, pl, stream);
+    return with_state ? launch_gated<E, false, true>(args, state, pl, stream)
+                      : launch_gated<E, false, false>(args, state, pl, stream);
+  }
   if (bwd)
     return with_state ? launch_typed<E, true, true>(args, state, pl, stream)
                       : launch_typed<E, true, false>(args, state, pl, stream);

@@ -18,7 +18,8 @@ from . import sequential_scan_cuda as _ext
 
 __all__ = [
     "SequentialScan", "SequentialScanSingle", "SequentialScanFp16", "SequentialScanState", "SequentialScanGated",
-    "SequentialScanChannelMajor", "scan", "scan_single", "scan_fp16", "scan_with_state", "scan_gated", "scan_cm",
+    "SequentialScanChannelMajor", "SequentialScanGatedState", "scan", "scan_single", "scan_fp16", "scan_with_state",
+    "scan_gated", "scan_gated_with_state", "scan_cm",
 ]
 
 
@@ -150,6 +151,41 @@ def scan_gated(gate: torch.Tensor, x: torch.Tensor) -> torch.Tensor:
     """The Hawk / RG-LRU style gated recurrence from its pre-activations:
     ``a = sigmoid(gate)``, ``h[t] = a[t]*h[t-1] + sqrt(1 - a[t]**2) * x[t]``."""
     return SequentialScanGated.apply(gate, x)
+
+
+class SequentialScanGatedState(Function):
+    """The gated scan with a state entering and leaving the sequence:
+    ``(h, h_last) = f(gate, x, h_before)``.  Not in the reference.  Differentiable in all three
+    inputs, through both outputs."""
+
+    @staticmethod
+    def forward(ctx: Any, gate: torch.Tensor, x: torch.Tensor, h_before: Optional[torch.Tensor]):
+        h, h_last = _ext.gated_scan_forward_state(gate, x, h_before)
+        ctx.has_state = h_before is not None
+        if ctx.has_state:
+            ctx.save_for_backward(gate, x, h, h_before)
+        else:
+            ctx.save_for_backward(gate, x, h)
+        return h, h_last
+
+    @staticmethod
+    @once_differentiable
+    def backward(ctx: Any, grad_h: torch.Tensor, grad_h_last: torch.Tensor):
+        if ctx.has_state:
+            gate, x, h, h_before = ctx.saved_tensors
+        else:
+            (gate, x, h), h_before = ctx.saved_tensors, None
+        grad_gate, grad_x, grad_h_before = _ext.gated_scan_backward_state(gate, x, h, grad_h, h_before, grad_h_last)
+        return grad_gate, grad_x, grad_h_before
+
+
+def scan_gated_with_state(
+    gate: torch.Tensor, x: torch.Tensor, h_before: Optional[torch.Tensor] = None
+) -> Tuple[torch.Tensor, torch.Tensor]:
+    """:func:`scan_gated` from ``h[-1] = h_before`` (fp32 ``(bs, d_model)``, zeros when None).  Returns
+    ``(h, h_last)`` with ``h_last`` the fp32 state after the last step, to be passed as ``h_before`` of
+    the next segment (chunked prefill, decoding, a sequence sharded over devices)."""
+    return SequentialScanGatedState.apply(gate, x, h_before)
 
 
 class SequentialScanChannelMajor(Function):

@@ -25,7 +25,7 @@ __all__ = [
     "scan_forward", "scan_backward", "scan_forward_half", "scan_backward_half",
     "scan_forward_fp16", "scan_backward_fp16",
     "scan_forward_state", "scan_backward_state",
-    "gated_scan_forward", "gated_scan_backward",
+    "gated_scan_forward", "gated_scan_backward", "gated_scan_forward_state", "gated_scan_backward_state",
     "scan_forward_cm", "scan_backward_cm",
 ]
 
@@ -317,6 +317,78 @@ def gated_scan_backward(
             )
         )
     return [grad_gate, grad_x]
+
+
+def gated_scan_forward_state(
+    gate: torch.Tensor, x: torch.Tensor, h_before: Optional[torch.Tensor] = None, config=None
+) -> Tuple[torch.Tensor, torch.Tensor]:
+    """(h, h_last) of the gated scan started from ``h[-1] = h_before`` (fp32 ``(bs, d)``, zeros when
+    None); ``h_last`` is the un-rounded fp32 state after the last step."""
+    dtype = _either_dtype(gate, "gate")
+    bs, seq, d = _validate(dtype, gate=gate, x=x)
+    h_before = _state("h_before", h_before, gate)
+    gate, x = gate.contiguous(), x.contiguous()
+    out = torch.empty_like(gate, memory_format=torch.contiguous_format)
+    h_last = torch.zeros((bs, d), dtype=torch.float32, device=gate.device)
+    if out.numel() == 0:
+        if h_before is not None and seq == 0:
+            h_last.copy_(h_before)
+        return out, h_last
+    lib = _native.lib()
+    code = _DTYPE_CODE[dtype]
+    cfg = _native.make_config(config)
+    with torch.cuda.device(gate.device):
+        stream = torch.cuda.current_stream()
+        ws = _workspace(gate.device, stream, lib.fss_workspace_bytes(bs, seq, d, code, _native.FSS_GATED_FWD, cfg))
+        _native.check(
+            lib.fss_gated_scan_fwd_state(
+                code, gate.data_ptr(), x.data_ptr(), out.data_ptr(),
+                h_before.data_ptr() if h_before is not None else None, h_last.data_ptr(),
+                bs, seq, d, ws.data_ptr(), ws.numel(), stream.cuda_stream, cfg,
+            )
+        )
+    return out, h_last
+
+
+def gated_scan_backward_state(
+    gate: torch.Tensor,
+    x: torch.Tensor,
+    h_saved: torch.Tensor,
+    grad_out: torch.Tensor,
+    h_before: Optional[torch.Tensor] = None,
+    grad_h_last: Optional[torch.Tensor] = None,
+    config=None,
+) -> Tuple[torch.Tensor, torch.Tensor, Optional[torch.Tensor]]:
+    """(grad_gate, grad_x, grad_h_before); the last is None when ``h_before`` is None."""
+    dtype = _either_dtype(gate, "gate")
+    bs, seq, d = _validate(dtype, gate=gate, x=x, h_saved=h_saved, grad_out=grad_out)
+    h_before = _state("h_before", h_before, gate)
+    grad_h_last = _state("grad_h_last", grad_h_last, gate)
+    gate, x, h_saved, grad_out = gate.contiguous(), x.contiguous(), h_saved.contiguous(), grad_out.contiguous()
+    grad_gate = torch.empty_like(gate, memory_format=torch.contiguous_format)
+    grad_x = torch.empty_like(gate, memory_format=torch.contiguous_format)
+    grad_h_before = torch.zeros((bs, d), dtype=torch.float32, device=gate.device) if h_before is not None else None
+    if grad_gate.numel() == 0:
+        if grad_h_before is not None and grad_h_last is not None and seq == 0:
+            grad_h_before.copy_(grad_h_last)
+        return grad_gate, grad_x, grad_h_before
+    lib = _native.lib()
+    code = _DTYPE_CODE[dtype]
+    cfg = _native.make_config(config)
+    with torch.cuda.device(gate.device):
+        stream = torch.cuda.current_stream()
+        ws = _workspace(gate.device, stream, lib.fss_workspace_bytes(bs, seq, d, code, _native.FSS_GATED_BWD, cfg))
+        _native.check(
+            lib.fss_gated_scan_bwd_state(
+                code, gate.data_ptr(), x.data_ptr(), h_saved.data_ptr(), grad_out.data_ptr(),
+                h_before.data_ptr() if h_before is not None else None,
+                grad_h_last.data_ptr() if grad_h_last is not None else None,
+                grad_gate.data_ptr(), grad_x.data_ptr(),
+                grad_h_before.data_ptr() if grad_h_before is not None else None,
+                bs, seq, d, ws.data_ptr(), ws.numel(), stream.cuda_stream, cfg,
+            )
+        )
+    return grad_gate, grad_x, grad_h_before
 
 
 # ---- channel-major layout: tensors (bs, d_model, seq), time contiguous (what the accelerated-scan

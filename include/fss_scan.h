@@ -224,6 +224,25 @@ int fss_gated_scan_bwd(int dtype, const void *gate, const void *x, const void *h
                        void *stream, const fss_config *cfg);
 
 /*
+ * The gated scan with a state entering and leaving the sequence: fss_gated_scan_fwd /
+ * fss_gated_scan_bwd with the state arguments, semantics and chaining property of
+ * fss_scan_fwd_state / fss_scan_bwd_state (alpha there = sigmoid(gate) here):
+ *   forward   h[-1] = h_before;  h_last = the un-rounded state after the last step.
+ *   backward  g[seq-1] = dout[seq-1] + grad_h_last;  h[-1] = h_before in grad_gate[0];
+ *             grad_h_before = alpha[0]*g[0] (needs h_before).
+ * No counterpart in the reference.  States are fp32 (bs, d); any may be NULL.
+ */
+int fss_gated_scan_fwd_state(int dtype, const void *gate, const void *x, void *h,
+                             const float *h_before, float *h_last, int64_t bs, int64_t seq,
+                             int64_t d, void *workspace, size_t workspace_bytes, void *stream,
+                             const fss_config *cfg);
+int fss_gated_scan_bwd_state(int dtype, const void *gate, const void *x, const void *h,
+                             const void *dout, const float *h_before, const float *grad_h_last,
+                             void *grad_gate, void *grad_x, float *grad_h_before, int64_t bs,
+                             int64_t seq, int64_t d, void *workspace, size_t workspace_bytes,
+                             void *stream, const fss_config *cfg);
+
+/*
  * Channel-major layout: tensors are (bs, d, seq) row-major, i.e. every (batch, channel)
  * pair is a contiguous run of seq timesteps - the layout of the `accelerated-scan`
  * package the reference benchmarks against after a permute().contiguous() of its own

@@ -123,6 +123,9 @@ int main(void) {
   if (fss_gated_scan_bwd(FSS_BF16, d_alpha, NULL, d_h, d_dout, d_ga, d_gb, bs, seq, d, d_ws, ws_bytes, stream, NULL) !=
       FSS_ERR_NULL_POINTER)
     ++failed;
+  if (fss_gated_scan_bwd_state(FSS_BF16, d_alpha, d_beta, d_h, d_dout, NULL, NULL, d_ga, d_gb, (float *)d_ws, bs, seq, d,
+                               d_ws, ws_bytes, stream, NULL) != FSS_ERR_NULL_POINTER)
+    ++failed; /* grad_h_before without h_before */
   if (fss_scan_fwd_cm(FSS_BF16, d_alpha, d_beta, d_h, bs, d, seq, d_ws, 0, stream, NULL) != FSS_OK)
     ++failed; /* seq 1000 fits one workgroup: no workspace needed */
   if (fss_scan_fwd_bf16(d_alpha, d_beta, d_h, bs, seq, d, d_ws, 64, stream) != FSS_ERR_WORKSPACE_SMALL) ++failed;

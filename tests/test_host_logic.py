@@ -193,6 +193,9 @@ def test_planning_of_the_gated_fp16_and_channel_major_entry_points():
     one = ctypes.c_void_p(256)
     assert lib.fss_gated_scan_fwd(0, None, one, one, 1, 8, 8, None, 0, None, None) == 1
     assert lib.fss_gated_scan_bwd(0, one, None, one, one, one, one, 1, 8, 8, None, 0, None, None) == 1
+    assert lib.fss_gated_scan_fwd_state(0, one, one, None, None, None, 1, 8, 8, None, 0, None, None) == 1
+    # the gradient with respect to h[-1] needs h[-1]
+    assert lib.fss_gated_scan_bwd_state(0, one, one, one, one, None, None, one, one, one, 1, 8, 8, None, 0, None, None) == 1
     assert lib.fss_scan_fwd_cm(0, one, one, None, 1, 8, 8, None, 0, None, None) == 1
     assert lib.fss_scan_bwd_cm(0, one, one, one, None, one, 1, 8, 8, None, 0, None, None) == 1
     assert lib.fss_scan_fwd_cm(0, one, one, one, 1, -8, 8, None, 0, None, None) == 2
