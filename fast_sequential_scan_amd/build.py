@@ -8,7 +8,7 @@ shared library (include/fss_scan.h): no torch headers, no pybind.
 
 Translation units (compiled in parallel, then linked):
   csrc/fss_api.hip       the C ABI, planning, small kernels
-  csrc/fss_scan_rm.hip   the row-major scan kernels, once per storage type
+  csrc/fss_scan_rm.hip   the row-major scan kernels, once per storage type and direction
   csrc/fss_scan_cm.hip   the channel-major scan kernels
 """
 from __future__ import annotations
@@ -39,9 +39,11 @@ HIPCC_FLAGS: List[str] = [
 # (object name, source, extra defines)
 UNITS: Sequence[Tuple[str, str, Tuple[str, ...]]] = (
     ("api", "fss_api.hip", ()),
-    ("rm_bf16", "fss_scan_rm.hip", ("-DFSS_RM_ELEM=BF16", "-DFSS_RM_LAUNCH=launch_rm_bf16")),
-    ("rm_f16", "fss_scan_rm.hip", ("-DFSS_RM_ELEM=F16", "-DFSS_RM_LAUNCH=launch_rm_f16")),
-    ("rm_f32", "fss_scan_rm.hip", ("-DFSS_RM_ELEM=F32", "-DFSS_RM_LAUNCH=launch_rm_f32")),
+    *(
+        (f"rm_{t.lower()}_{name}", "fss_scan_rm.hip",
+         (f"-DFSS_RM_ELEM={t}", f"-DFSS_RM_BWD={bwd}", f"-DFSS_RM_LAUNCH=launch_rm_{t.lower()}_{name}"))
+        for t in ("BF16", "F16", "F32") for bwd, name in ((0, "fwd"), (1, "bwd"))
+    ),
     ("cm", "fss_scan_cm.hip", ()),
 )
 

@@ -80,9 +80,11 @@ int run_scan(int dtype, int dir, const void *alpha, const void *in_b, const void
   const bool st = state_in || state_out || h_before;
   const bool bwd = dir == FSS_BWD;
   const ScanOrderGuard ordered(s);
-  if (dtype == FSS_BF16) return launch_rm_bf16(args, state, pl, bwd, gated, st, s);
-  if (dtype == FSS_F16) return launch_rm_f16(args, state, pl, bwd, gated, st, s);
-  return launch_rm_f32(args, state, pl, bwd, gated, st, s);
+  if (dtype == FSS_BF16)
+    return bwd ? launch_rm_bf16_bwd(args, state, pl, gated, st, s) : launch_rm_bf16_fwd(args, state, pl, gated, st, s);
+  if (dtype == FSS_F16)
+    return bwd ? launch_rm_f16_bwd(args, state, pl, gated, st, s) : launch_rm_f16_fwd(args, state, pl, gated, st, s);
+  return bwd ? launch_rm_f32_bwd(args, state, pl, gated, st, s) : launch_rm_f32_fwd(args, state, pl, gated, st, s);
 }
 
 }  // namespace fss

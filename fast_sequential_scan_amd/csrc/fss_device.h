@@ -231,6 +231,9 @@ constexpr size_t kHeaderBytes = 4096;
 constexpr uint32_t kSpinLimit = 1u << 20;
 // Most waves of a workgroup that look back in parallel, one earlier chunk each.
 constexpr int kMaxLookWaves = 16;
+// chunks one look-back wave covers at most (measured: 2 -> 4 gains up to 12 % on chains of
+// hundreds of chunks, 8 nothing more)
+constexpr int kMaxSpan = 4;
 enum : uint32_t { kPredNone = 0, kPredMap = 1, kPredState = 2 };
 
 __device__ __forceinline__ uint32_t ld_u32(const uint32_t *p) {

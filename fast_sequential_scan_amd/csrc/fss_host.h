@@ -377,14 +377,18 @@ inline int make_cm_plan(CmPlan &pl, int64_t rows, int64_t seq, int dtype, int di
 
 // ---- what each translation unit provides --------------------------------------------------
 
-// fss_scan_rm.hip, compiled once per storage type: launches the row-major kernel (plain,
-// with states, or gated) the plan asks for.
-int launch_rm_bf16(const ScanArgs &args, const StateArgs<true> &state, const Plan &pl, bool bwd, bool gated,
-                   bool with_state, hipStream_t stream);
-int launch_rm_f16(const ScanArgs &args, const StateArgs<true> &state, const Plan &pl, bool bwd, bool gated,
-                  bool with_state, hipStream_t stream);
-int launch_rm_f32(const ScanArgs &args, const StateArgs<true> &state, const Plan &pl, bool bwd, bool gated,
-                  bool with_state, hipStream_t stream);
+// fss_scan_rm.hip, compiled once per storage type and direction: launches the row-major
+// kernel (plain, with states, or gated) the plan asks for.
+#define FSS_DECLARE_RM_LAUNCH(name)                                                                        \
+  int name(const ScanArgs &args, const StateArgs<true> &state, const Plan &pl, bool gated, bool with_state, \
+           hipStream_t stream)
+FSS_DECLARE_RM_LAUNCH(launch_rm_bf16_fwd);
+FSS_DECLARE_RM_LAUNCH(launch_rm_bf16_bwd);
+FSS_DECLARE_RM_LAUNCH(launch_rm_f16_fwd);
+FSS_DECLARE_RM_LAUNCH(launch_rm_f16_bwd);
+FSS_DECLARE_RM_LAUNCH(launch_rm_f32_fwd);
+FSS_DECLARE_RM_LAUNCH(launch_rm_f32_bwd);
+#undef FSS_DECLARE_RM_LAUNCH
 
 // fss_scan_cm.hip
 int run_cm_scan(int dtype, int dir, const void *alpha, const void *in_b, const void *in_h, void *out0, void *out1,

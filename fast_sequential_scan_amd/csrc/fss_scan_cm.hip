@@ -202,11 +202,8 @@ __global__ __launch_bounds__(1024) void cm_scan_kernel(const ScanArgs p) {
   c.wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   c.n_waves = blockDim.x >> 6;
   c.look = p.look_waves;
-#ifndef FSS_MAX_SPAN
-#define FSS_MAX_SPAN 4
-#endif
   c.span = (p.n_chunks + p.look_waves - 1) / p.look_waves;
-  if (c.span > FSS_MAX_SPAN) c.span = FSS_MAX_SPAN;
+  if (c.span > kMaxSpan) c.span = kMaxSpan;
   float2 *const lds_maps = reinterpret_cast<float2 *>(lds);  // laid out as in scan_kernel with one slot per lane
   c.lds_pred = lds_maps + 2 * c.n_waves * 64;
   c.s_kind = s_kind;

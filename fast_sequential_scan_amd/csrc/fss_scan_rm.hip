@@ -67,10 +67,11 @@
 #include "fss_device.h"
 #include "fss_host.h"
 
-// This file is compiled once per storage type: FSS_RM_ELEM names the element type
-// (BF16, F16 or F32) and FSS_RM_LAUNCH the entry it defines (launch_rm_bf16, ...).
-#if !defined(FSS_RM_ELEM) || !defined(FSS_RM_LAUNCH)
-#error "define FSS_RM_ELEM and FSS_RM_LAUNCH"
+// This file is compiled once per storage type and direction: FSS_RM_ELEM names the element
+// type (BF16, F16 or F32), FSS_RM_BWD the direction (0 forward, 1 backward) and
+// FSS_RM_LAUNCH the entry it defines (launch_rm_bf16_fwd, ...).
+#if !defined(FSS_RM_ELEM) || !defined(FSS_RM_LAUNCH) || !defined(FSS_RM_BWD)
+#error "define FSS_RM_ELEM, FSS_RM_BWD and FSS_RM_LAUNCH"
 #endif
 
 namespace fss {
@@ -456,11 +457,8 @@ __global__ __launch_bounds__(1024) void scan_kernel(const ScanArgs p, const Stat
   c.wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   c.n_waves = blockDim.x >> 6;
   c.look = p.look_waves;
-#ifndef FSS_MAX_SPAN
-#define FSS_MAX_SPAN 4
-#endif
   c.span = (p.n_chunks + p.look_waves - 1) / p.look_waves;
-  if (c.span > FSS_MAX_SPAN) c.span = FSS_MAX_SPAN;
+  if (c.span > kMaxSpan) c.span = kMaxSpan;
   // LDS: two sets of per-wave maps (tiles alternate between them, so a wave that runs
   // ahead into the next tile cannot overwrite a map a slower wave still reads), then
   // the slots the look-back waves fill
@@ -628,21 +626,15 @@ int launch_gated(const ScanArgs &args, const StateArgs<true> &none, const Plan &
   return FSS_ERR_BAD_CONFIG;
 }
 
-int FSS_RM_LAUNCH(const ScanArgs &args, const StateArgs<true> &state, const Plan &pl, bool bwd, bool gated,
-                  bool with_state, hipStream_t stream) {
+int FSS_RM_LAUNCH(const ScanArgs &args, const StateArgs<true> &state, const Plan &pl, bool gated, bool with_state,
+                  hipStream_t stream) {
   using E = FSS_RM_ELEM;
-  if (gated) {
-    if (bwd)
-      return with_state ? launch_gated<E, true, true>(args, state, pl, stream)
-                        : launch_gated<E, true, false>(args, state, pl, stream);
-    return with_state ? launch_gated<E, false, true>(args, state, pl, stream)
-                      : launch_gated<E, false, false>(args, state, pl, stream);
-  }
-  if (bwd)
-    return with_state ? launch_typed<E, true, true>(args, state, pl, stream)
-                      : launch_typed<E, true, false>(args, state, pl, stream);
-  return with_state ? launch_typed<E, false, true>(args, state, pl, stream)
-                    : launch_typed<E, false, false>(args, state, pl, stream);
+  constexpr bool kBwd = FSS_RM_BWD != 0;
+  if (gated)
+    return with_state ? launch_gated<E, kBwd, true>(args, state, pl, stream)
+                      : launch_gated<E, kBwd, false>(args, state, pl, stream);
+  return with_state ? launch_typed<E, kBwd, true>(args, state, pl, stream)
+                    : launch_typed<E, kBwd, false>(args, state, pl, stream);
 }
 
 }  // namespace fss
