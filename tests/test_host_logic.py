@@ -215,3 +215,27 @@ def test_shipped_package_never_touches_the_oracle():
                 if re.search(r"^\s*(from|import)\s+oracle\b", text, flags=re.M) or "oracle/" in text:
                     offenders.append(os.path.join(base, name))
     assert not offenders, offenders
+
+
+def test_common_helpers_follow_their_definitions(oracle):
+    """The helper module under the reference's names: the scan's definition against the pinned
+    oracle, the metric and its digit rule against hand-computed values."""
+    import numpy as np
+
+    from sequential_scan.common import BFLOAT16_TOL, SINGLE_TOL, check_relative_error, relative_error, torch_ref
+
+    g = torch.Generator().manual_seed(5)
+    alpha = torch.rand(3, 17, 6, generator=g, dtype=torch.float64).requires_grad_(True)
+    beta = torch.randn(3, 17, 6, generator=g, dtype=torch.float64).requires_grad_(True)
+    h = torch_ref(alpha, beta)
+    np.testing.assert_allclose(h.detach().numpy(), oracle.scan_fwd_f64(alpha.detach().numpy(), beta.detach().numpy()),
+                               rtol=1e-13)
+    dy = torch.randn(3, 17, 6, generator=g, dtype=torch.float64)
+    h.backward(dy)
+    assert alpha.grad[:, 0].abs().max() == 0  # alpha[:, 0] is never used
+    x, y = torch.tensor([3.0, 4.0]), torch.tensor([0.0, 4.0])
+    assert relative_error(x, y) == pytest.approx(3.0 / 4.0)
+    assert (SINGLE_TOL, BFLOAT16_TOL) == (7.0, 2.0)
+    assert check_relative_error(0.0, 7) and check_relative_error(1e-8, 7) and check_relative_error(9e-7, 7)
+    assert not check_relative_error(1.1e-6, 7)
+    assert check_relative_error(0.09, 2) and not check_relative_error(0.11, 2)
