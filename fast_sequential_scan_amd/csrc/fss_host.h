@@ -51,6 +51,10 @@ inline bool config_valid(const fss_config &c, int dtype, bool gated = false, int
   return true;
 }
 
+// CUs of an unpartitioned MI355X: what "one tile per CU" means when a launch is planned
+// (planning must work without a device; the grid itself is sized from the runtime's count).
+constexpr int64_t kCus = 256;
+
 // One candidate launch configuration: taken when it yields at least `need` tiles.
 struct Rung {
   int vec, steps, waves;
@@ -66,7 +70,7 @@ struct Rung {
 // sequence (a short chain) and long uninterrupted streams per wave; 16 waves of 32
 // (backward 16) timesteps with 4 bytes per lane is the largest that fits the register
 // file.  So the choice walks down a ladder of tile sizes, each half the one before, and
-// takes the first with at least 256 tiles; which of time, channels per lane and waves
+// takes the first with at least one tile per CU; which of time, channels per lane and waves
 // is halved at each rung is what the sweeps decided.  Below the last rung the problem
 // is latency-bound and the smallest tile is as good as any.
 inline void complete_config(fss_config &c, int64_t bs, int64_t seq, int64_t d, int dtype, int dir,
@@ -82,7 +86,7 @@ inline void complete_config(fss_config &c, int64_t bs, int64_t seq, int64_t d, i
                       bs * seq * d >= (static_cast<int64_t>(1) << 26);
   Rung ladder[6];
   int n = 0;
-  auto rung = [&](int v, int s, int w, int64_t need = 256) { ladder[n++] = Rung{v, s, w, need}; };
+  auto rung = [&](int v, int s, int w, int64_t need = kCus) { ladder[n++] = Rung{v, s, w, need}; };
   const bool fwd = dir == FSS_FWD;
   if (!gated && fwd) {
     // (very long sequences: one channel per lane, i.e. twice the independent chains, is 5-16 % faster)
@@ -107,22 +111,21 @@ inline void complete_config(fss_config &c, int64_t bs, int64_t seq, int64_t d, i
     // The gated kernels spend as much time on arithmetic as on memory and like more, smaller
     // waves; a sequence that 8 waves cover wants two workgroups per CU before it takes them.
     if (narrow) {
-      if (seq > 256) rung(2, 32, 16); else rung(2, 32, 8, 512);
+      if (seq > 256) rung(2, 32, 16); else rung(2, 32, 8, 2 * kCus);
       if (seq >= 4096) rung(1, 32, 16); else rung(2, 16, 16);
       if (seq >= 16384) rung(1, 32, 8);
       rung(1, 16, 16);
       if (seq >= 1024) rung(1, 16, 8, 0); else rung(1, 16, 16, 0);
     } else {
-      if (seq > 256) rung(1, 32, 16); else rung(1, 32, 8, 512);
+      if (seq > 256) rung(1, 32, 16); else rung(1, 32, 8, 2 * kCus);
       rung(1, 16, 16, 0);
     }
   } else {
     // gated backward: four tensors per timestep, at most 16 steps per lane (fp32: 8 are faster)
     if (narrow) {
-      if (seq > 256) rung(2, 16, 16); else rung(2, 16, 8, 1024);
+      if (seq > 256) rung(2, 16, 16); else rung(2, 16, 8, 4 * kCus);
       rung(2, 8, 16);
-      rung(2, 8, 8);
-      if (seq <= 256) rung(2, 8, 8, 1);
+      rung(2, 8, 8, seq <= 256 ? 1 : kCus);
       rung(1, 8, 8, 0);
     } else {
       if (seq > 256) rung(1, 8, 16);
@@ -143,14 +146,14 @@ inline void complete_config(fss_config &c, int64_t bs, int64_t seq, int64_t d, i
     pick = fss_config{v, s, w, 0};
     if (bs * ceil_div(d, 64 * static_cast<int64_t>(v)) * ceil_div(seq, static_cast<int64_t>(s) * w) >= ladder[i].need) break;
   }
-  // Forward, 16-wave workgroups (one per CU) whose last round would leave CUs idle: the same
-  // tile shape as two 8-wave workgroups per CU spreads that round over all CUs (7-18 % on 59
-  // shapes with sequence lengths and widths that are no powers of two; the backward, already two
-  // tiles per CU and round at the sizes that matter, gains nothing).
+  // Forward, 16-wave workgroups (one per CU) whose last round would fill less than 90 % of the
+  // CUs: the same tile shape as 8-wave workgroups, two per CU, spreads that round over all CUs
+  // (7-18 % faster on 59 of 182 shapes with lengths and widths that are no powers of two; the
+  // backward measured no gain from it).
   if (fwd && !c.waves && pick.waves == 16) {
     const int64_t tiles = bs * ceil_div(d, 64 * static_cast<int64_t>(pick.vec)) * ceil_div(seq, static_cast<int64_t>(pick.steps) * 16);
-    const int64_t rounds = ceil_div(tiles, 256);
-    if (rounds >= 2 && tiles * 10 < rounds * 256 * 9) pick.waves = 8;
+    const int64_t rounds = ceil_div(tiles, kCus);
+    if (rounds >= 2 && tiles * 10 < rounds * kCus * 9) pick.waves = 8;
   }
   c.vec = pick.vec;
   c.steps = pick.steps;
