@@ -64,6 +64,12 @@ def parse_args():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline / parity leg")
     ap.add_argument("--cpu-seconds", type=float, default=12.0, help="budget of the CPU baseline leg")
     ap.add_argument("--flush-mb", type=int, default=1024, help="size of the cache-flush read for the cold timings")
+    ap.add_argument("--sweep", action="store_true",
+                    help="the reference's benchmark sweep (benchmark.py:37-110): sequence lengths 128..32768 at "
+                         "--sweep-bs x --sweep-d, forward and forward+backward through the public autograd API, "
+                         "one cache-clearing write before every timed call as triton's do_bench does; one JSON line")
+    ap.add_argument("--sweep-bs", type=int, default=8)
+    ap.add_argument("--sweep-d", type=int, default=1024)
     ap.add_argument("--copy-mb", type=int, default=0,
                     help="run only the library's plain copy kernel on this many MiB, --steps times "
                          "(hardware counters of the scan kernels are scaled by what they read for it)")
@@ -76,6 +82,55 @@ def quantile_pair(samples):
         return [round(samples[0], 5)] * 2 if samples else None
     q = statistics.quantiles(samples, n=5, method="inclusive")
     return [round(q[0], 5), round(q[3], 5)]
+
+
+def sweep(args, torch, scan_cu, dev) -> int:
+    """Times what the reference's benchmark.py times for its "cuda-bf16" provider: `scan_cu(alpha, beta)`
+    and `scan_cu(alpha, beta).backward(dy)` per sequence length, median and 20th/80th percentile of
+    100 calls, each after a 256 MB write that clears the caches."""
+    bs, d = args.sweep_bs, args.sweep_d
+    flush = torch.empty(256 << 20, dtype=torch.uint8, device=dev)
+    rows = []
+    for sq in (128, 256, 1024, 2048, 4096, 8192, 16384, 32768):
+        gen = torch.Generator(device=dev).manual_seed(sq)
+        alpha = torch.sigmoid(torch.randn(bs, sq, d, device=dev, generator=gen)).to(torch.bfloat16).requires_grad_(True)
+        beta = torch.randn(bs, sq, d, device=dev, generator=gen).to(torch.bfloat16).requires_grad_(True)
+        dy = (0.1 * torch.randn(bs, sq, d, device=dev, generator=gen)).to(torch.bfloat16)
+
+        def fwd():
+            with torch.no_grad():
+                return scan_cu(alpha, beta)
+
+        def fwd_bwd():
+            alpha.grad = beta.grad = None
+            scan_cu(alpha, beta).backward(dy)
+
+        row = {"seq": sq, "elements": bs * sq * d}
+        for name, fn, nbytes in (("fwd", fwd, 6), ("fwd_bwd", fwd_bwd, 16)):
+            for _ in range(10):
+                fn()
+            times = []
+            for _ in range(100):
+                flush.zero_()
+                e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                e0.record()
+                fn()
+                e1.record()
+                e1.synchronize()
+                times.append(e0.elapsed_time(e1))
+            med = statistics.median(times)
+            row[name + "_ms"] = round(med, 5)
+            row[name + "_ms_p20_p80"] = quantile_pair(times)
+            row[name + "_GBps"] = round(nbytes * bs * sq * d / (med * 1e-3) / 1e9, 1)
+        rows.append(row)
+        del alpha, beta, dy
+    print(json.dumps({
+        "metric": "scan_cu forward and forward+backward ms per sequence length (the reference's benchmark.py sweep)",
+        "unit": "ms", "bs": bs, "d_model": d, "dtype": "bf16", "data": "synthetic",
+        "protocol": "public autograd API, caches cleared by a 256 MB write before every timed call, median of 100",
+        "sweep": rows,
+    }))
+    return 0
 
 
 def main() -> int:
@@ -120,6 +175,9 @@ def main() -> int:
                           "ms_per_launch": round(ms, 5), "value": round(2 * n / (ms * 1e-3) / 1e9, 1),
                           "unit": "GB/s (read+write)"}))
         return 0
+
+    if args.sweep:
+        return sweep(args, torch, scan_cu, dev)
 
     recipe, bs, seq, d = BASELINE_CASES[args.case]
     n_elem = bs * seq * d
