@@ -188,6 +188,23 @@ def test_baseline_configs_full_size(oracle, case):
     ext.workspace_status()
 
 
+def test_fp32_at_headline_shape(oracle):
+    """fp32 at bs 8, seq 4096, d 1024: 128 MiB per tensor, so the backward runs the instantiation
+    that reads dout with the streaming hint.  Against the fp32 oracle, the reference's fp32 bar
+    (relative L2 error below 1e-6) and elementwise."""
+    alpha, beta, dout = make_inputs("sigmoid", 8, 4096, 1024, dtype=torch.float32, seed=83)
+    a, b, do = alpha.to(DEV), beta.to(DEV), dout.to(DEV)
+    h = ext.scan_forward(a, b)
+    ga, gb = ext.scan_backward(a, h, do)
+    ext.workspace_status()
+    h_ref = oracle.scan_fwd_f32(alpha.numpy(), beta.numpy())
+    ga_ref, gb_ref = oracle.scan_bwd_f32(alpha.numpy(), h_ref, dout.numpy())
+    for name, got, want in (("h", h, h_ref), ("grad_alpha", ga, ga_ref), ("grad_beta", gb, gb_ref)):
+        got = got.cpu().numpy()
+        assert rel_l2(got, want) < 1e-6, name
+        assert np.allclose(got, want, rtol=1e-4, atol=1e-5), name
+
+
 def test_closed_forms_at_headline_shape():
     """Size-independent properties at the full headline size (bs 8, seq 4096, d 1024)."""
     bs, seq, d = 8, 4096, 1024
