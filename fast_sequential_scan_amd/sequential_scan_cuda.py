@@ -15,6 +15,7 @@ Same names, argument order and return structure.  Differences, all supersets:
 """
 from __future__ import annotations
 
+import contextlib
 from typing import Dict, List, Optional, Tuple
 
 import torch
@@ -68,7 +69,34 @@ def _validate(expected: torch.dtype, **tensors: torch.Tensor) -> Tuple[int, int,
     return int(bs), int(seq), int(d)
 
 
-def _workspace(device: torch.device, stream: torch.cuda.Stream, need: int) -> torch.Tensor:
+class _RawStream:
+    """The current stream of the current device as the launch sites need it: its handle."""
+
+    __slots__ = ("cuda_stream",)
+
+    def __init__(self, handle: int):
+        self.cuda_stream = handle
+
+
+_raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
+_NO_SWITCH = contextlib.nullcontext()
+
+
+def _current_stream() -> "_RawStream":
+    # the raw handle costs a tenth of building a torch.cuda.Stream object per call
+    if _raw_stream is not None:
+        return _RawStream(_raw_stream(torch.cuda.current_device()))
+    return _RawStream(torch.cuda.current_stream().cuda_stream)
+
+
+def _on(device: torch.device):
+    """Context that makes `device` current - nothing to enter when it already is."""
+    if device.index is None or device.index == torch.cuda.current_device():
+        return _NO_SWITCH
+    return torch.cuda.device(device)
+
+
+def _workspace(device: torch.device, stream: "_RawStream", need: int) -> torch.Tensor:
     key = (device.index if device.index is not None else torch.cuda.current_device(), stream.cuda_stream)
     ws = _workspaces.get(key)
     if ws is None or ws.buf.numel() < need:
@@ -86,7 +114,7 @@ def workspace_status(device: Optional[torch.device] = None) -> None:
     """Synchronises the current stream and raises if a chained scan timed out (debug aid)."""
     device = torch.device("cuda", torch.cuda.current_device()) if device is None else device
     with torch.cuda.device(device):
-        stream = torch.cuda.current_stream()
+        stream = _current_stream()
         ws = _workspaces.get((device.index, stream.cuda_stream))
         if ws is not None:
             _native.check(_native.lib().fss_workspace_status(ws.buf.data_ptr(), stream.cuda_stream))
@@ -100,8 +128,8 @@ def _forward(dtype: torch.dtype, alpha: torch.Tensor, beta: torch.Tensor, config
         return out
     lib = _native.lib()
     code = _DTYPE_CODE[dtype]
-    with torch.cuda.device(alpha.device):
-        stream = torch.cuda.current_stream()
+    with _on(alpha.device):
+        stream = _current_stream()
         need = lib.fss_workspace_bytes(bs, seq, d, code, _native.FSS_FWD, _native.make_config(config))
         ws = _workspace(alpha.device, stream, need)
         _native.check(
@@ -124,8 +152,8 @@ def _backward(
         return [grad_alpha, grad_beta]
     lib = _native.lib()
     code = _DTYPE_CODE[dtype]
-    with torch.cuda.device(alpha_saved.device):
-        stream = torch.cuda.current_stream()
+    with _on(alpha_saved.device):
+        stream = _current_stream()
         need = lib.fss_workspace_bytes(bs, seq, d, code, _native.FSS_BWD, _native.make_config(config))
         ws = _workspace(alpha_saved.device, stream, need)
         _native.check(
@@ -203,8 +231,8 @@ def scan_forward_state(
         return out, h_last
     lib = _native.lib()
     code = _DTYPE_CODE[dtype]
-    with torch.cuda.device(alpha.device):
-        stream = torch.cuda.current_stream()
+    with _on(alpha.device):
+        stream = _current_stream()
         need = lib.fss_workspace_bytes(bs, seq, d, code, _native.FSS_FWD, _native.make_config(config))
         ws = _workspace(alpha.device, stream, need)
         _native.check(
@@ -242,8 +270,8 @@ def scan_backward_state(
         return grad_alpha, grad_beta, grad_h_before
     lib = _native.lib()
     code = _DTYPE_CODE[dtype]
-    with torch.cuda.device(alpha_saved.device):
-        stream = torch.cuda.current_stream()
+    with _on(alpha_saved.device):
+        stream = _current_stream()
         need = lib.fss_workspace_bytes(bs, seq, d, code, _native.FSS_BWD, _native.make_config(config))
         ws = _workspace(alpha_saved.device, stream, need)
         _native.check(
@@ -280,8 +308,8 @@ def gated_scan_forward(gate: torch.Tensor, x: torch.Tensor, config=None) -> torc
     lib = _native.lib()
     code = _DTYPE_CODE[dtype]
     cfg = _native.make_config(config)
-    with torch.cuda.device(gate.device):
-        stream = torch.cuda.current_stream()
+    with _on(gate.device):
+        stream = _current_stream()
         ws = _workspace(gate.device, stream, lib.fss_workspace_bytes(bs, seq, d, code, _native.FSS_GATED_FWD, cfg))
         _native.check(
             lib.fss_gated_scan_fwd(
@@ -306,8 +334,8 @@ def gated_scan_backward(
     lib = _native.lib()
     code = _DTYPE_CODE[dtype]
     cfg = _native.make_config(config)
-    with torch.cuda.device(gate.device):
-        stream = torch.cuda.current_stream()
+    with _on(gate.device):
+        stream = _current_stream()
         ws = _workspace(gate.device, stream, lib.fss_workspace_bytes(bs, seq, d, code, _native.FSS_GATED_BWD, cfg))
         _native.check(
             lib.fss_gated_scan_bwd(
@@ -337,8 +365,8 @@ def gated_scan_forward_state(
     lib = _native.lib()
     code = _DTYPE_CODE[dtype]
     cfg = _native.make_config(config)
-    with torch.cuda.device(gate.device):
-        stream = torch.cuda.current_stream()
+    with _on(gate.device):
+        stream = _current_stream()
         ws = _workspace(gate.device, stream, lib.fss_workspace_bytes(bs, seq, d, code, _native.FSS_GATED_FWD, cfg))
         _native.check(
             lib.fss_gated_scan_fwd_state(
@@ -375,8 +403,8 @@ def gated_scan_backward_state(
     lib = _native.lib()
     code = _DTYPE_CODE[dtype]
     cfg = _native.make_config(config)
-    with torch.cuda.device(gate.device):
-        stream = torch.cuda.current_stream()
+    with _on(gate.device):
+        stream = _current_stream()
         ws = _workspace(gate.device, stream, lib.fss_workspace_bytes(bs, seq, d, code, _native.FSS_GATED_BWD, cfg))
         _native.check(
             lib.fss_gated_scan_bwd_state(
@@ -406,8 +434,8 @@ def scan_forward_cm(alpha: torch.Tensor, beta: torch.Tensor, config=None) -> tor
     lib = _native.lib()
     code = _DTYPE_CODE[dtype]
     cfg = _native.make_config(config)
-    with torch.cuda.device(alpha.device):
-        stream = torch.cuda.current_stream()
+    with _on(alpha.device):
+        stream = _current_stream()
         ws = _workspace(alpha.device, stream, lib.fss_cm_workspace_bytes(bs, d, seq, code, _native.FSS_FWD, cfg))
         _native.check(
             lib.fss_scan_fwd_cm(
@@ -432,8 +460,8 @@ def scan_backward_cm(
     lib = _native.lib()
     code = _DTYPE_CODE[dtype]
     cfg = _native.make_config(config)
-    with torch.cuda.device(alpha_saved.device):
-        stream = torch.cuda.current_stream()
+    with _on(alpha_saved.device):
+        stream = _current_stream()
         ws = _workspace(alpha_saved.device, stream, lib.fss_cm_workspace_bytes(bs, d, seq, code, _native.FSS_BWD, cfg))
         _native.check(
             lib.fss_scan_bwd_cm(
