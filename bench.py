@@ -64,6 +64,8 @@ def parse_args():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline / parity leg")
     ap.add_argument("--cpu-seconds", type=float, default=12.0, help="budget of the CPU baseline leg")
     ap.add_argument("--flush-mb", type=int, default=1024, help="size of the cache-flush read for the cold timings")
+    ap.add_argument("--cache-policy", default="auto", choices=("auto", "streaming"),
+                    help="fss_set_cache_policy for the run (streaming: assume nothing is found in the caches again)")
     ap.add_argument("--sweep", action="store_true",
                     help="the reference's benchmark sweep (benchmark.py:37-110): sequence lengths 128..32768 at "
                          "--sweep-bs x --sweep-d, forward and forward+backward through the public autograd API, "
@@ -176,6 +178,7 @@ def main() -> int:
                           "unit": "GB/s (read+write)"}))
         return 0
 
+    ext.set_cache_policy(args.cache_policy)
     if args.sweep:
         return sweep(args, torch, scan_cu, dev)
 
@@ -490,6 +493,7 @@ def main() -> int:
         "dtype": args.dtype,
         "data": "synthetic",
         "tensor_sets_in_rotation": len(pointer_sets),
+        "cache_policy": args.cache_policy,
         "config": {
             "workload": f"{args.case}: bs{bs} seq{seq} d{d}, {'gated scan of N(0,1) gate and x' if gated else 'recipe ' + recipe}{', tensors (bs, d, seq)' if cm else ''}, {args.dtype} storage / fp32 carries, forward+backward",
             "bs": bs, "seq": seq, "d_model": d,

@@ -9,12 +9,13 @@ from .scan_cuda import (SequentialScan, SequentialScanGated, SequentialScanGated
                         SequentialScanState, SequentialScanChannelMajor, scan_cm, scan_gated,
                         scan_gated_with_state, scan_with_state)
 from .scan_cuda import scan as scan_cu
+from .sequential_scan_cuda import set_cache_policy
 from .scan_cuda import scan_fp16 as scan_cu_fp16
 from .scan_cuda import scan_single as scan_cu_single
 
 __all__ = [
     "scan_cu", "scan_cu_single", "scan_cu_fp16", "scan_tr", "scan_with_state", "scan_gated", "scan_gated_with_state",
-    "scan_cm",
+    "scan_cm", "set_cache_policy",
     "SequentialScan", "SequentialScanSingle", "SequentialScanState", "SequentialScanGated", "SequentialScanGatedState",
     "SequentialScanChannelMajor",
 ]

@@ -17,6 +17,7 @@ LIB_PATH = os.environ.get("FSS_SCAN_LIBRARY") or os.path.join(PKG_DIR, "_lib", "
 FSS_BF16, FSS_F32, FSS_F16 = 0, 1, 2
 FSS_FWD, FSS_BWD, FSS_GATED_FWD, FSS_GATED_BWD = 0, 1, 2, 3
 FSS_OK = 0
+FSS_CACHE_AUTO, FSS_CACHE_STREAMING = 0, 1
 FSS_ERR_CHAIN_TIMEOUT = 7
 
 EXPORTED_SYMBOLS = (
@@ -38,6 +39,7 @@ EXPORTED_SYMBOLS = (
     "fss_scan_bwd_state",
     "fss_gated_scan_fwd",
     "fss_gated_scan_bwd",
+    "fss_set_cache_policy",
     "fss_gated_scan_fwd_state",
     "fss_gated_scan_bwd_state",
     "fss_cm_workspace_bytes",
@@ -109,6 +111,8 @@ def _declare(lib: ctypes.CDLL) -> None:
     lib.fss_copy_bytes.restype = _int
     lib.fss_gated_scan_fwd.restype = _int
     lib.fss_gated_scan_fwd.argtypes = [_int, _vp, _vp, _vp, _i64, _i64, _i64, _vp, _sz, _vp, _cfgp]
+    lib.fss_set_cache_policy.restype = _int
+    lib.fss_set_cache_policy.argtypes = [_int]
     lib.fss_gated_scan_fwd_state.restype = _int
     lib.fss_gated_scan_fwd_state.argtypes = [_int, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _vp, _sz, _vp, _cfgp]
     lib.fss_gated_scan_bwd_state.restype = _int

@@ -24,6 +24,8 @@ __global__ void copy_kernel(const u32x4 *__restrict__ src, u32x4 *__restrict__ d
     dst[i] = src[i];
 }
 
+int g_cache_policy = FSS_CACHE_AUTO;  // fss_set_cache_policy
+
 int run_scan(int dtype, int dir, const void *alpha, const void *in_b, const void *in_h, void *out0,
              void *out1, int64_t bs, int64_t seq, int64_t d, void *workspace, size_t workspace_bytes,
              void *stream, const fss_config *cfg, const float *state_in = nullptr,
@@ -69,7 +71,10 @@ int run_scan(int dtype, int dir, const void *alpha, const void *in_b, const void
   args.n_tiles = static_cast<int32_t>(pl.n_tiles);
   args.look_waves = look_waves(pl.cfg.waves, pl.cfg.vec);
   const int64_t tensor_bytes = bs * seq * d * static_cast<int64_t>(esize);
-  pl.alt_policy = !gated && (dir == FSS_FWD ? tensor_bytes <= kKeepOutBytes : tensor_bytes > kStreamDoutBytes);
+  if (__atomic_load_n(&g_cache_policy, __ATOMIC_RELAXED) == FSS_CACHE_STREAMING)
+    pl.alt_policy = !gated && dir == FSS_BWD;
+  else
+    pl.alt_policy = !gated && (dir == FSS_FWD ? tensor_bytes <= kKeepOutBytes : tensor_bytes > kStreamDoutBytes);
   const StateArgs<true> state = {state_in, state_out, h_before};
   args.hdr = static_cast<uint32_t *>(workspace);
   args.words = workspace ? reinterpret_cast<uint64_t *>(static_cast<char *>(workspace) + kHeaderBytes) : nullptr;
@@ -98,6 +103,11 @@ void fss_debug_set_trace(void *p) { fss::g_trace = static_cast<uint64_t *>(p); }
 #endif
 
 int fss_abi_version(void) { return FSS_ABI_VERSION; }
+
+int fss_set_cache_policy(int policy) {
+  if (policy != FSS_CACHE_AUTO && policy != FSS_CACHE_STREAMING) return -1;
+  return __atomic_exchange_n(&fss::g_cache_policy, policy, __ATOMIC_RELAXED);
+}
 
 const char *fss_strerror(int status) {
   switch (status) {

@@ -27,7 +27,7 @@ __all__ = [
     "scan_forward_fp16", "scan_backward_fp16",
     "scan_forward_state", "scan_backward_state",
     "gated_scan_forward", "gated_scan_backward", "gated_scan_forward_state", "gated_scan_backward_state",
-    "scan_forward_cm", "scan_backward_cm",
+    "scan_forward_cm", "scan_backward_cm", "set_cache_policy",
 ]
 
 _DTYPE_CODE = {torch.bfloat16: _native.FSS_BF16, torch.float32: _native.FSS_F32, torch.float16: _native.FSS_F16}
@@ -108,6 +108,21 @@ def _workspace(device: torch.device, stream: "_RawStream", need: int) -> torch.T
         ws.launches = 0
     ws.launches += 1
     return ws.buf
+
+
+_CACHE_POLICIES = {"auto": _native.FSS_CACHE_AUTO, "streaming": _native.FSS_CACHE_STREAMING}
+
+
+def set_cache_policy(policy: str) -> str:
+    """Process-wide: ``"auto"`` (default) assumes the tensors of a step are touched again soon (a
+    benchmark loop, a short pipeline); ``"streaming"`` assumes nothing is found in the memory-side
+    cache again (a scan inside a large model) and marks the forward's output and the backward's
+    reads of ``dout`` as streaming at every size.  Results are bit-identical.  Returns the previous
+    policy."""
+    if policy not in _CACHE_POLICIES:
+        raise ValueError(f"unknown cache policy {policy!r}: expected one of {sorted(_CACHE_POLICIES)}")
+    previous = _native.lib().fss_set_cache_policy(_CACHE_POLICIES[policy])
+    return next(name for name, code in _CACHE_POLICIES.items() if code == previous)
 
 
 def workspace_status(device: Optional[torch.device] = None) -> None:

@@ -158,6 +158,21 @@ int fss_scan_bwd_f32(const void *alpha, const void *h, const void *dout,
                      int64_t d, void *workspace, size_t workspace_bytes,
                      void *stream);
 
+/*
+ * How the scans treat the memory-side cache (process-wide; no counterpart in the reference).
+ *   FSS_CACHE_AUTO       (default) assumes that the tensors of a step are touched again soon,
+ *                        as in a benchmark loop or a short pipeline: a small forward output is
+ *                        left in the cache for its reader, and the backward reads dout with the
+ *                        streaming hint only when the inputs of a step cannot fit the cache.
+ *   FSS_CACHE_STREAMING  assumes that nothing is found in the cache again (a scan inside a
+ *                        large model): the forward output always carries the streaming hint and
+ *                        the backward always reads dout with it (measured 2-3 % faster then, 3 % slower in a loop
+ *                        over one set of tensors).
+ * Results are bit-identical under both.  Returns the previous policy, or -1 for an unknown one.
+ */
+enum fss_cache_policy { FSS_CACHE_AUTO = 0, FSS_CACHE_STREAMING = 1 };
+int fss_set_cache_policy(int policy);
+
 /* Same four operations with an explicit dtype and launch configuration (tuning,
  * and tests that results do not depend on how the sequence is chunked). */
 int fss_scan_fwd_ex(int dtype, const void *alpha, const void *beta, void *h,

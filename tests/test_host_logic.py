@@ -239,3 +239,15 @@ def test_common_helpers_follow_their_definitions(oracle):
     assert check_relative_error(0.0, 7) and check_relative_error(1e-8, 7) and check_relative_error(9e-7, 7)
     assert not check_relative_error(1.1e-6, 7)
     assert check_relative_error(0.09, 2) and not check_relative_error(0.11, 2)
+
+
+def test_cache_policy_setter():
+    import fast_sequential_scan_amd as pkg
+
+    lib = _native.lib()
+    assert lib.fss_set_cache_policy(7) == -1  # unknown: refused, nothing changes
+    assert pkg.set_cache_policy("streaming") == "auto"
+    assert pkg.set_cache_policy("auto") == "streaming"
+    assert lib.fss_set_cache_policy(_native.FSS_CACHE_AUTO) == _native.FSS_CACHE_AUTO
+    with pytest.raises(ValueError):
+        pkg.set_cache_policy("hot")

@@ -205,6 +205,27 @@ def test_fp32_at_headline_shape(oracle):
         assert np.allclose(got, want, rtol=1e-4, atol=1e-5), name
 
 
+def test_cache_policies_give_identical_results():
+    """The streaming policy only changes cache hints: every output bit stays.  Shapes on both sides
+    of the sizes at which the automatic policy switches."""
+    import fast_sequential_scan_amd as pkg
+
+    for shape in ((4, 1000, 512), (8, 4096, 1024)):
+        alpha, beta, dout = make_inputs("sigmoid", *shape, seed=84)
+        a, b, do = alpha.to(DEV), beta.to(DEV), dout.to(DEV)
+        results = {}
+        for policy in ("auto", "streaming"):
+            previous = pkg.set_cache_policy(policy)
+            try:
+                h = ext.scan_forward_half(a, b)
+                results[policy] = (h, *ext.scan_backward_half(a, h, do))
+            finally:
+                pkg.set_cache_policy(previous)
+        for x, y in zip(results["auto"], results["streaming"]):
+            assert torch.equal(x, y)
+    ext.workspace_status()
+
+
 def test_closed_forms_at_headline_shape():
     """Size-independent properties at the full headline size (bs 8, seq 4096, d 1024)."""
     bs, seq, d = 8, 4096, 1024
