@@ -251,3 +251,14 @@ def test_cache_policy_setter():
     assert lib.fss_set_cache_policy(_native.FSS_CACHE_AUTO) == _native.FSS_CACHE_AUTO
     with pytest.raises(ValueError):
         pkg.set_cache_policy("hot")
+
+
+def test_bench_refuses_more_than_one_gpu():
+    import subprocess
+    import sys
+
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    proc = subprocess.run([sys.executable, os.path.join(root, "bench.py"), "--gpus", "2"],
+                          capture_output=True, text=True, timeout=120)
+    assert proc.returncode == 2
+    assert "one GPU" in proc.stderr and proc.stdout.strip() == ""
