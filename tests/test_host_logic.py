@@ -262,3 +262,37 @@ def test_bench_refuses_more_than_one_gpu():
                           capture_output=True, text=True, timeout=120)
     assert proc.returncode == 2
     assert "one GPU" in proc.stderr and proc.stdout.strip() == ""
+
+
+def test_chosen_configurations_are_valid_for_random_shapes():
+    """Property test of the launch planning: whatever the shape, storage type, direction and
+    alignment, the chosen configuration is one the kernels accept, never reaches further than the
+    sequence needs, and sizes a workspace within the shape's upper bound."""
+    rng = np.random.default_rng(2024)
+    lib = _native.lib()
+    cfg = _native.FssConfig()
+    for _ in range(4000):
+        bs = int(rng.choice([1, 2, 3, 7, 8, 16, 64, 250]))
+        seq = int(rng.choice([1, 2, 5, 31, 64, 255, 256, 257, 1000, 2048, 3000, 4096, 8192, 40000, 65521, 300000]))
+        d = int(rng.choice([1, 2, 3, 63, 64, 65, 126, 128, 200, 256, 768, 1024, 1537, 2560, 4096]))
+        dtype = int(rng.integers(0, 3))
+        direction = int(rng.integers(0, 4))
+        align = int(rng.choice([2, 4, 8, 16])) if dtype != _native.FSS_F32 else int(rng.choice([4, 8, 16]))
+        what = (bs, seq, d, dtype, direction, align)
+        assert lib.fss_choose_config(bs, seq, d, dtype, direction, align, ctypes.byref(cfg)) == 0, what
+        esize = 4 if dtype == _native.FSS_F32 else 2
+        gated, backward = direction >= 2, direction % 2 == 1
+        assert cfg.vec in (1, 2) and d % cfg.vec == 0 and align % (cfg.vec * esize) == 0, what
+        assert cfg.steps in (8, 16, 32) and 1 <= cfg.waves <= 16, what
+        if gated:
+            assert cfg.vec <= (1 if dtype == _native.FSS_F32 else 2), what
+            assert not backward or cfg.steps <= 16, what
+        # the tile is no longer than the sequence needs: half of it would not cover the sequence
+        assert cfg.waves == 1 or cfg.steps * (cfg.waves // 2) < seq, what
+        assert cfg.steps == 8 or cfg.steps // 2 < seq, what
+        need = lib.fss_workspace_bytes(bs, seq, d, dtype, direction, None)
+        assert 4096 <= need <= lib.fss_workspace_bytes_max(bs, seq, d), what
+        # the explicit form of the same configuration is accepted and sizes the same workspace
+        explicit = _native.FssConfig(cfg.vec, cfg.steps, cfg.waves, 0)
+        if align >= 16:  # fss_workspace_bytes plans for 16-byte aligned tensors
+            assert lib.fss_workspace_bytes(bs, seq, d, dtype, direction, ctypes.byref(explicit)) == need, what
