@@ -139,3 +139,29 @@ def test_channel_major_scans(oracle, seed):
     _check(gb.transpose(1, 2), gb_or, dtype, what + " grad_beta")
     _check(ga.transpose(1, 2), ga_or, dtype, what + " grad_alpha")
     ext.workspace_status()
+
+
+# Mid-size shapes whose lengths and widths are no powers of two, with the library's own
+# choices: they land on different rungs of the planning ladder (16- and 8-wave workgroups,
+# one and two channels per lane, ragged last chunks and column tiles).
+DEFAULT_CHOICE_SHAPES = [
+    (3, 3000, 1536), (8, 3000, 1024), (5, 1500, 2560), (2, 5000, 768), (1, 12000, 520),
+    (7, 700, 200), (2, 6000, 1030), (16, 1000, 384), (1, 40000, 130), (4, 2049, 1537),
+]
+
+
+@pytest.mark.parametrize("shape", DEFAULT_CHOICE_SHAPES, ids=[str(s) for s in DEFAULT_CHOICE_SHAPES])
+def test_library_choices_at_odd_mid_size_shapes(oracle, shape):
+    rng = np.random.default_rng(sum(shape))
+    for dtype in (torch.bfloat16, torch.float32):
+        alpha, beta, dout = _tensors(rng, shape, dtype)
+        a, b, do = alpha.to(DEV), beta.to(DEV), dout.to(DEV)
+        h = ext._forward(dtype, a, b)
+        ga, gb = ext._backward(dtype, a, h, do)
+        a32, b32, d32 = alpha.float().numpy(), beta.float().numpy(), dout.float().numpy()
+        what = f"{dtype} {shape}"
+        _check(h, oracle.scan_fwd_f32(a32, b32), dtype, what + " h")
+        ga_or, gb_or = oracle.scan_bwd_f32(a32, h.float().cpu().numpy(), d32)
+        _check(gb, gb_or, dtype, what + " grad_beta")
+        _check(ga, ga_or, dtype, what + " grad_alpha")
+    ext.workspace_status()
