@@ -11,11 +11,15 @@ uint64_t *g_trace = nullptr;
 #endif
 ScanOrder g_scan_order[64];
 
-// Zero everywhere (tag 0 = "never written"), launch counter starting at 1.
+// Zero everywhere: tag 0 = "never written", and the first launch takes tag 1.
 __global__ void workspace_init_kernel(uint32_t *p, size_t n_words) {
   const size_t stride = static_cast<size_t>(gridDim.x) * blockDim.x;
-  for (size_t i = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x; i < n_words; i += stride)
-    p[i] = (i == HDR_EPOCH) ? 1u : 0u;
+  for (size_t i = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x; i < n_words; i += stride) p[i] = 0u;
+}
+
+__global__ void workspace_attach_kernel(uint32_t *hdr, uint64_t flag_address) {
+  hdr[HDR_FLAG_LO] = static_cast<uint32_t>(flag_address);
+  hdr[HDR_FLAG_HI] = static_cast<uint32_t>(flag_address >> 32);
 }
 
 __global__ void copy_kernel(const u32x4 *__restrict__ src, u32x4 *__restrict__ dst, size_t n_vec) {
@@ -25,6 +29,7 @@ __global__ void copy_kernel(const u32x4 *__restrict__ src, u32x4 *__restrict__ d
 }
 
 int g_cache_policy = FSS_CACHE_AUTO;  // fss_set_cache_policy
+uint32_t g_spin_limit = kSpinLimit;    // fss_debug_set_spin_limit
 
 int run_scan(int dtype, int dir, const void *alpha, const void *in_b, const void *in_h, void *out0,
              void *out1, int64_t bs, int64_t seq, int64_t d, void *workspace, size_t workspace_bytes,
@@ -70,6 +75,7 @@ int run_scan(int dtype, int dir, const void *alpha, const void *in_b, const void
   args.n_chunks = static_cast<int32_t>(pl.n_chunks);
   args.n_tiles = static_cast<int32_t>(pl.n_tiles);
   args.look_waves = look_waves(pl.cfg.waves, pl.cfg.vec);
+  args.spin_limit = __atomic_load_n(&g_spin_limit, __ATOMIC_RELAXED);
   const int64_t tensor_bytes = bs * seq * d * static_cast<int64_t>(esize);
   if (__atomic_load_n(&g_cache_policy, __ATOMIC_RELAXED) == FSS_CACHE_STREAMING)
     pl.alt_policy = !gated && dir == FSS_BWD;
@@ -127,11 +133,15 @@ const char *fss_strerror(int status) {
 int fss_last_hip_error(void) { return fss::tls_hip_error; }
 
 size_t fss_workspace_bytes(int64_t bs, int64_t seq, int64_t d, int dtype, int dir, const fss_config *cfg) {
-  fss::Plan pl;
-  // alignment unknown here: assume the best the shape allows (the widest vector,
-  // hence the most words per tile, is what a less aligned call can only shrink)
-  if (fss::make_plan(pl, bs, seq, d, dtype, dir, 16, cfg) != FSS_OK) return fss::kHeaderBytes;
-  return pl.ws_bytes;
+  // The tensors' alignment is unknown here and changes the plan (less aligned tensors take
+  // fewer channels per lane, which can mean more, smaller tiles and more chaining words):
+  // the answer covers every alignment.
+  size_t best = fss::kHeaderBytes;
+  for (size_t align = 2; align <= 16; align <<= 1) {
+    fss::Plan pl;
+    if (fss::make_plan(pl, bs, seq, d, dtype, dir, align, cfg) == FSS_OK && pl.ws_bytes > best) best = pl.ws_bytes;
+  }
+  return best;
 }
 
 size_t fss_workspace_bytes_max(int64_t bs, int64_t seq, int64_t d) {
@@ -170,6 +180,24 @@ int fss_workspace_init(void *workspace, size_t bytes, void *stream) {
     return FSS_ERR_LAUNCH;
   }
   return FSS_OK;
+}
+
+int fss_workspace_attach_flag(void *workspace, uint32_t *flag, void *stream) {
+  if (!workspace) return FSS_ERR_NULL_POINTER;
+  if (reinterpret_cast<uintptr_t>(workspace) % 256 != 0 || reinterpret_cast<uintptr_t>(flag) % 4 != 0)
+    return FSS_ERR_MISALIGNED;
+  hipLaunchKernelGGL(fss::workspace_attach_kernel, dim3(1), dim3(1), 0, static_cast<hipStream_t>(stream),
+                     static_cast<uint32_t *>(workspace), static_cast<uint64_t>(reinterpret_cast<uintptr_t>(flag)));
+  const hipError_t e = hipGetLastError();
+  if (e != hipSuccess) {
+    fss::tls_hip_error = static_cast<int>(e);
+    return FSS_ERR_LAUNCH;
+  }
+  return FSS_OK;
+}
+
+uint32_t fss_debug_set_spin_limit(uint32_t polls) {
+  return __atomic_exchange_n(&fss::g_spin_limit, polls, __ATOMIC_RELAXED);
 }
 
 int fss_workspace_status(void *workspace, void *stream) {

@@ -218,16 +218,21 @@ __device__ __forceinline__ void keep_packed(RowT &r) {
 
 // ---- workspace ----------------------------------------------------------------
 //
-// Header (kHeaderBytes): word 1 = top-level completion counter, word 2 = epoch,
-// word 3 = sticky error flag, words 64+32*i (i < 16, one 128-byte line each) =
-// first-level completion counters.  Then the tagged words,
+// Header (kHeaderBytes): word 1 = top-level completion counter, word 2 = epoch (the tag
+// of the next launch minus 1: an all-zero workspace is ready for use),
+// word 3 = sticky error flag, words 4-5 = address of an optional 32-bit word the host
+// can read without a device call (0: none), which a wave that gives up also sets,
+// words 64+32*i (i < 16, one 128-byte line each) = first-level completion counters.
+// Then the tagged words,
 // [chunk][column tile][kind: map A, map B, outgoing state][VEC][64 lanes].
 
-enum : int { HDR_DONE = 1, HDR_EPOCH = 2, HDR_ERROR = 3, HDR_SLOT0 = 64, HDR_SLOT_STRIDE = 32 };
+enum : int { HDR_DONE = 1, HDR_EPOCH = 2, HDR_ERROR = 3, HDR_FLAG_LO = 4, HDR_FLAG_HI = 5, HDR_SLOT0 = 64, HDR_SLOT_STRIDE = 32 };
 constexpr int kDoneSlots = 16;
 constexpr size_t kHeaderBytes = 4096;
 // Polls a wave makes before it gives up on an earlier chunk (each poll is a memory
-// round trip plus a sleep: seconds in total, far beyond any healthy wait).
+// round trip plus a sleep: seconds in total, far beyond any healthy wait).  The limit
+// travels as a kernel argument so that a test can lower it from the host; 0 makes every
+// look-back give up before its first poll.
 constexpr uint32_t kSpinLimit = 1u << 20;
 // Most waves of a workgroup that look back in parallel, one earlier chunk each.
 constexpr int kMaxLookWaves = 16;
@@ -255,6 +260,25 @@ __device__ __forceinline__ void st_word(uint64_t *p, uint32_t tag, float v) {
 __device__ __forceinline__ uint32_t word_tag(uint64_t w) { return static_cast<uint32_t>(w >> 32); }
 __device__ __forceinline__ float word_val(uint64_t w) { return as_f32(static_cast<uint32_t>(w)); }
 
+// a*x + b where x is a state (or the constant part of a composed map) and a the
+// coefficient it meets.  A coefficient that is a product of many |alpha| > 1 may have
+// overflowed to inf while x is exactly 0; the sequential recurrence keeps such a state
+// at 0, inf*0 would make it NaN.  (A NaN x - the mark of a look-back that gave up -
+// still propagates.)
+__device__ __forceinline__ float fma0(float a, float x, float b) {
+  return x == 0.0f ? b : __builtin_fmaf(a, x, b);
+}
+
+// A wave that gives up on an earlier chunk: sticky error word, the host-visible word
+// if one is attached, and (by the caller) a NaN state, so that every output from here
+// to the end of the sequence is visibly poisoned.
+__device__ __forceinline__ void report_timeout(uint32_t *hdr) {
+  st_u32(hdr + HDR_ERROR, 1u);
+  const uint64_t addr = (static_cast<uint64_t>(ld_u32(hdr + HDR_FLAG_HI)) << 32) | ld_u32(hdr + HDR_FLAG_LO);
+  if (addr != 0)
+    __hip_atomic_store(reinterpret_cast<uint32_t *>(addr), 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+}
+
 struct ScanArgs {
   const char *in_a;  // alpha
   const char *in_b;  // beta (forward) / dout (backward)
@@ -268,6 +292,7 @@ struct ScanArgs {
   int32_t n_chunks;       // ceil(seq / (WAVES*STEPS))
   int32_t n_tiles;        // n_ctiles * n_chunks
   int32_t look_waves;     // waves that look back in parallel (1..min(WAVES, kMaxLookWaves))
+  uint32_t spin_limit;    // polls before a look-back gives up (kSpinLimit unless a test lowered it)
   uint32_t *hdr;          // workspace header
   uint64_t *words;        // tagged words
   const char *in_x;       // gated backward only: the scan's input x (in_a is the gate there)
@@ -450,7 +475,7 @@ __device__ __forceinline__ void fold_wave_maps(const float2 *lds_map, int lane, 
       if (w0 + i < count) {
 #pragma unroll
         for (int v = 0; v < VEC; ++v) {
-          B[v] = __builtin_fmaf(m[i][v].x, B[v], m[i][v].y);
+          B[v] = fma0(m[i][v].x, B[v], m[i][v].y);
           A[v] *= m[i][v].x;
         }
       }
@@ -513,10 +538,10 @@ __device__ __forceinline__ void chain_chunks(const ScanArgs &p, const TileCtx &c
     if (wave == 0 && c.chained && !c.last) {
 #pragma unroll
       for (int v = 0; v < VEC; ++v)
-        st_word(mine + (2 * VEC + v) * 64, c.tag, seq_in ? __builtin_fmaf(cA[v], seq_in[v], cB[v]) : cB[v]);
+        st_word(mine + (2 * VEC + v) * 64, c.tag, seq_in ? fma0(cA[v], seq_in[v], cB[v]) : cB[v]);
     }
 #pragma unroll
-    for (int v = 0; v < VEC; ++v) state[v] = seq_in ? __builtin_fmaf(pA[v], seq_in[v], pB[v]) : pB[v];
+    for (int v = 0; v < VEC; ++v) state[v] = seq_in ? fma0(pA[v], seq_in[v], pB[v]) : pB[v];
     FSS_STAMP(c, p, 5);
     return;
   }
@@ -557,14 +582,22 @@ __device__ __forceinline__ void chain_chunks(const ScanArgs &p, const TileCtx &c
         qB[v] = q0B[v];
       }
       kind0 = kPredNone;
-      while (kind == kPredNone && (kind = poll_chunk<VEC>(p, c, j, qA, qB)) == kPredNone) {
-        if (++polls > kSpinLimit) {
-          if (lane == 0) st_u32(p.hdr + HDR_ERROR, 1u);
-          kind = kPredState;  // give up: zero state, so that the grid still drains
+      if (p.spin_limit == 0) kind = kPredNone;
+      while (kind == kPredNone) {
+        if (polls >= p.spin_limit) {
+          // give up, so that the grid still drains: a NaN state poisons what follows
+          if (lane == 0) report_timeout(p.hdr);
+          kind = kPredState;
 #pragma unroll
-          for (int v = 0; v < VEC; ++v) qA[v] = qB[v] = 0.0f;
+          for (int v = 0; v < VEC; ++v) {
+            qA[v] = 0.0f;
+            qB[v] = __builtin_nanf("");
+          }
           break;
         }
+        kind = poll_chunk<VEC>(p, c, j, qA, qB);
+        if (kind != kPredNone) break;
+        ++polls;
         __builtin_amdgcn_s_sleep(2);
       }
       // long chains: the wave also takes the chunks before that one (by now they have nearly
@@ -572,20 +605,26 @@ __device__ __forceinline__ void chain_chunks(const ScanArgs &p, const TileCtx &c
       for (int k = 1; k < c.span && kind == kPredMap && j - k >= 0; ++k) {
         float rA[VEC], rB[VEC];
         polls = 0;
-        while ((kind = poll_chunk<VEC>(p, c, j - k, rA, rB)) == kPredNone) {
-          if (++polls > kSpinLimit) {
-            if (lane == 0) st_u32(p.hdr + HDR_ERROR, 1u);
+        for (;;) {
+          if (polls >= p.spin_limit) {
+            if (lane == 0) report_timeout(p.hdr);
             kind = kPredState;
 #pragma unroll
-            for (int v = 0; v < VEC; ++v) rA[v] = rB[v] = 0.0f;
+            for (int v = 0; v < VEC; ++v) {
+              rA[v] = 0.0f;
+              rB[v] = __builtin_nanf("");
+            }
             break;
           }
+          kind = poll_chunk<VEC>(p, c, j - k, rA, rB);
+          if (kind != kPredNone) break;
+          ++polls;
           __builtin_amdgcn_s_sleep(2);
         }
         // (a state is the map x -> 0*x + value)
 #pragma unroll
         for (int v = 0; v < VEC; ++v) {
-          qB[v] = __builtin_fmaf(qA[v], rB[v], qB[v]);
+          qB[v] = fma0(qA[v], rB[v], qB[v]);
           qA[v] *= rA[v];
         }
       }
@@ -603,9 +642,9 @@ __device__ __forceinline__ void chain_chunks(const ScanArgs &p, const TileCtx &c
       for (int v = 0; v < VEC; ++v) {
         const float2 m = c.lds_pred[(w * VEC + v) * 64 + lane];
         if (is_state) {
-          hin[v] = __builtin_fmaf(accA[v], m.y, accB[v]);
+          hin[v] = fma0(accA[v], m.y, accB[v]);
         } else {
-          accB[v] = __builtin_fmaf(accA[v], m.y, accB[v]);
+          accB[v] = fma0(accA[v], m.y, accB[v]);
           accA[v] *= m.x;
         }
       }
@@ -615,13 +654,13 @@ __device__ __forceinline__ void chain_chunks(const ScanArgs &p, const TileCtx &c
       if (wave == 0 && !c.last) {
 #pragma unroll
         for (int v = 0; v < VEC; ++v)
-          st_word(mine + (2 * VEC + v) * 64, c.tag, __builtin_fmaf(cA[v], hin[v], cB[v]));
+          st_word(mine + (2 * VEC + v) * 64, c.tag, fma0(cA[v], hin[v], cB[v]));
       }
       break;
     }
     nearest -= c.look * c.span;
     if (nearest < 0) {  // cannot happen; never spin on a logic error
-      if (threadIdx.x == 0) st_u32(p.hdr + HDR_ERROR, 1u);
+      if (threadIdx.x == 0) report_timeout(p.hdr);
       break;
     }
     __syncthreads();  // the slots are about to be overwritten: wait until every wave has read them
@@ -629,7 +668,7 @@ __device__ __forceinline__ void chain_chunks(const ScanArgs &p, const TileCtx &c
   FSS_STAMP(c, p, 4);
   fold_wave_maps<VEC>(c.lds_map, lane, wave, pA, pB);  // after the polls: those are what is waited for
 #pragma unroll
-  for (int v = 0; v < VEC; ++v) state[v] = __builtin_fmaf(pA[v], hin[v], pB[v]);
+  for (int v = 0; v < VEC; ++v) state[v] = fma0(pA[v], hin[v], pB[v]);
   FSS_STAMP(c, p, 5);
 }
 
@@ -646,8 +685,9 @@ __device__ __forceinline__ void count_out(const ScanArgs &p, const TileCtx &c) {
       const uint32_t slots_used = gridDim.x < kDoneSlots ? gridDim.x : kDoneSlots;
       if (add_u32(p.hdr + HDR_DONE, 1u) == slots_used - 1) {
         st_u32(p.hdr + HDR_DONE, 0u);
-        // 0 is the tag of never-written words: skip it when the counter wraps
-        st_u32(p.hdr + HDR_EPOCH, c.tag + 1u == 0u ? 1u : c.tag + 1u);
+        // the header holds the next launch's tag minus 1, so that zero-filled memory is a
+        // ready workspace; 0 is the tag of never-written words: skip it when the counter wraps
+        st_u32(p.hdr + HDR_EPOCH, (c.tag + 1u == 0u ? 1u : c.tag + 1u) - 1u);
       }
     }
   }

@@ -15,6 +15,7 @@
 namespace fss {
 
 extern thread_local int tls_hip_error;  // hipError_t of this thread's last failed HIP call
+extern uint32_t g_spin_limit;           // polls before a look-back gives up (a test may lower it)
 #ifdef FSS_TRACE
 extern uint64_t *g_trace;
 #endif
@@ -282,22 +283,25 @@ class ScanOrderGuard {
   ScanOrder *order_ = nullptr;
 };
 
-// Workgroups of `kernel` that are certainly resident together on the device (0 on
+inline int cu_count_of_current_device() {
+  static int cached[64];  // by device; 0 = not asked yet
+  int dev = 0, n = 0;
+  if (hipGetDevice(&dev) != hipSuccess) return 0;
+  const bool slot = dev >= 0 && dev < 64;
+  if (slot && (n = __atomic_load_n(&cached[dev], __ATOMIC_RELAXED)) > 0) return n;
+  if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) return 0;
+  if (slot) __atomic_store_n(&cached[dev], n, __ATOMIC_RELAXED);
+  return n;
+}
+
+// Workgroups of `kernel` that are certainly resident together on one compute unit (0 on
 // error).  Deliberately not the runtime's occupancy query: the kernel's waits
 // need a lower bound, and that query bounds by vector registers and LDS only.
 // These kernels hold many scalar registers as well (a row pointer per load); a
 // wave may be allocated 128 of the 800 a SIMD has, which caps a SIMD at 6 waves -
 // the residency measured on MI355X for the scalar-heaviest variants.
 template <typename Kernel>
-int resident_workgroups(Kernel kernel, int waves, size_t lds) {
-  static int cu_count = 0;
-  if (cu_count == 0) {
-    int dev = 0, n = 0;
-    if (hipGetDevice(&dev) != hipSuccess ||
-        hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0)
-      return 0;
-    cu_count = n;
-  }
+int resident_workgroups_per_cu(Kernel kernel, int waves, size_t lds) {
   hipFuncAttributes attr;
   const hipError_t e = hipFuncGetAttributes(&attr, reinterpret_cast<const void *>(kernel));
   if (e != hipSuccess) {
@@ -318,7 +322,21 @@ int resident_workgroups(Kernel kernel, int waves, size_t lds) {
   const int by_lds = static_cast<int>((160 * 1024) / (lds_alloc ? lds_alloc : 1024));
   if (per_cu > by_lds) per_cu = by_lds;
   if (per_cu > 32) per_cu = 32;
-  return per_cu * cu_count;
+  return per_cu;
+}
+
+// The same for the whole current device.  `cache` (one slot per waves-per-workgroup value
+// of one kernel instantiation) keeps the per-CU answer, which is a property of the code
+// object; the CU count is the current device's.
+template <typename Kernel>
+int resident_workgroups(Kernel kernel, int waves, size_t lds, int *cache) {
+  int per_cu = __atomic_load_n(&cache[waves], __ATOMIC_RELAXED);
+  if (per_cu == 0) {
+    per_cu = resident_workgroups_per_cu(kernel, waves, lds);
+    if (per_cu <= 0) return 0;
+    __atomic_store_n(&cache[waves], per_cu, __ATOMIC_RELAXED);
+  }
+  return per_cu * cu_count_of_current_device();
 }
 
 // ---- channel-major planning -------------------------------------------------------------

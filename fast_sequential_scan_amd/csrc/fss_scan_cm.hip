@@ -121,7 +121,7 @@ __device__ __forceinline__ void cm_tile(const ScanArgs &p, const TileCtx &c, int
     for (int r = 0; r < ROWS; ++r) {
       const float pa = __shfl_up(A[r], off), pb = __shfl_up(B[r], off);
       if (lane >= off) {
-        B[r] = __builtin_fmaf(A[r], pb, B[r]);
+        B[r] = fma0(A[r], pb, B[r]);
         A[r] *= pa;
       }
     }
@@ -167,7 +167,7 @@ __device__ __forceinline__ void cm_tile(const ScanArgs &p, const TileCtx &c, int
   }
 #pragma unroll
   for (int r = 0; r < ROWS; ++r) {
-    float state = __builtin_fmaf(A[r], lane_read(slice_in, r), B[r]);
+    float state = fma0(A[r], lane_read(slice_in, r), B[r]);
     float o0[VEC], o1[VEC];
 #pragma unroll
     for (int j = 0; j < VEC; ++j) {
@@ -216,7 +216,7 @@ __global__ __launch_bounds__(1024) void cm_scan_kernel(const ScanArgs p) {
   c.trace_wave = 0;
 #endif
   c.chained = p.n_chunks > 1;
-  c.tag = c.chained ? __builtin_amdgcn_readfirstlane(ld_u32(p.hdr + HDR_EPOCH)) : 0u;
+  c.tag = c.chained ? __builtin_amdgcn_readfirstlane(ld_u32(p.hdr + HDR_EPOCH)) + 1u : 0u;
 
   uint32_t parity = 0;
   for (uint32_t tile = blockIdx.x; tile < static_cast<uint32_t>(p.n_tiles); tile += gridDim.x, parity ^= 1u) {
@@ -239,12 +239,8 @@ int launch_cm_one(const ScanArgs &args, const CmPlan &pl, int max_groups, hipStr
   static int resident[17] = {0};
   const int waves = pl.waves;
   const size_t lds = lds_bytes(waves, 1);
-  int fit = __atomic_load_n(&resident[waves], __ATOMIC_RELAXED);
-  if (fit == 0) {
-    fit = resident_workgroups(cm_scan_kernel<E, VEC, kRows, BWD>, waves, lds);
-    if (fit <= 0) return FSS_ERR_LAUNCH;
-    __atomic_store_n(&resident[waves], fit, __ATOMIC_RELAXED);
-  }
+  const int fit = resident_workgroups(cm_scan_kernel<E, VEC, kRows, BWD>, waves, lds, resident);
+  if (fit <= 0) return FSS_ERR_LAUNCH;
   int64_t n_groups = pl.n_tiles < fit ? pl.n_tiles : fit;
   if (max_groups > 0 && max_groups < n_groups) n_groups = max_groups;
   hipLaunchKernelGGL((cm_scan_kernel<E, VEC, kRows, BWD>), dim3(static_cast<uint32_t>(n_groups)),
@@ -304,6 +300,7 @@ int run_cm_scan(int dtype, int dir, const void *alpha, const void *in_b, const v
   args.n_chunks = static_cast<int32_t>(pl.n_chunks);
   args.n_tiles = static_cast<int32_t>(pl.n_tiles);
   args.look_waves = look_waves(pl.waves, 1);
+  args.spin_limit = __atomic_load_n(&g_spin_limit, __ATOMIC_RELAXED);
   args.hdr = static_cast<uint32_t *>(workspace);
   args.words = workspace ? reinterpret_cast<uint64_t *>(static_cast<char *>(workspace) + kHeaderBytes) : nullptr;
 #ifdef FSS_TRACE

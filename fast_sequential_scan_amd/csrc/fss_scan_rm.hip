@@ -52,8 +52,9 @@
 //   the last one advances the epoch for the next launch.  The counter wraps
 //   after 2^32-1 launches; a host that can get there re-initialises the
 //   workspace first.  Every wait is bounded: a wave that exhausts its budget
-//   records an error in the workspace header and carries on with a zero state,
-//   so the grid always drains.
+//   records an error in the workspace header (and in the host-visible word attached
+//   to the workspace, if any) and carries on with a NaN state, so the grid always
+//   drains and the outputs from there on are visibly poisoned.
 //
 // The backward runs the same machine over reversed time r = seq-1-t with
 // a'[r] = alpha[t+1], b'[r] = dout[t], plus the elementwise g[t]*h[t-1].
@@ -481,7 +482,7 @@ __global__ __launch_bounds__(1024) void scan_kernel(const ScanArgs p, const Stat
 #endif
   c.chained = p.n_chunks > 1;
   // every workgroup of a launch reads the same value: it only changes when all are done
-  c.tag = c.chained ? __builtin_amdgcn_readfirstlane(ld_u32(p.hdr + HDR_EPOCH)) : 0u;
+  c.tag = c.chained ? __builtin_amdgcn_readfirstlane(ld_u32(p.hdr + HDR_EPOCH)) + 1u : 0u;
 
   // The grid is sized to be resident all at once; each workgroup walks tiles
   // blockIdx, blockIdx + gridDim, ...  Tiles are numbered chunk-major, so a tile
@@ -537,15 +538,11 @@ template <typename E, int VEC, int STEPS, bool BWD, bool STATE, bool GATED = fal
 int launch_one(const ScanArgs &args, const StateArgs<true> &state, const Plan &pl, hipStream_t stream) {
   // The kernel's waits are only safe if every workgroup of the grid is resident,
   // so the grid never exceeds what the device holds at once; workgroups loop.
-  static int resident[17] = {0};  // by waves per workgroup; same answer on every call
+  static int resident[17] = {0};  // workgroups per CU by waves per workgroup
   const int waves = pl.cfg.waves;
   const size_t lds = lds_bytes(waves, VEC);
-  int fit = __atomic_load_n(&resident[waves], __ATOMIC_RELAXED);
-  if (fit == 0) {
-    fit = resident_workgroups(scan_kernel<E, VEC, STEPS, BWD, STATE, GATED, ALT>, waves, lds);
-    if (fit <= 0) return FSS_ERR_LAUNCH;
-    __atomic_store_n(&resident[waves], fit, __ATOMIC_RELAXED);
-  }
+  const int fit = resident_workgroups(scan_kernel<E, VEC, STEPS, BWD, STATE, GATED, ALT>, waves, lds, resident);
+  if (fit <= 0) return FSS_ERR_LAUNCH;
   int64_t n_groups = pl.n_tiles < fit ? pl.n_tiles : fit;
   if (pl.cfg.max_groups > 0 && pl.cfg.max_groups < n_groups) n_groups = pl.cfg.max_groups;
   const dim3 grid(static_cast<uint32_t>(n_groups));

@@ -23,21 +23,36 @@ __all__ = [
 ]
 
 
+def _autocast_to_bf16(t: torch.Tensor) -> torch.Tensor:
+    # what torch.amp.custom_fwd(cast_inputs=torch.bfloat16) casts: floating-point GPU tensors
+    if isinstance(t, torch.Tensor) and t.is_cuda and t.is_floating_point() and t.dtype != torch.bfloat16:
+        return t.to(torch.bfloat16)
+    return t
+
+
 class SequentialScan(Function):
     """bf16 scan.  Under ``torch.autocast('cuda')`` floating inputs are cast to
     bf16 and autocast is switched off inside, as the reference's
     ``custom_fwd(cast_inputs=torch.bfloat16)`` does (scan_cuda.py:15); outside
-    autocast a non-bf16 input is an error, as it is there."""
+    autocast a non-bf16 input is an error, as it is there.
+
+    The two decorators of the reference are spelled out here: they build an autocast context
+    per call, tens of microseconds per training step for kernels that take as long, and the
+    backward (``custom_bwd``, scan_cuda.py:25: "run under the forward's autocast state") calls
+    nothing that autocast affects."""
 
     @staticmethod
-    @torch.amp.custom_fwd(device_type="cuda", cast_inputs=torch.bfloat16)
     def forward(ctx: Any, input_alpha: torch.Tensor, input_beta: torch.Tensor) -> torch.Tensor:
-        h = _ext.scan_forward_half(input_alpha, input_beta)
+        if torch.is_autocast_enabled("cuda"):
+            with torch.autocast("cuda", enabled=False):
+                input_alpha, input_beta = _autocast_to_bf16(input_alpha), _autocast_to_bf16(input_beta)
+                h = _ext.scan_forward_half(input_alpha, input_beta)
+        else:
+            h = _ext.scan_forward_half(input_alpha, input_beta)
         ctx.save_for_backward(input_alpha, h)
         return h
 
     @staticmethod
-    @torch.amp.custom_bwd(device_type="cuda")
     @once_differentiable
     def backward(ctx: Any, grad_output: torch.Tensor) -> Tuple[torch.Tensor, torch.Tensor]:
         input_alpha, h = ctx.saved_tensors

@@ -16,6 +16,7 @@ Same names, argument order and return structure.  Differences, all supersets:
 from __future__ import annotations
 
 import contextlib
+import ctypes
 from typing import Dict, List, Optional, Tuple
 
 import torch
@@ -39,17 +40,48 @@ _workspaces: Dict[Tuple[int, int], "_Workspace"] = {}
 # the validity tags in a workspace are a 32-bit launch counter: reset long before it wraps
 _REINIT_AFTER_LAUNCHES = 1 << 31
 
+# bytes of workspace per (entry-point family, dtype code, direction, bs, seq, d, config): the
+# library's answer covers every alignment of the tensors, so it is a pure function of these
+_need_cache: Dict[tuple, int] = {}
+
 
 class _Workspace:
-    __slots__ = ("buf", "launches")
+    """The chaining words of one (device, stream) plus a pinned host word the kernels set when a
+    chunk gives up waiting for its predecessor: read on the host, at the next call, with a plain
+    memory read - no device call, no synchronisation."""
 
-    def __init__(self, buf: torch.Tensor):
+    __slots__ = ("buf", "ptr", "size", "launches", "flag", "flag_word")
+
+    def __init__(self, buf: torch.Tensor, stream_handle: int):
+        lib = _native.lib()
         self.buf = buf
+        self.ptr = buf.data_ptr()
+        self.size = buf.numel()
         self.launches = 0
+        self.flag = torch.zeros(1, dtype=torch.int32).pin_memory()
+        self.flag_word = ctypes.c_uint32.from_address(self.flag.data_ptr())
+        _native.check(lib.fss_workspace_init(self.ptr, self.size, stream_handle))
+        _native.check(lib.fss_workspace_attach_flag(self.ptr, self.flag.data_ptr(), stream_handle))
+
+    def reinit(self, stream_handle: int) -> None:
+        lib = _native.lib()
+        _native.check(lib.fss_workspace_init(self.ptr, self.size, stream_handle))
+        _native.check(lib.fss_workspace_attach_flag(self.ptr, self.flag.data_ptr(), stream_handle))
+        self.launches = 0
+
+    def raise_if_flagged(self) -> None:
+        if self.flag_word.value:
+            self.flag_word.value = 0
+            raise _native.FssError(
+                _native.FSS_ERR_CHAIN_TIMEOUT,
+                _native.strerror(_native.FSS_ERR_CHAIN_TIMEOUT)
+                + ": an earlier scan on this stream was starved of compute units (another process or a "
+                "concurrently replayed graph holding them); its outputs are NaN from the affected chunk on",
+            )
 
 
 def _validate(expected: torch.dtype, **tensors: torch.Tensor) -> Tuple[int, int, int]:
-    first_name, first = next(iter(tensors.items()))
+    first_name = first = None
     for name, t in tensors.items():
         if not isinstance(t, torch.Tensor):
             raise TypeError(f"{name} must be a torch.Tensor, got {type(t).__name__}")
@@ -59,6 +91,9 @@ def _validate(expected: torch.dtype, **tensors: torch.Tensor) -> Tuple[int, int,
             raise RuntimeError(f"expected scalar type {expected} for {name} but found {t.dtype}")
         if t.dim() != 3:
             raise RuntimeError(f"{name} must have shape (bs, seq, d_model), got {tuple(t.shape)}")
+        if first is None:
+            first_name, first = name, t
+            continue
         if t.device != first.device:
             raise RuntimeError(f"{name} is on {t.device} but {first_name} is on {first.device}")
         if t.shape != first.shape:
@@ -66,7 +101,7 @@ def _validate(expected: torch.dtype, **tensors: torch.Tensor) -> Tuple[int, int,
                 f"{name} has shape {tuple(t.shape)} but {first_name} has shape {tuple(first.shape)}"
             )
     bs, seq, d = first.shape
-    return int(bs), int(seq), int(d)
+    return bs, seq, d
 
 
 class _RawStream:
@@ -96,18 +131,42 @@ def _on(device: torch.device):
     return torch.cuda.device(device)
 
 
-def _workspace(device: torch.device, stream: "_RawStream", need: int) -> torch.Tensor:
+def _need(family: str, code: int, direction: int, bs: int, seq: int, d: int, config) -> int:
+    """Workspace bytes of one entry-point family ("rm": fss_workspace_bytes with (bs, seq, d);
+    "cm": fss_cm_workspace_bytes with (bs, d, seq)); asked of the library once per key."""
+    key = (family, code, direction, bs, seq, d, config if config is None else tuple(config))
+    need = _need_cache.get(key)
+    if need is None:
+        lib = _native.lib()
+        sizer = lib.fss_workspace_bytes if family == "rm" else lib.fss_cm_workspace_bytes
+        need = int(sizer(bs, seq, d, code, direction, _native.make_config(config)))
+        if len(_need_cache) > 4096:
+            _need_cache.clear()
+        _need_cache[key] = need
+    return need
+
+
+def _workspace(device: torch.device, stream: "_RawStream", need: int) -> "_Workspace":
+    """The workspace of (device, stream), grown to `need` bytes; raises if a scan launched through
+    it earlier reported a chain time-out."""
     key = (device.index if device.index is not None else torch.cuda.current_device(), stream.cuda_stream)
     ws = _workspaces.get(key)
-    if ws is None or ws.buf.numel() < need:
-        ws = _Workspace(torch.empty(max(need, 1 << 20), dtype=torch.uint8, device=device))
-        _native.check(_native.lib().fss_workspace_init(ws.buf.data_ptr(), ws.buf.numel(), stream.cuda_stream))
+    if ws is None or ws.size < need:
+        if ws is not None:
+            ws.raise_if_flagged()
+        ws = _Workspace(torch.empty(max(need, 1 << 20), dtype=torch.uint8, device=device), stream.cuda_stream)
         _workspaces[key] = ws
-    elif ws.launches >= _REINIT_AFTER_LAUNCHES:
-        _native.check(_native.lib().fss_workspace_init(ws.buf.data_ptr(), ws.buf.numel(), stream.cuda_stream))
-        ws.launches = 0
+    else:
+        if ws.flag_word.value:
+            ws.raise_if_flagged()
+        if ws.launches >= _REINIT_AFTER_LAUNCHES:
+            ws.reinit(stream.cuda_stream)
     ws.launches += 1
-    return ws.buf
+    return ws
+
+
+def _contiguous(t: torch.Tensor) -> torch.Tensor:
+    return t if t.is_contiguous() else t.contiguous()
 
 
 _CACHE_POLICIES = {"auto": _native.FSS_CACHE_AUTO, "streaming": _native.FSS_CACHE_STREAMING}
@@ -126,33 +185,34 @@ def set_cache_policy(policy: str) -> str:
 
 
 def workspace_status(device: Optional[torch.device] = None) -> None:
-    """Synchronises the current stream and raises if a chained scan timed out (debug aid)."""
+    """Synchronises the current stream and raises if a chained scan launched on it timed out."""
     device = torch.device("cuda", torch.cuda.current_device()) if device is None else device
     with torch.cuda.device(device):
         stream = _current_stream()
         ws = _workspaces.get((device.index, stream.cuda_stream))
         if ws is not None:
-            _native.check(_native.lib().fss_workspace_status(ws.buf.data_ptr(), stream.cuda_stream))
+            try:
+                _native.check(_native.lib().fss_workspace_status(ws.ptr, stream.cuda_stream))
+            finally:
+                ws.flag_word.value = 0
 
 
 def _forward(dtype: torch.dtype, alpha: torch.Tensor, beta: torch.Tensor, config=None) -> torch.Tensor:
     bs, seq, d = _validate(dtype, alpha=alpha, beta=beta)
-    alpha, beta = alpha.contiguous(), beta.contiguous()
-    out = torch.empty_like(alpha, memory_format=torch.contiguous_format)
+    alpha, beta = _contiguous(alpha), _contiguous(beta)
+    out = torch.empty_like(alpha)
     if out.numel() == 0:
         return out
-    lib = _native.lib()
     code = _DTYPE_CODE[dtype]
     with _on(alpha.device):
         stream = _current_stream()
-        need = lib.fss_workspace_bytes(bs, seq, d, code, _native.FSS_FWD, _native.make_config(config))
-        ws = _workspace(alpha.device, stream, need)
-        _native.check(
-            lib.fss_scan_fwd_ex(
-                code, alpha.data_ptr(), beta.data_ptr(), out.data_ptr(), bs, seq, d,
-                ws.data_ptr(), ws.numel(), stream.cuda_stream, _native.make_config(config),
-            )
+        ws = _workspace(alpha.device, stream, _need("rm", code, _native.FSS_FWD, bs, seq, d, config))
+        rc = _native.lib().fss_scan_fwd_ex(
+            code, alpha.data_ptr(), beta.data_ptr(), out.data_ptr(), bs, seq, d,
+            ws.ptr, ws.size, stream.cuda_stream, _native.make_config(config),
         )
+        if rc:
+            _native.check(rc)
     return out
 
 
@@ -160,24 +220,22 @@ def _backward(
     dtype: torch.dtype, alpha_saved: torch.Tensor, h_saved: torch.Tensor, grad_out: torch.Tensor, config=None
 ) -> List[torch.Tensor]:
     bs, seq, d = _validate(dtype, alpha_saved=alpha_saved, h_saved=h_saved, grad_out=grad_out)
-    alpha_saved, h_saved, grad_out = alpha_saved.contiguous(), h_saved.contiguous(), grad_out.contiguous()
-    grad_alpha = torch.empty_like(alpha_saved, memory_format=torch.contiguous_format)
-    grad_beta = torch.empty_like(alpha_saved, memory_format=torch.contiguous_format)
+    alpha_saved, h_saved, grad_out = _contiguous(alpha_saved), _contiguous(h_saved), _contiguous(grad_out)
+    grad_alpha = torch.empty_like(alpha_saved)
+    grad_beta = torch.empty_like(alpha_saved)
     if grad_alpha.numel() == 0:
         return [grad_alpha, grad_beta]
-    lib = _native.lib()
     code = _DTYPE_CODE[dtype]
     with _on(alpha_saved.device):
         stream = _current_stream()
-        need = lib.fss_workspace_bytes(bs, seq, d, code, _native.FSS_BWD, _native.make_config(config))
-        ws = _workspace(alpha_saved.device, stream, need)
-        _native.check(
-            lib.fss_scan_bwd_ex(
-                code, alpha_saved.data_ptr(), h_saved.data_ptr(), grad_out.data_ptr(),
-                grad_alpha.data_ptr(), grad_beta.data_ptr(), bs, seq, d,
-                ws.data_ptr(), ws.numel(), stream.cuda_stream, _native.make_config(config),
-            )
+        ws = _workspace(alpha_saved.device, stream, _need("rm", code, _native.FSS_BWD, bs, seq, d, config))
+        rc = _native.lib().fss_scan_bwd_ex(
+            code, alpha_saved.data_ptr(), h_saved.data_ptr(), grad_out.data_ptr(),
+            grad_alpha.data_ptr(), grad_beta.data_ptr(), bs, seq, d,
+            ws.ptr, ws.size, stream.cuda_stream, _native.make_config(config),
         )
+        if rc:
+            _native.check(rc)
     return [grad_alpha, grad_beta]
 
 
@@ -248,13 +306,12 @@ def scan_forward_state(
     code = _DTYPE_CODE[dtype]
     with _on(alpha.device):
         stream = _current_stream()
-        need = lib.fss_workspace_bytes(bs, seq, d, code, _native.FSS_FWD, _native.make_config(config))
-        ws = _workspace(alpha.device, stream, need)
+        ws = _workspace(alpha.device, stream, _need("rm", code, _native.FSS_FWD, bs, seq, d, config))
         _native.check(
             lib.fss_scan_fwd_state(
                 code, alpha.data_ptr(), beta.data_ptr(), out.data_ptr(),
                 h_before.data_ptr() if h_before is not None else None, h_last.data_ptr(),
-                bs, seq, d, ws.data_ptr(), ws.numel(), stream.cuda_stream, _native.make_config(config),
+                bs, seq, d, ws.ptr, ws.size, stream.cuda_stream, _native.make_config(config),
             )
         )
     return out, h_last
@@ -287,8 +344,7 @@ def scan_backward_state(
     code = _DTYPE_CODE[dtype]
     with _on(alpha_saved.device):
         stream = _current_stream()
-        need = lib.fss_workspace_bytes(bs, seq, d, code, _native.FSS_BWD, _native.make_config(config))
-        ws = _workspace(alpha_saved.device, stream, need)
+        ws = _workspace(alpha_saved.device, stream, _need("rm", code, _native.FSS_BWD, bs, seq, d, config))
         _native.check(
             lib.fss_scan_bwd_state(
                 code, alpha_saved.data_ptr(), h_saved.data_ptr(), grad_out.data_ptr(),
@@ -296,7 +352,7 @@ def scan_backward_state(
                 grad_h_last.data_ptr() if grad_h_last is not None else None,
                 grad_alpha.data_ptr(), grad_beta.data_ptr(),
                 grad_h_before.data_ptr() if grad_h_before is not None else None,
-                bs, seq, d, ws.data_ptr(), ws.numel(), stream.cuda_stream, _native.make_config(config),
+                bs, seq, d, ws.ptr, ws.size, stream.cuda_stream, _native.make_config(config),
             )
         )
     return grad_alpha, grad_beta, grad_h_before
@@ -325,11 +381,11 @@ def gated_scan_forward(gate: torch.Tensor, x: torch.Tensor, config=None) -> torc
     cfg = _native.make_config(config)
     with _on(gate.device):
         stream = _current_stream()
-        ws = _workspace(gate.device, stream, lib.fss_workspace_bytes(bs, seq, d, code, _native.FSS_GATED_FWD, cfg))
+        ws = _workspace(gate.device, stream, _need("rm", code, _native.FSS_GATED_FWD, bs, seq, d, config))
         _native.check(
             lib.fss_gated_scan_fwd(
                 code, gate.data_ptr(), x.data_ptr(), out.data_ptr(), bs, seq, d,
-                ws.data_ptr(), ws.numel(), stream.cuda_stream, cfg,
+                ws.ptr, ws.size, stream.cuda_stream, cfg,
             )
         )
     return out
@@ -351,12 +407,12 @@ def gated_scan_backward(
     cfg = _native.make_config(config)
     with _on(gate.device):
         stream = _current_stream()
-        ws = _workspace(gate.device, stream, lib.fss_workspace_bytes(bs, seq, d, code, _native.FSS_GATED_BWD, cfg))
+        ws = _workspace(gate.device, stream, _need("rm", code, _native.FSS_GATED_BWD, bs, seq, d, config))
         _native.check(
             lib.fss_gated_scan_bwd(
                 code, gate.data_ptr(), x.data_ptr(), h_saved.data_ptr(), grad_out.data_ptr(),
                 grad_gate.data_ptr(), grad_x.data_ptr(), bs, seq, d,
-                ws.data_ptr(), ws.numel(), stream.cuda_stream, cfg,
+                ws.ptr, ws.size, stream.cuda_stream, cfg,
             )
         )
     return [grad_gate, grad_x]
@@ -382,12 +438,12 @@ def gated_scan_forward_state(
     cfg = _native.make_config(config)
     with _on(gate.device):
         stream = _current_stream()
-        ws = _workspace(gate.device, stream, lib.fss_workspace_bytes(bs, seq, d, code, _native.FSS_GATED_FWD, cfg))
+        ws = _workspace(gate.device, stream, _need("rm", code, _native.FSS_GATED_FWD, bs, seq, d, config))
         _native.check(
             lib.fss_gated_scan_fwd_state(
                 code, gate.data_ptr(), x.data_ptr(), out.data_ptr(),
                 h_before.data_ptr() if h_before is not None else None, h_last.data_ptr(),
-                bs, seq, d, ws.data_ptr(), ws.numel(), stream.cuda_stream, cfg,
+                bs, seq, d, ws.ptr, ws.size, stream.cuda_stream, cfg,
             )
         )
     return out, h_last
@@ -420,7 +476,7 @@ def gated_scan_backward_state(
     cfg = _native.make_config(config)
     with _on(gate.device):
         stream = _current_stream()
-        ws = _workspace(gate.device, stream, lib.fss_workspace_bytes(bs, seq, d, code, _native.FSS_GATED_BWD, cfg))
+        ws = _workspace(gate.device, stream, _need("rm", code, _native.FSS_GATED_BWD, bs, seq, d, config))
         _native.check(
             lib.fss_gated_scan_bwd_state(
                 code, gate.data_ptr(), x.data_ptr(), h_saved.data_ptr(), grad_out.data_ptr(),
@@ -428,7 +484,7 @@ def gated_scan_backward_state(
                 grad_h_last.data_ptr() if grad_h_last is not None else None,
                 grad_gate.data_ptr(), grad_x.data_ptr(),
                 grad_h_before.data_ptr() if grad_h_before is not None else None,
-                bs, seq, d, ws.data_ptr(), ws.numel(), stream.cuda_stream, cfg,
+                bs, seq, d, ws.ptr, ws.size, stream.cuda_stream, cfg,
             )
         )
     return grad_gate, grad_x, grad_h_before
@@ -451,11 +507,11 @@ def scan_forward_cm(alpha: torch.Tensor, beta: torch.Tensor, config=None) -> tor
     cfg = _native.make_config(config)
     with _on(alpha.device):
         stream = _current_stream()
-        ws = _workspace(alpha.device, stream, lib.fss_cm_workspace_bytes(bs, d, seq, code, _native.FSS_FWD, cfg))
+        ws = _workspace(alpha.device, stream, _need("cm", code, _native.FSS_FWD, bs, d, seq, config))
         _native.check(
             lib.fss_scan_fwd_cm(
                 code, alpha.data_ptr(), beta.data_ptr(), out.data_ptr(), bs, d, seq,
-                ws.data_ptr(), ws.numel(), stream.cuda_stream, cfg,
+                ws.ptr, ws.size, stream.cuda_stream, cfg,
             )
         )
     return out
@@ -477,12 +533,12 @@ def scan_backward_cm(
     cfg = _native.make_config(config)
     with _on(alpha_saved.device):
         stream = _current_stream()
-        ws = _workspace(alpha_saved.device, stream, lib.fss_cm_workspace_bytes(bs, d, seq, code, _native.FSS_BWD, cfg))
+        ws = _workspace(alpha_saved.device, stream, _need("cm", code, _native.FSS_BWD, bs, d, seq, config))
         _native.check(
             lib.fss_scan_bwd_cm(
                 code, alpha_saved.data_ptr(), h_saved.data_ptr(), grad_out.data_ptr(),
                 grad_alpha.data_ptr(), grad_beta.data_ptr(), bs, d, seq,
-                ws.data_ptr(), ws.numel(), stream.cuda_stream, cfg,
+                ws.ptr, ws.size, stream.cuda_stream, cfg,
             )
         )
     return [grad_alpha, grad_beta]

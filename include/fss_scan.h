@@ -9,7 +9,12 @@
  *              grad_beta[t] = g[t];  grad_alpha[t] = g[t]*h[t-1] (t >= 1);  grad_alpha[0] = 0
  *
  * with fp32 carries in both directions.  The values in alpha[:,0,:] are never used
- * (they may be NaN).
+ * (they may be NaN).  Long sequences are scanned in chunks whose effect on the state is
+ * handed on as x -> A*x + B with A the product of the chunk's alphas (up to 512 of them):
+ * with |alpha| <= 1, the recurrence's regime, this matches the sequential order to fp32
+ * rounding.  With |alpha| > 1 over long stretches A can overflow to inf; a state of exactly
+ * 0 still stays 0 (as sequentially), but a tiny non-zero state times such an A is inf where
+ * the sequential order might have stayed finite.
  *
  * This header replaces, for a host written in any language, the pybind11 module
  * `sequential_scan_cuda` of the reference (csrc/sequential_scan.cpp:13-22) and
@@ -59,7 +64,7 @@
 extern "C" {
 #endif
 
-#define FSS_ABI_VERSION 1
+#define FSS_ABI_VERSION 2
 
 typedef enum fss_status {
   FSS_OK = 0,
@@ -104,7 +109,8 @@ const char *fss_strerror(int status);
 /* hipError_t of the most recent failed HIP call made by this thread, 0 if none */
 int fss_last_hip_error(void);
 
-/* Bytes of workspace a scan of this shape needs (a multiple of 256, never 0).
+/* Bytes of workspace a scan of this shape needs (a multiple of 256, never 0), whatever
+ * the alignment of its tensors (which changes how the library tiles the scan).
  * cfg may be NULL. */
 size_t fss_workspace_bytes(int64_t bs, int64_t seq, int64_t d, int dtype, int dir,
                            const fss_config *cfg);
@@ -116,6 +122,24 @@ int fss_workspace_init(void *workspace, size_t bytes, void *stream);
 /* Synchronises `stream`, then reports FSS_OK or FSS_ERR_CHAIN_TIMEOUT and clears
  * the sticky error word.  For tests and debugging. */
 int fss_workspace_status(void *workspace, void *stream);
+/*
+ * A chunk that gives up waiting (see FSS_ERR_CHAIN_TIMEOUT above) hands on a NaN state, so
+ * every output from there to the end of its sequence is NaN, and sets the workspace's
+ * sticky error word.  To learn of it without a device call or a synchronisation, attach a
+ * 32-bit word that the device can write and the host can read (hipHostMalloc memory): a
+ * kernel that gives up stores 1 there as well.  The host polls the word whenever it likes
+ * (it is set by the time the kernel has finished) and clears it itself.  Asynchronous on
+ * `stream` (a small kernel, graph-capturable); fss_workspace_init detaches the word; NULL
+ * detaches it too.  No counterpart in the reference, whose kernels never wait.
+ */
+int fss_workspace_attach_flag(void *workspace, uint32_t *flag, void *stream);
+/*
+ * Test hook: the number of polls after which a look-back gives up (default 2^20, seconds of
+ * waiting).  0 makes every look-back give up before its first poll, which exercises the
+ * time-out path on a healthy device with every kernel still running to completion.
+ * Process-wide; returns the previous value.
+ */
+uint32_t fss_debug_set_spin_limit(uint32_t polls);
 
 /* The configuration the library would choose for this shape (for reporting). */
 int fss_choose_config(int64_t bs, int64_t seq, int64_t d, int dtype, int dir,

@@ -165,3 +165,23 @@ def test_cm_c_abi_rejects_bad_arguments():
     assert lib.fss_scan_fwd_cm(_native.FSS_BF16, p, p, p, 2, 0, 512, *tail, None) == 0
     # chained sequence without a workspace
     assert lib.fss_scan_fwd_cm(_native.FSS_BF16, p, p, p, 1, 1, 8192, None, 0, sp, None) == 4
+
+
+def test_cm_growing_recurrence_with_zero_state_stays_zero():
+    """alpha == 2 along 9000 contiguous steps: the products the lanes exchange overflow fp32; a
+    state of exactly 0 must stay 0, as in the sequential order, and one impulse grows in exact
+    powers of two until it overflows to inf - never NaN."""
+    for dtype in (torch.bfloat16, torch.float32):
+        alpha = torch.full((2, 6, 9000), 2.0, dtype=dtype, device=DEV)
+        zeros = torch.zeros_like(alpha)
+        h = ext.scan_forward_cm(alpha, zeros)
+        ga, gb = ext.scan_backward_cm(alpha, zeros, zeros)
+        ext.workspace_status()
+        assert not h.any() and not ga.any() and not gb.any()
+        e0 = zeros.clone()
+        e0[..., 0] = 1.0
+        h = ext.scan_forward_cm(alpha, e0).float()
+        ext.workspace_status()
+        assert not torch.isnan(h).any()
+        want = torch.pow(2.0, torch.arange(9000, device=DEV, dtype=torch.float64)).to(torch.float32).to(dtype).float()
+        assert torch.equal(h, want.expand_as(h))

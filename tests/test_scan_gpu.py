@@ -493,3 +493,226 @@ def test_scans_on_two_streams_do_not_overlap(oracle):
     for i in range(2):
         for g, w in zip(got[i], want[i]):
             assert torch.equal(g, w)
+
+
+# ------------------------------------------- tensors with only their element alignment
+
+
+def _offset_view(t: torch.Tensor, offset_bytes: int) -> torch.Tensor:
+    """A contiguous copy of `t` on the device that starts `offset_bytes` into a 256-byte aligned
+    allocation."""
+    n_off = offset_bytes // t.element_size()
+    flat = torch.empty(t.numel() + n_off, dtype=t.dtype, device=DEV)
+    view = flat[n_off:].view(t.shape)
+    view.copy_(t)
+    assert view.data_ptr() % 256 == offset_bytes and view.is_contiguous()
+    return view
+
+
+@pytest.mark.parametrize("offset", [2, 4])
+@pytest.mark.parametrize("shape", [(1, 4096, 2048), (8, 3000, 1024), (1, 20000, 512)], ids=str)
+def test_offset_views_at_sizes_that_chain_many_chunks(oracle, shape, offset):
+    """Contiguous tensors that start 2 or 4 bytes into their storage take fewer channels per lane
+    and smaller tiles than aligned ones, so they chain more chunks and need a larger workspace
+    than the 16-byte aligned plan of the same shape: the public wrappers must size for that.
+    Forward and backward against the oracle; the reference takes any contiguous tensor
+    (csrc/sequential_scan_kernel.cu:126-187)."""
+    alpha, beta, dout = make_inputs("sigmoid", *shape, seed=91 + offset)
+    a, b, do = (_offset_view(t, offset) for t in (alpha, beta, dout))
+    h = ext.scan_forward_half(a, b)
+    ga, gb = ext.scan_backward_half(a, _offset_view(h, offset), do)
+    ext.workspace_status()
+    a_bits, b_bits, d_bits = bits(alpha), bits(beta), bits(dout)
+    h32 = oracle.scan_fwd_bf16_f32out(a_bits, b_bits)
+    ga32, gb32 = oracle.scan_bwd_bf16_f32out(a_bits, h32, d_bits)
+    assert_close_f32(h, h32, "h")
+    assert_close_f32(gb, gb32, "grad_beta")
+    assert_close_f32(ga, ga32, "grad_alpha")
+    # and through autograd, as a user would
+    a_req, b_req = a.detach().requires_grad_(True), b.detach().requires_grad_(True)
+    scan_cu(a_req, b_req).backward(do)
+    assert torch.equal(a_req.grad, ga) and torch.equal(b_req.grad, gb)
+
+
+# ------------------------------------------------------- |alpha| > 1 over long stretches
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32], ids=["bf16", "f32"])
+def test_growing_recurrence_with_zero_state_stays_zero(oracle, dtype):
+    """alpha == 2 over 300 steps: the product of a chunk's alphas overflows fp32 (2^128) long
+    before the sequence ends.  Where the state is exactly 0 the sequential recurrence keeps it 0
+    (sequential_scan/common.py:55) and so must the chunked one (inf * 0 would be NaN); where it
+    is not, both overflow to inf at the same step.  Every tiling, forward and backward."""
+    bs, seq, d = 2, 300, 128
+    alpha = torch.full((bs, seq, d), 2.0, dtype=dtype)
+    zeros = torch.zeros_like(alpha)
+    e0 = zeros.clone()
+    e0[:, 0] = 1.0
+    e_last = zeros.clone()
+    e_last[:, -1] = 1.0
+    small = torch.full_like(alpha, 2.0 ** -20)
+
+    def run(beta, dout, h_for_bwd, config):
+        h = ext._forward(dtype, alpha.to(DEV), beta.to(DEV), config)
+        ga, gb = ext._backward(dtype, alpha.to(DEV), h_for_bwd.to(DEV), dout.to(DEV), config)
+        ext.workspace_status()
+        return h.float().cpu().numpy(), ga.float().cpu().numpy(), gb.float().cpu().numpy()
+
+    def want(beta, dout, h_for_bwd):
+        if dtype == torch.float32:
+            h = oracle.scan_fwd_f32(alpha.numpy(), beta.numpy(), fused=True)
+            ga, gb = oracle.scan_bwd_f32(alpha.numpy(), h_for_bwd.numpy(), dout.numpy(), fused=True)
+            return h, ga, gb
+        h = oracle.scan_fwd_bf16(bits(alpha), bits(beta), fused=True)
+        ga, gb = oracle.scan_bwd_bf16(bits(alpha), bits(h_for_bwd), bits(dout), fused=True)
+        return tuple(oracle.bf16_bits_to_f32(x) for x in (h, ga, gb))
+
+    with np.errstate(over="ignore", invalid="ignore"):
+        for config in [None, (1, 8, 4), (2, 16, 8), (2, 8, 16), (1, 32, 2)]:
+            # zero everywhere: stays zero, no NaN from inf * 0
+            h, ga, gb = run(zeros, zeros, small, config)
+            assert not h.any() and not ga.any() and not gb.any(), config
+            # one impulse: exact powers of two until fp32 (or bf16) overflows, then inf - never NaN
+            h, ga, gb = run(e0, e_last, small, config)
+            h_w, ga_w, gb_w = want(e0, e_last, small)
+            assert not np.isnan(h).any() and not np.isnan(gb).any() and not np.isnan(ga).any(), config
+            np.testing.assert_array_equal(h, h_w, err_msg=str(config))
+            np.testing.assert_array_equal(gb, gb_w, err_msg=str(config))
+            np.testing.assert_array_equal(ga, ga_w, err_msg=str(config))
+
+
+# ------------------------------------------------------------------ chain time-outs
+
+
+def test_chain_timeout_poisons_the_output_and_is_reported(oracle):
+    """A look-back that gives up must be impossible to miss: NaN from the affected chunk on, the
+    workspace's sticky word, and the host-visible word that makes the NEXT call on that stream
+    raise without any synchronisation.  Forced from the host (a poll budget of zero makes every
+    look-back give up at once), so every kernel runs to completion."""
+    lib = _native.lib()
+    alpha, beta, dout = make_inputs("sigmoid", 2, 3000, 256, seed=95)
+    a, b, do = alpha.to(DEV), beta.to(DEV), dout.to(DEV)
+    good = ext.scan_forward_half(a, b)
+    ext.workspace_status()
+    first_chunk = 32 * 16  # rows of the largest tile any configuration covers in one chunk
+    previous = lib.fss_debug_set_spin_limit(0)
+    try:
+        assert previous == 1 << 20
+        h = ext.scan_forward_half(a, b)
+        torch.cuda.synchronize()
+        assert torch.isnan(h[:, first_chunk:].float()).all()      # everything behind the first chunk
+        assert torch.equal(h[:, :8], good[:, :8])                  # the first chunk needs no look-back
+        with pytest.raises(_native.FssError) as err:              # the next call reports it, before launching
+            ext.scan_forward_half(a, b)
+        assert err.value.status == _native.FSS_ERR_CHAIN_TIMEOUT
+        # the backward path and the debug query report it as well
+        ga, gb = ext.scan_backward_half(a, good, do)
+        torch.cuda.synchronize()
+        assert torch.isnan(gb[:, : 3000 - first_chunk].float()).all()
+        with pytest.raises(_native.FssError):
+            ext.workspace_status()
+    finally:
+        lib.fss_debug_set_spin_limit(previous)
+    # back to normal: same workspace, correct results, nothing pending
+    h = ext.scan_forward_half(a, b)
+    ext.workspace_status()
+    assert torch.equal(h, good)
+    # through the C ABI without the Python layer: sticky word and attached flag
+    ws = torch.zeros(lib.fss_workspace_bytes_max(*a.shape), dtype=torch.uint8, device=DEV)
+    flag = torch.zeros(1, dtype=torch.int32).pin_memory()
+    sp = torch.cuda.current_stream().cuda_stream
+    _native.check(lib.fss_workspace_init(ws.data_ptr(), ws.numel(), sp))
+    _native.check(lib.fss_workspace_attach_flag(ws.data_ptr(), flag.data_ptr(), sp))
+    out = torch.empty_like(a)
+    lib.fss_debug_set_spin_limit(0)
+    try:
+        _native.check(lib.fss_scan_fwd_bf16(a.data_ptr(), b.data_ptr(), out.data_ptr(), *a.shape, ws.data_ptr(), ws.numel(), sp))
+        torch.cuda.synchronize()
+    finally:
+        lib.fss_debug_set_spin_limit(1 << 20)
+    assert int(flag[0]) == 1
+    assert lib.fss_workspace_status(ws.data_ptr(), sp) == _native.FSS_ERR_CHAIN_TIMEOUT
+    assert lib.fss_workspace_status(ws.data_ptr(), sp) == 0  # cleared by the query
+    _native.check(lib.fss_scan_fwd_bf16(a.data_ptr(), b.data_ptr(), out.data_ptr(), *a.shape, ws.data_ptr(), ws.numel(), sp))
+    torch.cuda.synchronize()
+    assert torch.equal(out, good)
+
+
+# --------------------------------- residency of every kernel family (no wait is left unserved)
+
+
+def _big(dtype, shape=(8, 4096, 1024), seed=97):
+    return tuple(t.to(DEV) for t in make_inputs("sigmoid", *shape, dtype=dtype, seed=seed))
+
+
+def test_full_grids_of_small_workgroups_are_resident_in_every_kernel_family(oracle):
+    """The grid of a chained scan is sized from a hand-derived bound on how many workgroups are
+    resident at once; were it too high for some instantiation, workgroups that are not running
+    would be waited for and the scan would time out.  One case per kernel family with the
+    smallest workgroups and far more tiles than the device holds, each checked for a time-out
+    and against the same kernel run with large workgroups."""
+    from fast_sequential_scan_amd.sequential_scan_cuda import (
+        gated_scan_backward, gated_scan_forward, scan_backward_cm, scan_backward_state, scan_forward_cm,
+        scan_forward_state)
+
+    def same(x, y, tol):
+        assert torch.allclose(x.float(), y.float(), rtol=tol, atol=tol)
+
+    for dtype, small_cfgs, tol in ((torch.float32, [(1, 8, 1), (1, 8, 2), (2, 8, 1)], 1e-4),
+                                   (torch.float16, [(1, 8, 1), (2, 8, 2)], 2e-3)):
+        a, b, do = _big(dtype)
+        h_ref = ext._forward(dtype, a, b, (1, 16, 16))
+        ga_ref, gb_ref = ext._backward(dtype, a, h_ref, do, (1, 16, 16))
+        for cfg in small_cfgs:
+            h = ext._forward(dtype, a, b, cfg)
+            ga, gb = ext._backward(dtype, a, h_ref, do, cfg)
+            ext.workspace_status()
+            same(h, h_ref, tol), same(ga, ga_ref, tol), same(gb, gb_ref, tol)
+    # bf16: the state kernels, the gated kernels, and the other cache policies of the plain scan
+    a, b, do = _big(torch.bfloat16)
+    h0 = torch.randn(8, 1024, device=DEV)
+    h_ref, last_ref = scan_forward_state(a, b, h0, (2, 32, 16))
+    ref = scan_backward_state(a, h_ref, do, h0, None, (2, 16, 16))
+    for cfg in [(1, 8, 1), (2, 8, 2)]:
+        h, last = scan_forward_state(a, b, h0, cfg)
+        got = scan_backward_state(a, h_ref, do, h0, None, cfg)
+        ext.workspace_status()
+        same(h, h_ref, 2e-2), same(last, last_ref, 2e-2)
+        for x, y in zip(got, ref):
+            same(x, y, 2e-2)
+    gate = (a.float() * 4 - 2).to(torch.bfloat16)
+    g_ref = gated_scan_forward(gate, b, (2, 32, 16))
+    gb_ref = gated_scan_backward(gate, b, g_ref, do, (2, 16, 16))
+    for cfg in [(1, 8, 1), (2, 8, 2)]:
+        hg = gated_scan_forward(gate, b, cfg)
+        got = gated_scan_backward(gate, b, g_ref, do, cfg)
+        ext.workspace_status()
+        same(hg, g_ref, 2e-2)
+        for x, y in zip(got, gb_ref):
+            same(x, y, 2e-2)
+    # plain forward with a kept output (tensors up to 48 MiB) and plain backward that streams dout
+    # (tensors above 80 MiB): both are separate instantiations
+    a, b, do = _big(torch.bfloat16, (8, 2048, 1024))
+    h_ref = ext._forward(torch.bfloat16, a, b, (2, 32, 16))
+    for cfg in [(1, 8, 1), (2, 8, 2)]:
+        assert torch.equal(ext._forward(torch.bfloat16, a, b, cfg)[:, :8], h_ref[:, :8])
+        ext.workspace_status()
+    a, b, do = _big(torch.bfloat16, (8, 8192, 1024))
+    h_ref = ext._forward(torch.bfloat16, a, b, (2, 32, 16))
+    ga_ref, gb_ref = ext._backward(torch.bfloat16, a, h_ref, do, (2, 16, 16))
+    for cfg in [(1, 8, 1), (2, 8, 2)]:
+        ga, gb = ext._backward(torch.bfloat16, a, h_ref, do, cfg)
+        ext.workspace_status()
+        same(ga, ga_ref, 2e-2), same(gb, gb_ref, 2e-2)
+    del a, b, do, h_ref, ga_ref, gb_ref
+    # channel-major, chained (sequences beyond one workgroup's reach), one-wave workgroups
+    for dtype, vec in ((torch.bfloat16, 8), (torch.float32, 4)):
+        a, b, do = (t.transpose(1, 2).contiguous() for t in _big(dtype, (4, 8192, 1024)))
+        h_ref = scan_forward_cm(a, b)
+        ga_ref, gb_ref = scan_backward_cm(a, h_ref, do)
+        h = scan_forward_cm(a, b, (vec, 0, 1))
+        ga, gb = scan_backward_cm(a, h_ref, do, (vec, 0, 1))
+        ext.workspace_status()
+        tol = 2e-2 if dtype == torch.bfloat16 else 1e-4
+        same(h, h_ref, tol), same(ga, ga_ref, tol), same(gb, gb_ref, tol)
+    torch.cuda.empty_cache()
