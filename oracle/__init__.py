@@ -249,32 +249,70 @@ def _round_to(a: np.ndarray, rounding: str) -> np.ndarray:
         return a32
     if rounding == "bf16":
         return bf16_bits_to_f32(f32_to_bf16_bits(a32))
+    if rounding == "f16":
+        return a32.astype(np.float16).astype(np.float32)
     raise ValueError(rounding)
 
 
-def gate_transform(gate, x, rounding: str) -> Tuple[np.ndarray, np.ndarray]:
-    """(alpha, beta) as float32 arrays of storage-type values."""
+def _step_storage(v: np.ndarray, rounding: str, up: np.ndarray) -> np.ndarray:
+    """The storage-type value next to `v` (non-negative storage-type values held in float32):
+    one step up where `up`, else one step down (0 stays 0)."""
+    if rounding == "bf16":
+        bits = f32_to_bf16_bits(v).astype(np.int32)
+        bits = np.where(up, bits + 1, np.maximum(bits - 1, 0))
+        return bf16_bits_to_f32(bits.astype(np.uint16))
+    if rounding == "f16":
+        bits = v.astype(np.float16).view(np.uint16).astype(np.int32)
+        bits = np.where(up, bits + 1, np.maximum(bits - 1, 0))
+        return bits.astype(np.uint16).view(np.float16).astype(np.float32)
+    raise ValueError(rounding)
+
+
+def gate_alpha_variants(gate, rounding: str, fp32_ulps: float = 8.0):
+    """(alpha, alpha_other, ambiguous): alpha = sigmoid(gate) rounded to the storage type to
+    nearest; `ambiguous` marks the elements whose exact sigmoid lies within `fp32_ulps` fp32
+    units in the last place of the midpoint between two storage values, i.e. where an fp32
+    evaluation with a few ulps of error (a hardware exp2 and reciprocal) may legitimately round
+    to the other neighbour; `alpha_other` holds that neighbour there and alpha elsewhere.
+    fp32 storage has no such elements (its tests allow no deviation beyond their tolerance)."""
     g64 = np.asarray(gate, dtype=np.float64)
-    alpha = _round_to(1.0 / (1.0 + np.exp(-g64)), rounding)
+    exact = 1.0 / (1.0 + np.exp(-g64))
+    alpha = _round_to(exact, rounding)
+    if rounding == "f32":
+        return alpha, alpha, np.zeros(alpha.shape, dtype=bool)
+    up = exact > alpha.astype(np.float64)  # the exact value lies above the rounded one: the other neighbour is above
+    other = _step_storage(alpha, rounding, up)
+    mid = 0.5 * (alpha.astype(np.float64) + other.astype(np.float64))
+    eps = fp32_ulps * 2.0 ** -24 * np.maximum(exact, 2.0 ** -126)
+    ambiguous = np.abs(exact - mid) <= eps
+    return alpha, np.where(ambiguous, other, alpha).astype(np.float32), ambiguous
+
+
+def gate_transform(gate, x, rounding: str, other_rounding: bool = False) -> Tuple[np.ndarray, np.ndarray]:
+    """(alpha, beta) as float32 arrays of storage-type values.  `other_rounding`: alpha takes
+    the other neighbour wherever its rounding is ambiguous (see gate_alpha_variants)."""
+    alpha, alpha_other, _ = gate_alpha_variants(gate, rounding)
+    if other_rounding:
+        alpha = alpha_other
     a64 = alpha.astype(np.float64)
-    beta = _round_to(np.asarray(x, dtype=np.float64) * np.sqrt(1.0 - a64 * a64), rounding)
+    beta = _round_to(np.asarray(x, dtype=np.float64) * np.sqrt(np.maximum(1.0 - a64 * a64, 0.0)), rounding)
     return alpha, beta
 
 
-def gated_scan_fwd(gate, x, rounding: str) -> np.ndarray:
+def gated_scan_fwd(gate, x, rounding: str, other_rounding: bool = False) -> np.ndarray:
     """Un-rounded fp32 h of the scan over the rounded alpha and beta."""
-    alpha, beta = gate_transform(gate, x, rounding)
+    alpha, beta = gate_transform(gate, x, rounding, other_rounding)
     return scan_fwd_f32(alpha, beta)
 
 
-def gated_scan_bwd(gate, x, h, dout, rounding: str) -> Tuple[np.ndarray, np.ndarray]:
+def gated_scan_bwd(gate, x, h, dout, rounding: str, other_rounding: bool = False) -> Tuple[np.ndarray, np.ndarray]:
     """(grad_gate, grad_x) in float32, un-rounded: the plain backward, then the chain rule
     through beta = x*s, s = sqrt(1-alpha^2), alpha = sigmoid(gate).  Where alpha is exactly 1
     the x term of grad_gate is dropped."""
-    alpha, _ = gate_transform(gate, x, rounding)
+    alpha, _ = gate_transform(gate, x, rounding, other_rounding)
     grad_alpha, grad_beta = scan_bwd_f32(alpha, np.asarray(h, dtype=np.float32), np.asarray(dout, dtype=np.float32))
     a = alpha.astype(np.float64)
-    om = 1.0 - a * a
+    om = np.maximum(1.0 - a * a, 0.0)
     s = np.sqrt(om)
     with np.errstate(divide="ignore", invalid="ignore"):
         a_over_s = np.where(om > 0.0, a / s, 0.0)
@@ -282,3 +320,15 @@ def gated_scan_bwd(gate, x, h, dout, rounding: str) -> Tuple[np.ndarray, np.ndar
     grad_x = gb * s
     grad_gate = (grad_alpha.astype(np.float64) - gb * np.asarray(x, dtype=np.float64) * a_over_s) * a * (1.0 - a)
     return grad_gate.astype(np.float32), grad_x.astype(np.float32)
+
+
+def within_rounding_envelope(got, want, want_other, rtol: float, atol: float) -> np.ndarray:
+    """Elementwise: `got` lies within rtol/atol of the interval spanned by the two oracle
+    evaluations (alpha rounded to nearest / to the other neighbour where that is ambiguous).
+    Where no ambiguous element influences a result the two agree and this is the plain
+    tolerance check."""
+    got = np.asarray(got, dtype=np.float64)
+    lo = np.minimum(want, want_other).astype(np.float64)
+    hi = np.maximum(want, want_other).astype(np.float64)
+    tol = atol + rtol * np.maximum(np.abs(lo), np.abs(hi))
+    return (got >= lo - tol) & (got <= hi + tol)

@@ -132,3 +132,53 @@ def test_torch_gated_baseline_equals_numpy_oracle(oracle, rounding, dtype):
     want_gg, want_gx = oracle.gated_scan_bwd(g32, x32, h.numpy(), d32, rounding)
     np.testing.assert_allclose(gx.numpy(), want_gx, rtol=1e-5, atol=1e-5)
     np.testing.assert_allclose(gg.numpy(), want_gg, rtol=1e-4, atol=1e-5)
+
+
+@pytest.mark.parametrize("rounding", ["bf16", "f16"])
+def test_ambiguous_roundings_of_alpha(oracle, rounding):
+    """gate_alpha_variants: the elements it calls ambiguous are exactly those whose sigmoid sits on
+    a midpoint between two storage values (to a few fp32 ulps); the other rounding differs from
+    the nearest one there by one storage step and nowhere else.  Pinned on gates constructed from
+    the midpoints themselves (logit of the midpoint), without using the oracle's own formula."""
+    if rounding == "bf16":  # pairs of adjacent storage values in [0.25, 1)
+        bits = np.arange(0x3E80, 0x3F7F, dtype=np.uint16)
+        lo, hi = (oracle.bf16_bits_to_f32(b).astype(np.float64) for b in (bits, bits + 1))
+    else:
+        bits = np.arange(0x3400, 0x3BFF, 7, dtype=np.uint16)
+        lo, hi = (b.view(np.float16).astype(np.float64) for b in (bits, bits + 1))
+    mid = 0.5 * (lo + hi)
+    gate_at_mid = np.log(mid / (1.0 - mid))  # float64 gates: sigmoid lands on the midpoint to ~1e-16
+    alpha, other, ambiguous = oracle.gate_alpha_variants(gate_at_mid.reshape(1, -1, 1), rounding)
+    assert ambiguous.all()
+    a, o = alpha.ravel().astype(np.float64), other.ravel().astype(np.float64)
+    assert (np.minimum(a, o) == lo).all() and (np.maximum(a, o) == hi).all()
+    # a quarter of a storage step away from the midpoint nothing is ambiguous, and both variants agree
+    quarter = lo + 0.25 * (hi - lo)
+    alpha, other, ambiguous = oracle.gate_alpha_variants(np.log(quarter / (1.0 - quarter)).reshape(1, -1, 1), rounding)
+    assert not ambiguous.any()
+    np.testing.assert_array_equal(alpha, other)
+    np.testing.assert_array_equal(alpha.ravel(), lo.astype(np.float32))
+    # random gates: the ambiguous share is the window over the storage step (a few in 10^4)
+    rng = np.random.default_rng(21)
+    gate = (1.5 * rng.standard_normal((4, 500, 100))).astype(np.float32)
+    alpha, other, ambiguous = oracle.gate_alpha_variants(gate, rounding)
+    assert 0 < ambiguous.mean() < (2e-3 if rounding == "bf16" else 2e-2)
+    changed = alpha != other
+    np.testing.assert_array_equal(changed, ambiguous & changed)
+    # fp32 storage: never ambiguous
+    assert not oracle.gate_alpha_variants(gate, "f32")[2].any()
+
+
+def test_rounding_envelope_is_the_plain_tolerance_where_the_variants_agree(oracle):
+    want = np.array([1.0, -2.0, 0.0, 5.0], np.float32)
+    other = np.array([1.0, -2.0, 0.0, 6.0], np.float32)
+    got = np.array([1.02, -2.05, 0.011, 5.5], np.float32)
+    ok = oracle.within_rounding_envelope(got, want, other, 1e-2, 1e-2)
+    np.testing.assert_array_equal(ok, [True, False, False, True])
+    got = np.array([1.0, -2.0, 0.0, 6.2], np.float32)
+    np.testing.assert_array_equal(oracle.within_rounding_envelope(got, want, other, 1e-2, 1e-2), [True, True, True, False])
+    # the other-rounding evaluation equals the nearest one when no element is ambiguous
+    rng = np.random.default_rng(22)
+    gate, x = _rand(rng, (1, 30, 4)), _rand(rng, (1, 30, 4))
+    if not oracle.gate_alpha_variants(gate, "bf16")[2].any():
+        np.testing.assert_array_equal(oracle.gated_scan_fwd(gate, x, "bf16"), oracle.gated_scan_fwd(gate, x, "bf16", True))

@@ -2,11 +2,14 @@
 alpha = sigmoid(gate), beta = x*sqrt(1-alpha^2) computed inside the scan kernels.
 
 Tolerances: rtol = atol = 1e-2 in bf16 (the bar of the plain bf16 scan), 1e-4 / 1e-5 in
-fp32.  In bf16 the device's sigmoid (hardware exp2 and reciprocal, ~2 fp32 ulps) can land
-on the other side of a bf16 rounding boundary than the oracle's float64 one for a few
-elements in 10^5; alpha then differs by one bf16 ulp there, and near alpha -> 1 the
-backward amplifies that (alpha/s).  Those tests therefore allow a stated, tiny fraction of
-elements outside the tolerance; the fp32 tests allow none.
+fp32, for every element.  In bf16 the device's sigmoid (hardware exp2 and reciprocal, a few
+fp32 ulps) can land on the other side of a bf16 rounding boundary than the oracle's float64
+one for a few elements in 10^4; alpha then differs by one bf16 ulp there, and near
+alpha -> 1 the backward amplifies that (alpha/s).  The oracle therefore evaluates twice -
+alpha rounded to nearest, and to the other neighbour wherever the exact sigmoid lies within
+8 fp32 ulps of the rounding boundary - and every element must lie within the tolerance of
+the interval the two evaluations span.  Where no such element influences a result the two
+agree and the check is the plain tolerance: nothing is ever let through unexplained.
 """
 import ctypes
 
@@ -20,7 +23,6 @@ from fast_sequential_scan_amd import _native, scan_cu_single, scan_gated  # noqa
 from fast_sequential_scan_amd import sequential_scan_cuda as ext  # noqa: E402
 
 DEV = "cuda:0"
-BF16_OUTLIER_FRACTION = 2e-4
 
 
 def _inputs(shape, dtype, seed, gate_scale=1.5):
@@ -31,12 +33,25 @@ def _inputs(shape, dtype, seed, gate_scale=1.5):
     return gate, x, dout
 
 
-def _check(got, want, rtol, atol, what, outliers=0.0):
+def _check(oracle, got, want, want_other, rtol, atol, what):
     got = got.detach().float().cpu().numpy()
     assert np.isfinite(got).all(), what
-    bad = ~(np.abs(got - want) <= atol + rtol * np.abs(want))
-    assert bad.mean() <= outliers, (
-        f"{what}: {bad.sum()} of {bad.size} outside tolerance, worst {np.abs(got - want).max():.4g}")
+    ok = oracle.within_rounding_envelope(got, want, want_other, rtol, atol)
+    assert ok.all(), (
+        f"{what}: {(~ok).sum()} of {ok.size} outside tolerance of both roundings, first at {np.argwhere(~ok)[0]}, "
+        f"worst {np.abs(got - want)[~ok].max():.4g}")
+
+
+def _check_all(oracle, rounding, rtol, atol, gate, x, dout, h, grad_gate, grad_x):
+    g32, x32, d32 = gate.float().numpy(), x.float().numpy(), dout.float().numpy()
+    h_dev = h.float().cpu().numpy()
+    _check(oracle, h, oracle.gated_scan_fwd(g32, x32, rounding), oracle.gated_scan_fwd(g32, x32, rounding, True),
+           rtol, atol, "h")
+    # the backward is fed the stored (rounded) h, as the product path does
+    want_gate, want_x = oracle.gated_scan_bwd(g32, x32, h_dev, d32, rounding)
+    other_gate, other_x = oracle.gated_scan_bwd(g32, x32, h_dev, d32, rounding, True)
+    _check(oracle, grad_x, want_x, other_x, rtol, atol, "grad_x")
+    _check(oracle, grad_gate, want_gate, other_gate, rtol, atol, "grad_gate")
 
 
 CASES = [
@@ -56,18 +71,12 @@ def test_gated_scan_matches_oracle(oracle, dtype, shape, fwd_cfg, bwd_cfg):
         bwd_cfg = (1,) + tuple(bwd_cfg[1:]) if bwd_cfg else None
     rounding = "bf16" if bf16 else "f32"
     rtol, atol = (1e-2, 1e-2) if bf16 else (1e-4, 1e-5)
-    outliers = BF16_OUTLIER_FRACTION if bf16 else 0.0
     gate, x, dout = _inputs(shape, dtype, seed=sum(shape))
     gd, xd, dd = gate.to(DEV), x.to(DEV), dout.to(DEV)
     h = ext.gated_scan_forward(gd, xd, fwd_cfg)
     grad_gate, grad_x = ext.gated_scan_backward(gd, xd, h, dd, bwd_cfg)
     ext.workspace_status()
-    g32, x32, d32 = gate.float().numpy(), x.float().numpy(), dout.float().numpy()
-    _check(h, oracle.gated_scan_fwd(g32, x32, rounding), rtol, atol, "h", outliers)
-    # the backward is fed the stored (rounded) h, as the product path does
-    want_gate, want_x = oracle.gated_scan_bwd(g32, x32, h.float().cpu().numpy(), d32, rounding)
-    _check(grad_x, want_x, rtol, atol, "grad_x", outliers)
-    _check(grad_gate, want_gate, rtol, atol, "grad_gate", outliers)
+    _check_all(oracle, rounding, rtol, atol, gate, x, dout, h, grad_gate, grad_x)
 
 
 def test_every_chunking_gives_the_same_result():
@@ -140,11 +149,7 @@ def test_headline_size_against_oracle(oracle):
     h = ext.gated_scan_forward(gd, xd)
     grad_gate, grad_x = ext.gated_scan_backward(gd, xd, h, dd)
     ext.workspace_status()
-    g32, x32 = gate.float().numpy(), x.float().numpy()
-    _check(h, oracle.gated_scan_fwd(g32, x32, "bf16"), 1e-2, 1e-2, "h", BF16_OUTLIER_FRACTION)
-    want_gate, want_x = oracle.gated_scan_bwd(g32, x32, h.float().cpu().numpy(), dout.float().numpy(), "bf16")
-    _check(grad_x, want_x, 1e-2, 1e-2, "grad_x", BF16_OUTLIER_FRACTION)
-    _check(grad_gate, want_gate, 1e-2, 1e-2, "grad_gate", BF16_OUTLIER_FRACTION)
+    _check_all(oracle, "bf16", 1e-2, 1e-2, gate, x, dout, h, grad_gate, grad_x)
 
 
 def test_autograd_and_validation():
