@@ -79,7 +79,7 @@ def build(verbose: bool = False, extra_flags: Sequence[str] = (), output: str = 
         with ThreadPoolExecutor(max_workers=min(len(commands), os.cpu_count() or 1, 8)) as pool:
             list(pool.map(lambda c: _run(c, verbose), commands))
         linked = output + ".tmp"
-        _run([hipcc, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", linked, *objects], verbose)
+        _run([hipcc, "--offload-arch=gfx950", "-shared", "-fPIC", "-Wl,-soname,libfss_scan.so", "-o", linked, *objects], verbose)
         os.replace(linked, output)
     return output
 
