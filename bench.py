@@ -11,10 +11,14 @@ tensors already resident in HBM.  Prints ONE JSON line:
                    writes grad_alpha, grad_beta = 10 B) divided by the wall time per step
   roofline         the dominant kernel (the backward scan, 10 of the 16 B): its
                    algorithmic bytes per launch over its mean duration, measured with
-                   HIP events recorded around the launches of every 8th step of the
-                   timed region (less what an empty pair of events reads, calibrated
-                   in the same run); `traffic` is the counter-measured HBM bytes per
-                   launch from profiles/, when that summary covers the configuration
+                   HIP events recorded around the launches of sampled steps of the timed
+                   region and of a sampling loop that follows it (at least 32 samples
+                   whatever --steps is), less what a pair of events adds to a kernel
+                   between them (calibrated in the same run with the library's copy
+                   kernel: one launch between two events against four); `traffic` is
+                   the counter-measured HBM bytes per launch from profiles/, when that
+                   summary covers the configuration; `frac_no_reuse` is the same
+                   fraction with eight sets of tensors in rotation
   rotating_sets    the same step over eight sets of tensors in rotation, so that no step finds its
                    inputs in the memory-side cache (`value` reuses one set, as the reference's
                    benchmark does); `--rotate 8` makes that the timed region itself
@@ -313,16 +317,60 @@ def main() -> int:
     _native.check(lib.fss_workspace_status(pws, sp))
 
     ms_per_step = wall * 1e3 / K
-    # What a pair of events reads with nothing between them: the cost of the event
-    # packets themselves, taken off every kernel interval below.
-    pairs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(100)]
+
+    def launch_pair_samples(n):
+        """n more steps with events around both launches of each: [(fwd_ms, bwd_ms)] raw."""
+        evs = [[torch.cuda.Event(enable_timing=True) for _ in range(3)] for _ in range(n)]
+        for e in evs:
+            e[0].record(stream)
+            fwd()
+            e[1].record(stream)
+            bwd()
+            e[2].record(stream)
+            next_set()
+        torch.cuda.synchronize()
+        return [(e[0].elapsed_time(e[1]), e[1].elapsed_time(e[2])) for e in evs]
+
+    # What a pair of events adds to the kernel between them.  An empty pair overstates it (the
+    # second event's packet is processed while a kernel runs, not after), so it is calibrated with
+    # the library's copy kernel on a cache-resident buffer: events around one launch against
+    # events around four launches back to back; a launch costs (t4 - t1)/3, the rest of t1 is the
+    # events'.  What is left in the kernel times after subtracting it is the gap between two
+    # launches, so they err on the long side.
+    cal = torch.empty(4 << 20, dtype=torch.uint8, device=dev)
+    cal2 = torch.empty_like(cal)
+
+    def copy_between_events(n_launches):
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record(stream)
+        for _ in range(n_launches):
+            lib.fss_copy_bytes(cal.data_ptr(), cal2.data_ptr(), cal.numel(), sp)
+        e1.record(stream)
+        return e0, e1
+
+    for _ in range(10):
+        copy_between_events(4)
+    ones = [copy_between_events(1) for _ in range(60)]
+    fours = [copy_between_events(4) for _ in range(60)]
+    pairs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(60)]
     for e0, e1 in pairs:
         e0.record(stream)
         e1.record(stream)
     torch.cuda.synchronize()
-    event_overhead = statistics.median(e0.elapsed_time(e1) for e0, e1 in pairs)
+    t1 = statistics.median(e0.elapsed_time(e1) for e0, e1 in ones)
+    t4 = statistics.median(e0.elapsed_time(e1) for e0, e1 in fours)
+    empty_pair = statistics.median(e0.elapsed_time(e1) for e0, e1 in pairs)
+    event_overhead = min(max(t1 - (t4 - t1) / 3.0, 0.0), empty_pair)
+    del cal, cal2
+
     fwd_raw = [ev[k][0].elapsed_time(ev[k][1]) for k in sampled]
     bwd_raw = [ev[k][1].elapsed_time(ev[k][2]) for k in sampled]
+    in_region = len(sampled)
+    if in_region < 32:  # the same loop goes on, untimed, until there are enough samples
+        more = launch_pair_samples(32 - in_region)
+        first_set()
+        fwd_raw += [f for f, _ in more]
+        bwd_raw += [b for _, b in more]
     fwd_ms = [max(t - event_overhead, 1e-6) for t in fwd_raw]
     bwd_ms = [max(t - event_overhead, 1e-6) for t in bwd_raw]
     fwd_mean, bwd_mean = statistics.fmean(fwd_ms), statistics.fmean(bwd_ms)
@@ -351,11 +399,23 @@ def main() -> int:
             next_set()
         torch.cuda.synchronize()
         rot_ms = (time.perf_counter() - t0) * 1e3 / n_rot
+        rot = launch_pair_samples(32)
+        rot_fwd = statistics.fmean(max(f - event_overhead, 1e-6) for f, _ in rot)
+        rot_bwd = statistics.fmean(max(b - event_overhead, 1e-6) for _, b in rot)
         rotating = {"tensor_sets": len(pointer_sets), "steps": n_rot, "ms_per_step": round(rot_ms, 5),
-                    "GBps": round(step_bytes / (rot_ms * 1e-3) / 1e9, 1)}
+                    "GBps": round(step_bytes / (rot_ms * 1e-3) / 1e9, 1),
+                    "pct_of_hbm_peak": round(100.0 * step_bytes / (rot_ms * 1e-3) / 1e9 / HBM_PEAK_GBPS, 2),
+                    "fwd_ms": round(rot_fwd, 5), "bwd_ms": round(rot_bwd, 5),
+                    "fwd_frac": round(fwd_bytes_per_elem * n_elem / (rot_fwd * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4),
+                    "bwd_frac": round(bwd_bytes_per_elem * n_elem / (rot_bwd * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4)}
         del pointer_sets[1:]
         del extra
         first_set()
+    elif len(pointer_sets) > 1:
+        rotating = {"tensor_sets": len(pointer_sets), "steps": K, "ms_per_step": round(ms_per_step, 5),
+                    "GBps": round(value, 1), "pct_of_hbm_peak": round(100.0 * value / HBM_PEAK_GBPS, 2),
+                    "fwd_ms": round(fwd_mean, 5), "bwd_ms": round(bwd_mean, 5),
+                    "fwd_frac": round(fwd_gbps / HBM_PEAK_GBPS, 4), "bwd_frac": round(bwd_gbps / HBM_PEAK_GBPS, 4)}
 
     # ---- cold timings: reading a large buffer between launches evicts L2 and the memory-side
     # cache and leaves them clean (a large write would leave dirty lines whose write-back is then
@@ -433,18 +493,35 @@ def main() -> int:
             reps += 1
         cpu_step = statistics.median(f_times) + statistics.median(b_times)
 
-        # gated bf16: sigmoid lands on the other side of a bf16 rounding boundary for a few elements in
-        # 10^5 (device exp2/rcp against the CPU's), so a stated fraction may sit outside the tolerance
-        allowed = 2e-4 if (gated and is_16bit) else 0.0
+        # gated, 16-bit storage: where sigmoid(gate) sits on a rounding boundary of the storage type the
+        # device's exp2/rcp and the CPU's may round alpha to different neighbours; the NumPy oracle is
+        # therefore evaluated with both roundings and every element must lie within the tolerance of
+        # the interval they span (identical to the plain tolerance wherever no such element matters)
+        other = None
+        if gated and is_16bit:
+            import oracle
+
+            rounding = "bf16" if args.dtype == "bf16" else "f16"
+            g32, x32, d32 = alpha_c.float().numpy(), beta_c.float().numpy(), dout_c.float().numpy()
+            h_dev = h_gpu.numpy()
+            want = (oracle.gated_scan_fwd(g32, x32, rounding), *oracle.gated_scan_bwd(g32, x32, h_dev, d32, rounding))
+            alt = (oracle.gated_scan_fwd(g32, x32, rounding, True), *oracle.gated_scan_bwd(g32, x32, h_dev, d32, rounding, True))
+            other = {id(t): (w, a) for t, w, a in zip((h_ref, ga_ref, gb_ref), want, alt)}
 
         def ok(got, want):
-            return bool(((got - want).abs() > tol + tol * want.abs()).float().mean().item() <= allowed)
+            if other is not None:
+                import oracle
+
+                w, a = other[id(want)]
+                return bool(oracle.within_rounding_envelope(got.numpy(), w, a, tol, tol).all())
+            return bool(((got - want).abs() <= tol + tol * want.abs()).all().item())
 
         names = ("h", "grad_gate", "grad_x") if gated else ("h", "grad_alpha", "grad_beta")
         parity = {
             names[0]: ok(h_gpu, h_ref), names[1]: ok(ga_gpu, ga_ref), names[2]: ok(gb_gpu, gb_ref),
-            "rtol": tol, "atol": tol, "outlier_fraction_allowed": allowed,
-            "against": f"fp32 sequential loop on the CPU, same {args.dtype} inputs",
+            "rtol": tol, "atol": tol, "outlier_fraction_allowed": 0.0,
+            "against": (f"fp32 sequential loop on the CPU, same {args.dtype} inputs"
+                        + (", alpha rounded either way where its rounding is ambiguous" if other is not None else "")),
         }
         cpu = {
             "value": round(step_bytes / cpu_step / 1e9, 3),
@@ -501,6 +578,7 @@ def main() -> int:
             "launch_config_bwd_vec_steps_waves": chosen["bwd"],
         },
         "pct_of_hbm_peak": round(100.0 * value / HBM_PEAK_GBPS, 2),
+        "pct_of_hbm_peak_no_reuse": rotating.get("pct_of_hbm_peak"),
         "fwd_ms": round(fwd_mean, 5),
         "bwd_ms": round(bwd_mean, 5),
         "fwd_ms_median": round(statistics.median(fwd_ms), 5),
@@ -508,8 +586,10 @@ def main() -> int:
         "fwd_ms_p20_p80": quantile_pair(fwd_ms),
         "bwd_ms_p20_p80": quantile_pair(bwd_ms),
         "algorithmic_bytes_per_step": step_bytes,
-        "event_sampled_steps": len(sampled),
+        "event_samples": len(fwd_ms),
+        "event_samples_in_timed_region": in_region,
         "event_pair_overhead_ms": round(event_overhead, 5),
+        "event_pair_empty_ms": round(empty_pair, 5),
         "fwd_ms_event_raw": round(statistics.fmean(fwd_raw), 5),
         "bwd_ms_event_raw": round(statistics.fmean(bwd_raw), 5),
         "roofline": {
@@ -519,6 +599,7 @@ def main() -> int:
             "peak": HBM_PEAK_GBPS,
             "unit": "GB/s",
             "frac": round(bwd_gbps / HBM_PEAK_GBPS, 4),
+            "frac_no_reuse": rotating.get("bwd_frac"),
             "traffic": traffic["bwd"],
             "bytes_per_launch": bwd_bytes_per_elem * n_elem,
             "avg_launch_ms": round(bwd_mean, 5),
@@ -530,6 +611,7 @@ def main() -> int:
             "peak": HBM_PEAK_GBPS,
             "unit": "GB/s",
             "frac": round(fwd_gbps / HBM_PEAK_GBPS, 4),
+            "frac_no_reuse": rotating.get("fwd_frac"),
             "traffic": traffic["fwd"],
             "bytes_per_launch": fwd_bytes_per_elem * n_elem,
             "avg_launch_ms": round(fwd_mean, 5),
