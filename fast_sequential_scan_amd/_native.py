@@ -19,7 +19,9 @@ FSS_FWD, FSS_BWD, FSS_GATED_FWD, FSS_GATED_BWD = 0, 1, 2, 3
 FSS_OK = 0
 FSS_CACHE_AUTO, FSS_CACHE_STREAMING = 0, 1
 FSS_ERR_CHAIN_TIMEOUT = 7
+FSS_ERR_TOO_LARGE = 9
 FSS_ABI_VERSION = 2
+FSS_NOALLOC_SCRATCH_BYTES = 16 << 20
 
 EXPORTED_SYMBOLS = (
     "fss_abi_version",
@@ -31,6 +33,7 @@ EXPORTED_SYMBOLS = (
     "fss_workspace_status",
     "fss_workspace_attach_flag",
     "fss_debug_set_spin_limit",
+    "fss_scan_fwd_noalloc",
     "fss_choose_config",
     "fss_scan_fwd_bf16",
     "fss_scan_bwd_bf16",
@@ -97,6 +100,8 @@ def _declare(lib: ctypes.CDLL) -> None:
     lib.fss_workspace_attach_flag.argtypes = [_vp, _vp, _vp]
     lib.fss_debug_set_spin_limit.restype = ctypes.c_uint32
     lib.fss_debug_set_spin_limit.argtypes = [ctypes.c_uint32]
+    lib.fss_scan_fwd_noalloc.restype = _int
+    lib.fss_scan_fwd_noalloc.argtypes = [_int, _vp, _vp, _vp, _i64, _i64, _i64, _vp]
     lib.fss_choose_config.restype = _int
     lib.fss_choose_config.argtypes = [_i64, _i64, _i64, _int, _int, _sz, _cfgp]
     fwd = [_vp, _vp, _vp, _i64, _i64, _i64, _vp, _sz, _vp]

@@ -31,6 +31,53 @@ __global__ void copy_kernel(const u32x4 *__restrict__ src, u32x4 *__restrict__ d
 int g_cache_policy = FSS_CACHE_AUTO;  // fss_set_cache_policy
 uint32_t g_spin_limit = kSpinLimit;    // fss_debug_set_spin_limit
 
+// ---- the chaining scratch of the entry point that allocates nothing ----------------------
+//
+// One array per device (every GPU the library runs on holds its own copy, at its own
+// address, until the process ends).  Zero-initialised memory is a ready workspace, so it
+// needs no reset before its first use.  In host code the array's name is only a handle
+// for hipGetSymbolAddress: what the kernels get is the address looked up once per device.
+static __device__ __align__(256) unsigned char scratch[FSS_NOALLOC_SCRATCH_BYTES];
+
+struct ScratchSlot {
+  std::mutex lock;
+  void *ptr = nullptr;
+};
+static ScratchSlot g_scratch[64];
+
+// Address of the current device's copy of `scratch`; looked up at the first call on that
+// device.  The same set-up creates the event that orders scans across streams, so that no
+// later call through this entry point has anything left to create.
+static int scratch_of_current_device(void **out) {
+  int dev = 0;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) {
+    tls_hip_error = static_cast<int>(e);
+    return FSS_ERR_LAUNCH;
+  }
+  if (dev < 0 || dev >= 64) return FSS_ERR_UNSUPPORTED_DEVICE;
+  ScratchSlot &slot = g_scratch[dev];
+  std::lock_guard<std::mutex> guard(slot.lock);
+  if (!slot.ptr) {
+    void *ptr = nullptr;
+    e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+    if (e != hipSuccess || !ptr) {
+      tls_hip_error = static_cast<int>(e);
+      (void)hipGetLastError();
+      return FSS_ERR_LAUNCH;
+    }
+    ScanOrder &order = g_scan_order[dev];
+    std::lock_guard<std::mutex> order_guard(order.lock);
+    if (!order.event && hipEventCreateWithFlags(&order.event, hipEventDisableTiming) != hipSuccess) {
+      order.event = nullptr;
+      (void)hipGetLastError();
+    }
+    slot.ptr = ptr;
+  }
+  *out = slot.ptr;
+  return FSS_OK;
+}
+
 int run_scan(int dtype, int dir, const void *alpha, const void *in_b, const void *in_h, void *out0,
              void *out1, int64_t bs, int64_t seq, int64_t d, void *workspace, size_t workspace_bytes,
              void *stream, const fss_config *cfg, const float *state_in = nullptr,
@@ -126,6 +173,9 @@ const char *fss_strerror(int status) {
     case FSS_ERR_LAUNCH: return "HIP reported an error (see fss_last_hip_error)";
     case FSS_ERR_CHAIN_TIMEOUT: return "a chunk gave up waiting for the state of its predecessor";
     case FSS_ERR_UNSUPPORTED_DEVICE: return "the current device is not gfx950";
+    case FSS_ERR_TOO_LARGE:
+      return "the shape needs more chaining scratch than the entry point that allocates nothing holds "
+             "(FSS_NOALLOC_SCRATCH_BYTES): use fss_scan_fwd_ex with a workspace";
     default: return "unknown status";
   }
 }
@@ -224,6 +274,18 @@ int fss_scan_fwd_ex(int dtype, const void *alpha, const void *beta, void *h, int
                     const fss_config *cfg) {
   return fss::run_scan(dtype, FSS_FWD, alpha, beta, nullptr, h, nullptr, bs, seq, d, workspace,
                        workspace_bytes, stream, cfg);
+}
+
+int fss_scan_fwd_noalloc(int dtype, const void *alpha, const void *beta, void *h, int64_t bs, int64_t seq,
+                         int64_t d, void *stream) {
+  if (bs < 0 || seq < 0 || d < 0) return FSS_ERR_BAD_SHAPE;
+  if (bs == 0 || seq == 0 || d == 0) return FSS_OK;
+  if (fss_workspace_bytes(bs, seq, d, dtype, FSS_FWD, nullptr) > FSS_NOALLOC_SCRATCH_BYTES) return FSS_ERR_TOO_LARGE;
+  void *ptr = nullptr;
+  const int rc = fss::scratch_of_current_device(&ptr);
+  if (rc != FSS_OK) return rc;
+  return fss::run_scan(dtype, FSS_FWD, alpha, beta, nullptr, h, nullptr, bs, seq, d, ptr, FSS_NOALLOC_SCRATCH_BYTES,
+                       stream, nullptr);
 }
 
 int fss_scan_bwd_ex(int dtype, const void *alpha, const void *h, const void *dout, void *grad_alpha,

@@ -75,7 +75,8 @@ typedef enum fss_status {
   FSS_ERR_BAD_CONFIG = 5,      /* explicit launch configuration not supported     */
   FSS_ERR_LAUNCH = 6,          /* HIP reported an error at launch (see fss_last_hip_error) */
   FSS_ERR_CHAIN_TIMEOUT = 7,   /* reported by fss_workspace_status: a chunk gave up waiting */
-  FSS_ERR_UNSUPPORTED_DEVICE = 8 /* current device is not gfx950                  */
+  FSS_ERR_UNSUPPORTED_DEVICE = 8, /* current device is not gfx950                 */
+  FSS_ERR_TOO_LARGE = 9        /* fss_scan_fwd_noalloc: the shape needs more than FSS_NOALLOC_SCRATCH_BYTES */
 } fss_status;
 
 /* FSS_F16 (IEEE half) has no counterpart in the reference; same kernels, same fp32 carries */
@@ -196,6 +197,24 @@ int fss_scan_bwd_f32(const void *alpha, const void *h, const void *dout,
  */
 enum fss_cache_policy { FSS_CACHE_AUTO = 0, FSS_CACHE_STREAMING = 1 };
 int fss_set_cache_policy(int policy);
+
+/*
+ * fss_scan_fwd_ex with cfg = NULL for callers that cannot allocate device memory and have
+ * no workspace to bring (code under graph capture, tight serving loops, harnesses that
+ * forbid hipMalloc): the chaining words live in a static device array of
+ * FSS_NOALLOC_SCRATCH_BYTES inside the library, one copy per GPU, held until the process
+ * ends.  No counterpart in the reference.  The call allocates and frees nothing, in the
+ * library or in the HIP runtime (the first call on a device looks up the array's address
+ * and creates the event that orders scans across streams).  A shape whose
+ * fss_workspace_bytes(.., FSS_FWD, NULL) exceeds the array is refused with
+ * FSS_ERR_TOO_LARGE.  All calls on one GPU share that GPU's array: calls that can overlap
+ * on one GPU race (within one process the library already orders scans across streams;
+ * replays of different captured graphs and different processes are the caller's to keep
+ * apart).  Results are bit-identical to fss_scan_fwd_ex.
+ */
+#define FSS_NOALLOC_SCRATCH_BYTES (16u << 20)
+int fss_scan_fwd_noalloc(int dtype, const void *alpha, const void *beta, void *h, int64_t bs,
+                         int64_t seq, int64_t d, void *stream);
 
 /* Same four operations with an explicit dtype and launch configuration (tuning,
  * and tests that results do not depend on how the sequence is chunked). */

@@ -115,6 +115,21 @@ def test_entry_points_reject_bad_arguments_without_a_gpu():
     assert lib.fss_scan_fwd_ex(0, p, p, p, 1, 9, 8, None, 0, None, ctypes.byref(two_chunks)) == 4
 
 
+def test_noalloc_entry_point_refuses_oversized_shapes_before_touching_a_device():
+    lib = _native.lib()
+    buf = (ctypes.c_char * 64)()
+    p = ctypes.addressof(buf)
+    assert lib.fss_workspace_bytes(64, 8192, 4096, 0, 0, None) > _native.FSS_NOALLOC_SCRATCH_BYTES
+    assert lib.fss_scan_fwd_noalloc(0, p, p, p, 64, 8192, 4096, None) == _native.FSS_ERR_TOO_LARGE
+    assert lib.fss_scan_fwd_noalloc(0, p, p, p, -1, 4, 4, None) == 2
+    assert lib.fss_scan_fwd_noalloc(0, p, p, p, 0, 4, 4, None) == 0
+    assert "FSS_NOALLOC_SCRATCH_BYTES" in _native.strerror(_native.FSS_ERR_TOO_LARGE)
+    # every measured workload fits the static array, at any alignment
+    from fast_sequential_scan_amd.workloads import BASELINE_CASES
+    for _recipe, bs, seq, d in BASELINE_CASES.values():
+        assert lib.fss_workspace_bytes(bs, seq, d, 0, 0, None) <= _native.FSS_NOALLOC_SCRATCH_BYTES
+
+
 def test_wrappers_validate_tensors():
     a = torch.zeros(2, 4, 8, dtype=torch.bfloat16)
     with pytest.raises(RuntimeError, match="GPU"):
