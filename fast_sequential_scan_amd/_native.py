@@ -61,6 +61,7 @@ class FssConfig(ctypes.Structure):
         ("steps", ctypes.c_int32),
         ("waves", ctypes.c_int32),
         ("max_groups", ctypes.c_int32),
+        ("cols", ctypes.c_int32),
     ]
 
 
@@ -171,9 +172,10 @@ def check(status: int) -> None:
 
 
 def make_config(cfg: Optional[Tuple[int, int, int]]):
-    """(vec, steps, waves[, max_groups]) -> pointer for the *_ex entry points; None -> NULL."""
+    """(vec, steps, waves[, max_groups[, cols]]) -> pointer for the *_ex entry points; None -> NULL."""
     if cfg is None:
         return None
     vec, steps, waves = cfg[:3]
     max_groups = cfg[3] if len(cfg) > 3 else 0
-    return ctypes.byref(FssConfig(int(vec), int(steps), int(waves), int(max_groups)))
+    cols = cfg[4] if len(cfg) > 4 else 0
+    return ctypes.byref(FssConfig(int(vec), int(steps), int(waves), int(max_groups), int(cols)))

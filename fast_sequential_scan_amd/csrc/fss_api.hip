@@ -121,7 +121,9 @@ int run_scan(int dtype, int dir, const void *alpha, const void *in_b, const void
   args.n_ctiles = static_cast<int32_t>(pl.n_ctiles);
   args.n_chunks = static_cast<int32_t>(pl.n_chunks);
   args.n_tiles = static_cast<int32_t>(pl.n_tiles);
-  args.look_waves = look_waves(pl.cfg.waves, pl.cfg.vec);
+  args.n_groups = static_cast<int32_t>(pl.n_groups);
+  args.wg_cols = pl.cfg.cols;
+  args.look_waves = look_waves(pl.cfg.waves, pl.cfg.vec, pl.cfg.cols);
   args.spin_limit = __atomic_load_n(&g_spin_limit, __ATOMIC_RELAXED);
   const int64_t tensor_bytes = bs * seq * d * static_cast<int64_t>(esize);
   if (__atomic_load_n(&g_cache_policy, __ATOMIC_RELAXED) == FSS_CACHE_STREAMING)

@@ -129,6 +129,60 @@ struct DwordIO<4, NT> {
   }
 };
 
+// The kernels of the row-major layout address row segments through buffer descriptors: four
+// scalar registers per tensor and slice, the row as a scalar byte offset that all tensors share,
+// and the lane's channels as the only vector offset.  No 64-bit vector address exists per row
+// (the compiler forms one per access from a scalar base plus a lane offset otherwise, and
+// keeps dozens of them alive).  The hardware compares lane offset + row offset with the
+// descriptor's size, kRowsLimit: the offsets of a slice stay below it (the planner sees to
+// that), and a lane that must not touch memory - its channels lie beyond the end of the
+// row - carries kRowsLimit in its offset: it reads zeros and stores nothing.
+typedef __amdgpu_buffer_rsrc_t rows_t;
+constexpr int kRowsFlags = 0x00020000;  // raw 32-bit data, no swizzling
+constexpr uint32_t kRowsLimit = 0x80000000u;
+__device__ __forceinline__ rows_t make_rows(const void *first_row) {
+  return __builtin_amdgcn_make_buffer_rsrc(const_cast<void *>(uniform_ptr(first_row)), 0,
+                                           static_cast<int>(kRowsLimit), kRowsFlags);
+}
+
+template <int N, bool NT>
+struct RowsIO;
+template <bool NT>
+struct RowsIO<1, NT> {
+  static __device__ __forceinline__ void load(uint32_t *dst, rows_t r, uint32_t lane_off, int32_t row_off) {
+    dst[0] = __builtin_amdgcn_raw_buffer_load_b32(r, lane_off, row_off, NT ? 2 : 0);
+  }
+  static __device__ __forceinline__ void store(rows_t r, uint32_t lane_off, int32_t row_off, const uint32_t *src) {
+    __builtin_amdgcn_raw_buffer_store_b32(src[0], r, lane_off, row_off, NT ? 2 : 0);
+  }
+};
+template <bool NT>
+struct RowsIO<2, NT> {
+  static __device__ __forceinline__ void load(uint32_t *dst, rows_t r, uint32_t lane_off, int32_t row_off) {
+    const u32x2 v = __builtin_amdgcn_raw_buffer_load_b64(r, lane_off, row_off, NT ? 2 : 0);
+    dst[0] = v.x;
+    dst[1] = v.y;
+  }
+  static __device__ __forceinline__ void store(rows_t r, uint32_t lane_off, int32_t row_off, const uint32_t *src) {
+    const u32x2 v = {src[0], src[1]};
+    __builtin_amdgcn_raw_buffer_store_b64(v, r, lane_off, row_off, NT ? 2 : 0);
+  }
+};
+template <bool NT>
+struct RowsIO<4, NT> {
+  static __device__ __forceinline__ void load(uint32_t *dst, rows_t r, uint32_t lane_off, int32_t row_off) {
+    const u32x4 v = __builtin_amdgcn_raw_buffer_load_b128(r, lane_off, row_off, NT ? 2 : 0);
+    dst[0] = v.x;
+    dst[1] = v.y;
+    dst[2] = v.z;
+    dst[3] = v.w;
+  }
+  static __device__ __forceinline__ void store(rows_t r, uint32_t lane_off, int32_t row_off, const uint32_t *src) {
+    const u32x4 v = {src[0], src[1], src[2], src[3]};
+    __builtin_amdgcn_raw_buffer_store_b128(v, r, lane_off, row_off, NT ? 2 : 0);
+  }
+};
+
 // One row segment owned by a lane: VEC channels of element type E, kept packed.
 template <typename E, int VEC, int BYTES = E::kBytes>
 struct Row;
@@ -146,6 +200,14 @@ struct Row<E, VEC, 2> {
   template <bool NT = false>
   __device__ __forceinline__ void store(gptr_t p) const {
     DwordIO<kDwords, NT>::store(p, dw);
+  }
+  template <bool NT = false>
+  __device__ __forceinline__ void load(rows_t r, uint32_t lane_off, int32_t row_off) {
+    RowsIO<kDwords, NT>::load(dw, r, lane_off, row_off);
+  }
+  template <bool NT = false>
+  __device__ __forceinline__ void store(rows_t r, uint32_t lane_off, int32_t row_off) const {
+    RowsIO<kDwords, NT>::store(r, lane_off, row_off, dw);
   }
   __device__ __forceinline__ float get(int i) const { return (i & 1) ? E::hi(dw[i >> 1]) : E::lo(dw[i >> 1]); }
   __device__ __forceinline__ void fill(float x) {  // x exactly representable in E
@@ -177,6 +239,14 @@ struct Row<E, 1, 2> {
     else
       *q = static_cast<uint16_t>(dw[0]);
   }
+  template <bool NT = false>
+  __device__ __forceinline__ void load(rows_t r, uint32_t lane_off, int32_t row_off) {
+    dw[0] = __builtin_amdgcn_raw_buffer_load_b16(r, lane_off, row_off, NT ? 2 : 0);
+  }
+  template <bool NT = false>
+  __device__ __forceinline__ void store(rows_t r, uint32_t lane_off, int32_t row_off) const {
+    __builtin_amdgcn_raw_buffer_store_b16(static_cast<uint16_t>(dw[0]), r, lane_off, row_off, NT ? 2 : 0);
+  }
   __device__ __forceinline__ float get(int) const { return E::lo(dw[0]); }
   __device__ __forceinline__ void fill(float x) { dw[0] = E::bits(x); }
   __device__ __forceinline__ void pack(const float *f) { dw[0] = E::pack2(f[0], 0.0f) & 0xffffu; }
@@ -195,6 +265,14 @@ struct Row<E, VEC, 4> {
   template <bool NT = false>
   __device__ __forceinline__ void store(gptr_t p) const {
     DwordIO<kDwords, NT>::store(p, dw);
+  }
+  template <bool NT = false>
+  __device__ __forceinline__ void load(rows_t r, uint32_t lane_off, int32_t row_off) {
+    RowsIO<kDwords, NT>::load(dw, r, lane_off, row_off);
+  }
+  template <bool NT = false>
+  __device__ __forceinline__ void store(rows_t r, uint32_t lane_off, int32_t row_off) const {
+    RowsIO<kDwords, NT>::store(r, lane_off, row_off, dw);
   }
   __device__ __forceinline__ float get(int i) const { return as_f32(dw[i]); }
   __device__ __forceinline__ void fill(float x) {
@@ -290,8 +368,10 @@ struct ScanArgs {
   int32_t tiles_per_row;  // ceil(d / (64*VEC))
   int32_t n_ctiles;       // bs * tiles_per_row
   int32_t n_chunks;       // ceil(seq / (WAVES*STEPS))
-  int32_t n_tiles;        // n_ctiles * n_chunks
-  int32_t look_waves;     // waves that look back in parallel (1..min(WAVES, kMaxLookWaves))
+  int32_t n_tiles;        // tiles the workgroups walk: n_groups * n_chunks
+  int32_t n_groups;       // column groups per chunk: n_ctiles / wg_cols
+  int32_t wg_cols;        // adjacent column tiles a workgroup covers side by side (1 or 2)
+  int32_t look_waves;     // waves per column tile that look back in parallel (1..kMaxLookWaves)
   uint32_t spin_limit;    // polls before a look-back gives up (kSpinLimit unless a test lowered it)
   uint32_t *hdr;          // workspace header
   uint64_t *words;        // tagged words
@@ -374,7 +454,8 @@ constexpr int64_t kStreamDoutBytes = static_cast<int64_t>(80) << 20;
 
 // What is fixed for a wave while it works on one tile.
 struct TileCtx {
-  int lane, wave, n_waves, look;
+  int lane, wave, n_waves, look;   // wave, n_waves: along time, within this wave's column tile
+  int wcol;              // which of the workgroup's column tiles this wave belongs to
   int chunk, ctile;      // position of the tile: chunk of the sequence, column tile
   bool chained, last;    // more than one chunk in the sequence; this is the last one
   uint32_t tag;          // epoch of this launch
@@ -382,16 +463,29 @@ struct TileCtx {
   int64_t chan_row;      // index of (batch, first channel of the tile) in a (bs, d) array; wave-uniform
   int64_t r0;            // first scan-order index of this wave's slice
   int64_t seq, row_bytes;
-  uint32_t lane_off;     // byte offset of the lane's channels inside the tile's row segment
+  uint32_t lane_off;     // byte offset of the lane's channels inside the tile's row segment (kRowsLimit set: no such channels)
   bool col_ok;           // the lane's channels exist (d % VEC == 0, so all or none)
   float2 *lds_map;       // [wave][v][lane] = (A, B) of this tile
   float2 *lds_pred;      // [look wave][v][lane] = what an earlier chunk offers
   uint32_t *s_kind;      // [look wave] kind of that offer
+  uint32_t *s_kind_other;  // the same of the workgroup's other column tile (two column tiles per workgroup only)
   int span;              // chunks one look-back wave covers: more than 1 when the sequence has more chunks than such waves
 #ifdef FSS_TRACE
   int trace_wave;
 #endif
 };
+
+// Chunks one look-back wave covers, one after the other.  Only the chunks of a column group
+// that the grid works on at once (gridDim / n_groups of them, tiles being numbered chunk-major)
+// can still lack an outgoing state; whatever lies before them was finished in an earlier round
+// of the grid, so the first look there ends the walk.  One round of the look-back should reach
+// across those chunks; a chain it does not reach simply takes another round.
+__device__ __forceinline__ int look_span(int n_chunks, int n_groups, int look) {
+  const int in_flight = (static_cast<int>(gridDim.x) + n_groups - 1) / n_groups;
+  const int need = n_chunks - 1 < in_flight ? n_chunks - 1 : in_flight;
+  const int span = (need + look - 1) / look;
+  return span < 1 ? 1 : (span > kMaxSpan ? kMaxSpan : span);
+}
 
 // One look at what chunk `j` of this column tile offers: its outgoing state if it
 // has published one, else (j > 0) its map.  Split in two so that other work can be
@@ -553,6 +647,7 @@ __device__ __forceinline__ void chain_chunks(const ScanArgs &p, const TileCtx &c
     accB[v] = hin[v] = 0.0f;
   }
   int nearest = c.chunk - 1;  // nearest earlier chunk not folded yet
+  int other_nearest = nearest;
   // The first look goes out ahead of the loop, with `mid` in a straight line between the
   // issue of its loads and their use: only so does the compiler wait for exactly those
   // loads and not for the ones `mid` has issued behind them.
@@ -570,9 +665,15 @@ __device__ __forceinline__ void chain_chunks(const ScanArgs &p, const TileCtx &c
       mid();
     }
   }
+  // A workgroup that covers two column tiles runs two look-backs side by side, which must
+  // leave this loop together (they share the barriers).  Every wave therefore follows the
+  // other column's look-back as well: what its look-back waves found is in LDS behind the
+  // same barrier, so all waves of the workgroup see the same two answers and agree.
+  bool done = false;
+  bool other_done = p.wg_cols <= 1;  // (wg_cols is 1 wherever the kernel was compiled for one column)
   for (;;) {
     const int j = nearest - wave * c.span;
-    if (wave < c.look && j >= 0) {
+    if (!done && wave < c.look && j >= 0) {
       float qA[VEC], qB[VEC];
       uint32_t polls = 0;
       uint32_t kind = kind0;  // what the first look found (nothing, in later rounds)
@@ -635,34 +736,47 @@ __device__ __forceinline__ void chain_chunks(const ScanArgs &p, const TileCtx &c
     __syncthreads();
     // every wave folds what the look-back waves found (the same few LDS reads in each wave
     // cost less than a second barrier and a broadcast by wave 0)
-    bool resolved = false;
-    for (int w = 0; w < c.look && nearest - w * c.span >= 0 && !resolved; ++w) {
-      const bool is_state = c.s_kind[w] == kPredState;
+    if (!done) {
+      bool resolved = false;
+      for (int w = 0; w < c.look && nearest - w * c.span >= 0 && !resolved; ++w) {
+        const bool is_state = c.s_kind[w] == kPredState;
 #pragma unroll
-      for (int v = 0; v < VEC; ++v) {
-        const float2 m = c.lds_pred[(w * VEC + v) * 64 + lane];
-        if (is_state) {
-          hin[v] = fma0(accA[v], m.y, accB[v]);
-        } else {
-          accB[v] = fma0(accA[v], m.y, accB[v]);
-          accA[v] *= m.x;
+        for (int v = 0; v < VEC; ++v) {
+          const float2 m = c.lds_pred[(w * VEC + v) * 64 + lane];
+          if (is_state) {
+            hin[v] = fma0(accA[v], m.y, accB[v]);
+          } else {
+            accB[v] = fma0(accA[v], m.y, accB[v]);
+            accA[v] *= m.x;
+          }
+        }
+        resolved = is_state;
+      }
+      if (resolved) {  // chunk 0 always offers a state, so this is reached
+        done = true;
+        if (wave == 0 && !c.last) {
+#pragma unroll
+          for (int v = 0; v < VEC; ++v)
+            st_word(mine + (2 * VEC + v) * 64, c.tag, fma0(cA[v], hin[v], cB[v]));
+        }
+      } else {
+        nearest -= c.look * c.span;
+        if (nearest < 0) {  // cannot happen; never spin on a logic error
+          if (lane == 0 && wave == 0) report_timeout(p.hdr);
+          done = true;
         }
       }
-      resolved = is_state;
     }
-    if (resolved) {  // chunk 0 always offers a state, so this is reached
-      if (wave == 0 && !c.last) {
-#pragma unroll
-        for (int v = 0; v < VEC; ++v)
-          st_word(mine + (2 * VEC + v) * 64, c.tag, fma0(cA[v], hin[v], cB[v]));
+    if (!other_done) {
+      // (the other column is at the same chunk and in the same round, so the same slots count)
+      for (int w = 0; w < c.look && other_nearest - w * c.span >= 0 && !other_done; ++w)
+        other_done = c.s_kind_other[w] == kPredState;
+      if (!other_done) {
+        other_nearest -= c.look * c.span;
+        if (other_nearest < 0) other_done = true;  // as above: cannot happen
       }
-      break;
     }
-    nearest -= c.look * c.span;
-    if (nearest < 0) {  // cannot happen; never spin on a logic error
-      if (threadIdx.x == 0) report_timeout(p.hdr);
-      break;
-    }
+    if (done && other_done) break;
     __syncthreads();  // the slots are about to be overwritten: wait until every wave has read them
   }
   FSS_STAMP(c, p, 4);

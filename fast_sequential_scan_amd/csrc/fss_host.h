@@ -25,16 +25,32 @@ inline int64_t ceil_div(int64_t a, int64_t b) { return (a + b - 1) / b; }
 // Register budget: packed dwords a lane may hold per input tensor.
 inline int max_vec_steps(int dtype) { return dtype != FSS_F32 ? 64 : 32; }  // vec*steps
 
+// Most waves a workgroup of the row-major kernels may have, by what a lane holds: the kernels
+// are compiled for that many (launch bounds), so that their registers fit without spilling.
+// 16 waves leave a lane 128 registers: enough for 64 dwords of rows with up to two channels
+// per lane.  Wider lanes (whose chaining state grows with the channels) and the plain
+// backward with 32 steps of two channels (three tensors) get 256 or 512 registers instead.
+constexpr int max_waves(int esize, int vec, int steps, bool bwd, bool gated) {
+  const int dwords = vec * esize >= 4 ? vec * esize / 4 : 1;  // per lane and row
+  if (vec >= 8) return 4;
+  if (vec >= 4) return 8;
+  if (!gated && vec >= 2 && dwords * steps * (bwd ? 3 : 2) > 64) return 8;
+  return 16;
+}
+
 // LDS: one (A,B) slot per lane and vector element for every wave, twice (tiles
-// alternate between two sets), and the same for every wave that looks back.
+// alternate between two sets), and the same for every wave that looks back (per
+// column tile of the workgroup).  `waves` counts all waves of the workgroup, of which
+// waves/cols lie along time.
 constexpr size_t kLdsBudget = 60 * 1024;
-inline int look_waves(int waves, int vec) {
-  int look = waves < kMaxLookWaves ? waves : kMaxLookWaves;
-  while (look > 1 && static_cast<size_t>(2 * waves + look) * vec * 512 > kLdsBudget) --look;
+inline int look_waves(int waves, int vec, int cols = 1) {
+  const int along_time = waves / cols;
+  int look = along_time < kMaxLookWaves ? along_time : kMaxLookWaves;
+  while (look > 1 && static_cast<size_t>(2 * waves + look * cols) * vec * 512 > kLdsBudget) --look;
   return look;
 }
-inline size_t lds_bytes(int waves, int vec) {
-  return static_cast<size_t>(2 * waves + look_waves(waves, vec)) * vec * 512;
+inline size_t lds_bytes(int waves, int vec, int cols = 1) {
+  return static_cast<size_t>(2 * waves + look_waves(waves, vec, cols) * cols) * vec * 512;
 }
 
 inline bool config_valid(const fss_config &c, int dtype, bool gated = false, int dir = FSS_FWD) {
@@ -47,8 +63,10 @@ inline bool config_valid(const fss_config &c, int dtype, bool gated = false, int
   if (!vec_ok || !steps_ok) return false;
   if (c.vec * c.steps > max_vec_steps(dtype)) return false;
   if (dtype != FSS_F32 && c.vec == 1 && c.steps > 32) return false;
-  if (c.waves < 1 || c.waves > 16) return false;
-  if (lds_bytes(c.waves, c.vec) > kLdsBudget) return false;
+  if (c.waves < 1 || c.waves > max_waves(dtype != FSS_F32 ? 2 : 4, c.vec, c.steps, (dir & 1) == FSS_BWD, gated)) return false;
+  if (c.cols != 1 && c.cols != 2) return false;
+  if (c.waves % c.cols != 0) return false;
+  if (lds_bytes(c.waves, c.vec, c.cols) > kLdsBudget) return false;
   return true;
 }
 
@@ -61,6 +79,15 @@ struct Rung {
   int vec, steps, waves;
   int64_t need;
 };
+
+// Column tiles a workgroup covers side by side (fss_config.cols) when the caller leaves the
+// choice open; vec, steps and waves of `c` are already fixed.
+inline int choose_cols(const fss_config &c, int64_t bs, int64_t seq, int64_t d, int dtype, int dir, bool gated) {
+  (void)bs; (void)seq; (void)dtype; (void)dir; (void)gated;
+  const int64_t tiles_per_row = ceil_div(d, 64 * static_cast<int64_t>(c.vec));
+  if (c.waves % 2 != 0 || tiles_per_row % 2 != 0) return 1;
+  return 1;
+}
 
 // Fills the zero fields of `c`.  `align` is the common alignment in bytes of all
 // tensors of the call.
@@ -133,7 +160,7 @@ inline void complete_config(fss_config &c, int64_t bs, int64_t seq, int64_t d, i
       rung(1, 8, 8, 0);
     }
   }
-  fss_config pick = {0, 0, 0, 0};
+  fss_config pick = {0, 0, 0, 0, 0};
   for (int i = 0; i < n; ++i) {
     // what the caller fixed stays fixed
     int v = c.vec ? c.vec : ladder[i].vec;
@@ -143,8 +170,9 @@ inline void complete_config(fss_config &c, int64_t bs, int64_t seq, int64_t d, i
     // never more waves or steps than the sequence needs
     while (!c.waves && w > 1 && static_cast<int64_t>(s) * (w / 2) >= seq) w /= 2;
     while (!c.steps && s > 8 && s / 2 >= seq) s /= 2;
+    while (!c.waves && w > max_waves(esize, v, s, !fwd, gated)) w /= 2;  // (only when the caller fixed a wide lane)
     while (!c.waves && w > 1 && lds_bytes(w, v) > kLdsBudget) --w;
-    pick = fss_config{v, s, w, 0};
+    pick = fss_config{v, s, w, 0, 0};
     if (bs * ceil_div(d, 64 * static_cast<int64_t>(v)) * ceil_div(seq, static_cast<int64_t>(s) * w) >= ladder[i].need) break;
   }
   // Forward, 16-wave workgroups (one per CU) whose last round would fill less than 90 % of the
@@ -159,12 +187,15 @@ inline void complete_config(fss_config &c, int64_t bs, int64_t seq, int64_t d, i
   c.vec = pick.vec;
   c.steps = pick.steps;
   c.waves = pick.waves;
+  if (!c.cols) c.cols = choose_cols(c, bs, seq, d, dtype, dir, gated);
 }
 
 struct Plan {
   fss_config cfg;
   bool alt_policy = false;  // plain scan: the other cache policy (see kKeepOutBytes, kStreamDoutBytes)
-  int64_t tiles_per_row, n_ctiles, n_chunks, n_tiles;
+  int64_t tiles_per_row, n_ctiles, n_chunks;
+  int64_t n_groups;  // column groups per chunk: n_ctiles / cfg.cols
+  int64_t n_tiles;   // what the workgroups walk: n_groups * n_chunks
   size_t ws_bytes;
 };
 
@@ -181,22 +212,27 @@ inline int make_plan(Plan &pl, int64_t bs, int64_t seq, int64_t d, int dtype, in
     const __int128 total = static_cast<__int128>(bs) * seq * d * esize;
     if (total > (static_cast<__int128>(1) << 62)) return FSS_ERR_BAD_SHAPE;
   }
-  fss_config c = {0, 0, 0, 0};
+  fss_config c = {0, 0, 0, 0, 0};
   if (user) c = *user;
-  if (c.max_groups < 0) return FSS_ERR_BAD_CONFIG;
+  if (c.max_groups < 0 || c.cols < 0) return FSS_ERR_BAD_CONFIG;
   const int64_t dd = d > 0 ? d : 1, ss = seq > 0 ? seq : 1, bb = bs > 0 ? bs : 1;
   complete_config(c, bb, ss, dd, dtype, dir, align, gated);
   if (!config_valid(c, dtype, gated, dir)) return FSS_ERR_BAD_CONFIG;
+  // the kernels address the rows of a slice (steps + 1 of them at most) by 32-bit byte offsets
+  if (static_cast<__int128>(c.steps + 1) * dd * esize >= (static_cast<__int128>(1) << 31)) return FSS_ERR_BAD_SHAPE;
   if (dd % c.vec != 0) return FSS_ERR_BAD_CONFIG;
   if (align % (static_cast<size_t>(c.vec) * esize) != 0) return FSS_ERR_MISALIGNED;
   pl.cfg = c;
   pl.tiles_per_row = ceil_div(dd, 64 * c.vec);
+  if (pl.tiles_per_row % c.cols != 0) return FSS_ERR_BAD_CONFIG;
   pl.n_ctiles = bb * pl.tiles_per_row;
-  pl.n_chunks = ceil_div(ss, static_cast<int64_t>(c.waves) * c.steps);
-  pl.n_tiles = pl.n_ctiles * pl.n_chunks;
-  if (pl.n_ctiles > INT32_MAX || pl.n_chunks > INT32_MAX || pl.n_tiles > INT32_MAX) return FSS_ERR_BAD_SHAPE;
+  pl.n_chunks = ceil_div(ss, static_cast<int64_t>(c.waves / c.cols) * c.steps);
+  pl.n_groups = pl.n_ctiles / c.cols;
+  pl.n_tiles = pl.n_groups * pl.n_chunks;
+  if (pl.n_ctiles > INT32_MAX || pl.n_chunks > INT32_MAX || pl.n_ctiles * pl.n_chunks > INT32_MAX) return FSS_ERR_BAD_SHAPE;
   pl.ws_bytes = kHeaderBytes;
-  if (pl.n_chunks > 1) pl.ws_bytes += static_cast<size_t>(pl.n_tiles) * 3 * 64 * c.vec * sizeof(uint64_t);
+  if (pl.n_chunks > 1)
+    pl.ws_bytes += static_cast<size_t>(pl.n_ctiles * pl.n_chunks) * 3 * 64 * c.vec * sizeof(uint64_t);
   return FSS_OK;
 }
 

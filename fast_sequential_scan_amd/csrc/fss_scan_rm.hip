@@ -91,11 +91,14 @@ __device__ __forceinline__ void scan_tile(const ScanArgs &p, const StateArgs<STA
   RowT hp[BWD ? STEPS : 1];
 
   // scan-order index r -> row: forward t = r; backward t = seq-1-r, with alpha taken
-  // from row t+1 and the saved h from row t-1
+  // from row t+1 and the saved h from row t-1.  In memory the rows of a slice run upwards
+  // from row `low`; step s of the scan is row row_off(s) / row_bytes of them, whatever the tensor.
   const int64_t t_first = BWD ? seq - 1 - r0 : r0;
-  gcptr_t pa = (gcptr_t)p.in_a + c.tile_base + (BWD ? t_first + 1 : t_first) * row_bytes;
-  gcptr_t pb = (gcptr_t)p.in_b + c.tile_base + t_first * row_bytes;
-  const int64_t step_bytes = BWD ? -row_bytes : row_bytes;  // one step in scan order
+  const int64_t low = BWD ? t_first - (STEPS - 1) : t_first;
+  const int32_t rb = static_cast<int32_t>(row_bytes);  // (the planner keeps a slice below 2^31 bytes)
+  auto row_off = [rb](int s) -> int32_t { return (BWD ? STEPS - 1 - s : s) * rb; };
+  const rows_t rows_a = make_rows(p.in_a + c.tile_base + (low + (BWD ? 1 : 0)) * row_bytes);
+  const rows_t rows_b = make_rows(p.in_b + c.tile_base + low * row_bytes);
 
   FSS_STAMP(c, p, 0);
   // ---- phase 1a: issue every load of the slice -------------------------------------
@@ -105,9 +108,9 @@ __device__ __forceinline__ void scan_tile(const ScanArgs &p, const StateArgs<STA
       // The scan's very first step (r = 0) has no predecessor: its coefficient is replaced
       // below, whatever is loaded here.  The backward would find it one row past the end
       // of the sequence, so it loads the row before instead.
-      const int row = (BWD && s == 0 && r0 == 0) ? 1 : s;
-      a[s].template load<(BWD ? kNtABwd : kNtAFwd)>(uniform_ptr(pa + row * step_bytes) + lane_off);
-      b[s].template load<(BWD ? (kNtBBwd || ALT) : kNtBFwd)>(uniform_ptr(pb + s * step_bytes) + lane_off);
+      const int32_t off_a = (BWD && s == 0 && r0 == 0) ? row_off(s) - rb : row_off(s);
+      a[s].template load<(BWD ? kNtABwd : kNtAFwd)>(rows_a, lane_off, off_a);
+      b[s].template load<(BWD ? (kNtBBwd || ALT) : kNtBFwd)>(rows_b, lane_off, row_off(s));
     } else {
       const int64_t r = r0 + s;
       // Outside the sequence the step is the identity map (a=1, b=0).  The first step
@@ -115,10 +118,10 @@ __device__ __forceinline__ void scan_tile(const ScanArgs &p, const StateArgs<STA
       // state coming in, the forward applies alpha[0] to it and the backward adds it (a=1).
       a[s].fill((r >= seq || (STATE && BWD && r == 0 && st.state_in)) ? 1.0f : 0.0f);
       b[s].fill(0.0f);
-      if (c.col_ok && r < seq) {
+      if (r < seq) {  // (wave-uniform; a lane without channels reads zeros through its offset)
         if (r >= 1 || (STATE && !BWD && st.state_in))
-          a[s].template load<(BWD ? kNtABwd : kNtAFwd)>(uniform_ptr(pa + s * step_bytes) + lane_off);
-        b[s].template load<(BWD ? (kNtBBwd || ALT) : kNtBFwd)>(uniform_ptr(pb + s * step_bytes) + lane_off);
+          a[s].template load<(BWD ? kNtABwd : kNtAFwd)>(rows_a, lane_off, row_off(s));
+        b[s].template load<(BWD ? (kNtBBwd || ALT) : kNtBFwd)>(rows_b, lane_off, row_off(s));
       }
     }
   }
@@ -137,14 +140,14 @@ __device__ __forceinline__ void scan_tile(const ScanArgs &p, const StateArgs<STA
   // the registers that the steps already done have released, which is what lets a
   // lane of the backward hold as many timesteps as one of the forward.
   constexpr int kHEarly = (BWD && STEPS * Row<E, VEC>::kDwords > 16) ? STEPS / 2 : STEPS;
-  gcptr_t ph = BWD ? (gcptr_t)p.in_h + c.tile_base + (t_first - 1) * row_bytes : (gcptr_t) nullptr;
+  const rows_t rows_h = make_rows(BWD ? p.in_h + c.tile_base + (low - 1) * row_bytes : p.in_a);
   auto load_h = [&](int s) {
     if (FULL) {
-      hp[s].template load<kNtH>(uniform_ptr(ph + s * step_bytes) + lane_off);
+      hp[s].template load<kNtH>(rows_h, lane_off, row_off(s));
     } else {
       hp[s].fill(0.0f);
-      if (c.col_ok && r0 + s < seq - 1)  // t - 1 >= 0
-        hp[s].template load<kNtH>(uniform_ptr(ph + s * step_bytes) + lane_off);
+      if (r0 + s < seq - 1)  // t - 1 >= 0
+        hp[s].template load<kNtH>(rows_h, lane_off, row_off(s));
     }
   };
   auto load_h_early = [&] {
@@ -197,8 +200,8 @@ __device__ __forceinline__ void scan_tile(const ScanArgs &p, const StateArgs<STA
     keep_packed(b[s]);
     if (BWD && s < kHEarly) keep_packed(hp[s]);
   }
-  gptr_t po0 = (gptr_t)p.out0 + c.tile_base + t_first * row_bytes;
-  gptr_t po1 = BWD ? (gptr_t)p.out1 + c.tile_base + t_first * row_bytes : (gptr_t) nullptr;
+  const rows_t rows_o0 = make_rows(p.out0 + c.tile_base + low * row_bytes);
+  const rows_t rows_o1 = make_rows(BWD ? p.out1 + c.tile_base + low * row_bytes : p.out0);
 #pragma unroll
   for (int s = 0; s < STEPS; ++s) {
     float ga[VEC];
@@ -208,10 +211,10 @@ __device__ __forceinline__ void scan_tile(const ScanArgs &p, const StateArgs<STA
       if (BWD) ga[v] = state[v] * hp[s].get(v);
     }
     const int64_t r = r0 + s;
-    if (FULL || (c.col_ok && r < seq)) {
+    if (FULL || r < seq) {  // (a lane without channels stores nothing: its offset says so)
       RowT o;
       o.pack(state);
-      o.template store<(BWD ? kNtOutBwd : (kNtOutFwd && !ALT))>(uniform_ptr(po0 + s * step_bytes) + lane_off);
+      o.template store<(BWD ? kNtOutBwd : (kNtOutFwd && !ALT))>(rows_o0, lane_off, row_off(s));
       if (BWD) {
         if (!FULL && r == seq - 1) {  // t = 0: grad_alpha[0] = g[0] * h[-1], 0 in the plain scan
 #pragma unroll
@@ -220,7 +223,7 @@ __device__ __forceinline__ void scan_tile(const ScanArgs &p, const StateArgs<STA
         }
         RowT oa;
         oa.pack(ga);
-        oa.template store<kNtOutBwd>(uniform_ptr(po1 + s * step_bytes) + lane_off);
+        oa.template store<kNtOutBwd>(rows_o1, lane_off, row_off(s));
       }
     }
     if (BWD && s + kHEarly < STEPS) load_h(s + kHEarly);
@@ -231,7 +234,7 @@ __device__ __forceinline__ void scan_tile(const ScanArgs &p, const StateArgs<STA
   if (STATE && st.state_out && c.col_ok && r0 <= seq - 1 && seq - 1 < r0 + STEPS) {
     if (BWD) {
       RowT a0;
-      a0.template load<false>((gcptr_t)p.in_a + c.tile_base + lane_off);
+      a0.template load<false>((gcptr_t)p.in_a + c.tile_base + (lane_off & ~kRowsLimit));
 #pragma unroll
       for (int v = 0; v < VEC; ++v) st.state_out[c.chan_row + c.lane * VEC + v] = a0.get(v) * state[v];
     } else {
@@ -277,40 +280,44 @@ __device__ __forceinline__ void gated_tile(const ScanArgs &p, const StateArgs<ST
   RowT a[kARows], b[STEPS];
   RowT hp[BWD ? STEPS : 1], xs[BWD ? STEPS : 1];
 
-  // forward: a[s] = gate row t = r0+s.  backward: a[s] = gate row t+1 = seq-(r0+s), s = 0..STEPS
+  // forward: a[s] = gate row t = r0+s.  backward: a[s] = gate row t+1 = seq-(r0+s), s = 0..STEPS.
+  // In memory the rows of the slice run upwards from row `low` (the gate of the backward: one
+  // row more at the top); step s is row row_off(s, rows of the tensor) / row_bytes of them.
   const int64_t t_first = BWD ? seq - 1 - r0 : r0;
-  gcptr_t pa = (gcptr_t)p.in_a + c.tile_base + (BWD ? t_first + 1 : t_first) * row_bytes;
-  gcptr_t pb = (gcptr_t)p.in_b + c.tile_base + t_first * row_bytes;
-  const int64_t step_bytes = BWD ? -row_bytes : row_bytes;
+  const int64_t low = BWD ? t_first - (STEPS - 1) : t_first;
+  const int32_t rb = static_cast<int32_t>(row_bytes);  // (the planner keeps a slice below 2^31 bytes)
+  auto row_off = [rb](int s, int n_rows) -> int32_t { return (BWD ? n_rows - 1 - s : s) * rb; };
+  const rows_t rows_a = make_rows(p.in_a + c.tile_base + low * row_bytes);
+  const rows_t rows_b = make_rows(p.in_b + c.tile_base + low * row_bytes);
 
   // ---- phase 1a: loads ---------------------------------------------------------------
 #pragma unroll
   for (int s = 0; s < kARows; ++s) {
     const int64_t r = r0 + s;
     // the gate row of a[s] exists: forward r < seq; backward 1 <= r <= seq
-    const bool a_ok = FULL || (c.col_ok && (BWD ? (r >= 1 && r <= seq) : (r < seq)));
+    const bool a_ok = FULL || (BWD ? (r >= 1 && r <= seq) : (r < seq));  // (lanes without channels read zeros)
     if (!FULL) a[s].fill(0.0f);
-    if (a_ok) a[s].template load<(BWD ? kNtABwd : kNtAFwd)>(uniform_ptr(pa + s * step_bytes) + lane_off);
+    if (a_ok) a[s].template load<(BWD ? kNtABwd : kNtAFwd)>(rows_a, lane_off, row_off(s, kARows));
     if (s < STEPS) {
       if (!FULL) b[s].fill(0.0f);
-      if (FULL || (c.col_ok && r < seq)) b[s].template load<(BWD ? kNtBBwd : kNtBFwd)>(uniform_ptr(pb + s * step_bytes) + lane_off);
+      if (FULL || r < seq) b[s].template load<(BWD ? kNtBBwd : kNtBFwd)>(rows_b, lane_off, row_off(s, STEPS));
     }
   }
   // x and the saved h only feed phase 3 of the backward: half of their rows now, the
   // rest during phase 3 into registers that finished steps have released
   constexpr int kEarly = BWD ? (STEPS >= 16 ? STEPS / 2 : STEPS) : 0;
-  gcptr_t ph = BWD ? (gcptr_t)p.in_h + c.tile_base + (t_first - 1) * row_bytes : (gcptr_t) nullptr;
-  gcptr_t px = BWD ? (gcptr_t)p.in_x + c.tile_base + t_first * row_bytes : (gcptr_t) nullptr;
+  const rows_t rows_h = make_rows(BWD ? p.in_h + c.tile_base + (low - 1) * row_bytes : p.in_a);
+  const rows_t rows_x = make_rows(BWD ? p.in_x + c.tile_base + low * row_bytes : p.in_a);
   auto load_hx = [&](int s) {
     if (FULL) {
-      hp[s].template load<kNtH>(uniform_ptr(ph + s * step_bytes) + lane_off);
-      xs[s].template load<kNtH>(uniform_ptr(px + s * step_bytes) + lane_off);
+      hp[s].template load<kNtH>(rows_h, lane_off, row_off(s, STEPS));
+      xs[s].template load<kNtH>(rows_x, lane_off, row_off(s, STEPS));
     } else {
       hp[s].fill(0.0f);
       xs[s].fill(0.0f);
-      if (c.col_ok && r0 + s < seq - 1)  // t - 1 >= 0
-        hp[s].template load<kNtH>(uniform_ptr(ph + s * step_bytes) + lane_off);
-      if (c.col_ok && r0 + s < seq) xs[s].template load<kNtH>(uniform_ptr(px + s * step_bytes) + lane_off);
+      if (r0 + s < seq - 1)  // t - 1 >= 0
+        hp[s].template load<kNtH>(rows_h, lane_off, row_off(s, STEPS));
+      if (r0 + s < seq) xs[s].template load<kNtH>(rows_x, lane_off, row_off(s, STEPS));
     }
   };
   if (BWD) {
@@ -391,8 +398,8 @@ __device__ __forceinline__ void gated_tile(const ScanArgs &p, const StateArgs<ST
       keep_packed(xs[s]);
     }
   }
-  gptr_t po0 = (gptr_t)p.out0 + c.tile_base + t_first * row_bytes;
-  gptr_t po1 = BWD ? (gptr_t)p.out1 + c.tile_base + t_first * row_bytes : (gptr_t) nullptr;
+  const rows_t rows_o0 = make_rows(p.out0 + c.tile_base + low * row_bytes);
+  const rows_t rows_o1 = make_rows(BWD ? p.out1 + c.tile_base + low * row_bytes : p.out0);
 #pragma unroll
   for (int s = 0; s < STEPS; ++s) {
     const int64_t r = r0 + s;
@@ -422,14 +429,14 @@ __device__ __forceinline__ void gated_tile(const ScanArgs &p, const StateArgs<ST
         o0[v] = state[v];
       }
     }
-    if (FULL || (c.col_ok && r < seq)) {
+    if (FULL || r < seq) {
       RowT o;
       o.pack(o0);
-      o.template store<(BWD ? kNtOutBwd : kNtOutFwd)>(uniform_ptr(po0 + s * step_bytes) + lane_off);
+      o.template store<(BWD ? kNtOutBwd : kNtOutFwd)>(rows_o0, lane_off, row_off(s, STEPS));
       if (BWD) {
         RowT oz;
         oz.pack(o1);
-        oz.template store<kNtOutBwd>(uniform_ptr(po1 + s * step_bytes) + lane_off);
+        oz.template store<kNtOutBwd>(rows_o1, lane_off, row_off(s, STEPS));
       }
     }
     if (BWD && s + kEarly < STEPS) load_hx(s + kEarly);
@@ -446,29 +453,38 @@ __device__ __forceinline__ void gated_tile(const ScanArgs &p, const StateArgs<ST
 // the plain and the gated scan are compiled without them.  GATED: the gated scan.
 // ALT: the other cache policy of the plain scan - the forward for small outputs, which stores h
 // without the non-temporal hint; the backward for large tensors, which reads dout with it.
-template <typename E, int VEC, int STEPS, bool BWD, bool STATE, bool GATED = false, bool ALT = false>
-__global__ __launch_bounds__(1024) void scan_kernel(const ScanArgs p, const StateArgs<STATE> st) {
+// COLS: column tiles a workgroup covers side by side (compile-time, so that the common
+// one-column kernels keep their compile-time LDS addresses and scalar register count).
+// MAXW: the most waves a workgroup may have (max_waves of the planner): what the registers are allotted for.
+template <typename E, int VEC, int STEPS, bool BWD, bool STATE, bool GATED, bool ALT, int COLS, int MAXW>
+__global__ __launch_bounds__(MAXW * 64) void scan_kernel(const ScanArgs p, const StateArgs<STATE> st) {
   constexpr int kLaneSlots = 64 * VEC;  // channels per tile
 
   extern __shared__ float lds[];
-  __shared__ uint32_t s_kind[kMaxLookWaves];
+  __shared__ uint32_t s_kind[2 * kMaxLookWaves];
 
+  // The waves of a workgroup: wg_cols column tiles side by side, each with n_waves waves
+  // that take consecutive time slices.  Everything the chain phase touches is per column tile.
   TileCtx c;
   c.lane = threadIdx.x & 63;
-  c.wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-  c.n_waves = blockDim.x >> 6;
+  // (wave-uniform values, pinned to scalar registers: the row addresses derive from them)
+  const int wave_in_group = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int waves_total = __builtin_amdgcn_readfirstlane(blockDim.x >> 6);
+  c.n_waves = waves_total / COLS;
+  // (adjacent waves side by side: they issue the two halves of a 512-byte row segment together)
+  c.wcol = COLS > 1 ? (wave_in_group & 1) : 0;
+  c.wave = COLS > 1 ? (wave_in_group >> 1) : wave_in_group;
   c.look = p.look_waves;
-  c.span = (p.n_chunks + p.look_waves - 1) / p.look_waves;
-  if (c.span > kMaxSpan) c.span = kMaxSpan;
+  c.span = look_span(p.n_chunks, p.n_groups, p.look_waves);
   // LDS: two sets of per-wave maps (tiles alternate between them, so a wave that runs
   // ahead into the next tile cannot overwrite a map a slower wave still reads), then
   // the slots the look-back waves fill
   float2 *const lds_maps = reinterpret_cast<float2 *>(lds);
-  c.lds_pred = lds_maps + 2 * c.n_waves * kLaneSlots;
-  c.s_kind = s_kind;
+  c.lds_pred = lds_maps + (2 * waves_total + c.wcol * c.look) * kLaneSlots;
+  c.s_kind = s_kind + c.wcol * kMaxLookWaves;
+  c.s_kind_other = s_kind + (1 - c.wcol) * kMaxLookWaves;
   c.seq = p.seq;
   c.row_bytes = p.d * E::kBytes;
-  c.lane_off = static_cast<uint32_t>(c.lane * Row<E, VEC>::kBytes);
 #ifdef FSS_TRACE
   c.trace_wave = FSS_TRACE_WAVE < 0 ? c.n_waves - 1 : FSS_TRACE_WAVE;
 #endif
@@ -490,11 +506,11 @@ __global__ __launch_bounds__(1024) void scan_kernel(const ScanArgs p, const Stat
   // workgroup that reaches them no later than this one reaches its own.
   uint32_t parity = 0;
   for (uint32_t tile = blockIdx.x; tile < static_cast<uint32_t>(p.n_tiles); tile += gridDim.x, parity ^= 1u) {
-    c.lds_map = lds_maps + parity * c.n_waves * kLaneSlots;
+    c.lds_map = lds_maps + (parity * waves_total + c.wcol * c.n_waves) * kLaneSlots;
     // unsigned, wave-uniform arithmetic: stays on the scalar unit
     // (the compiler divides through a vector-unit reciprocal: pin the quotients back)
-    const uint32_t chunk = __builtin_amdgcn_readfirstlane(tile / static_cast<uint32_t>(p.n_ctiles));
-    const uint32_t ctile = tile - chunk * static_cast<uint32_t>(p.n_ctiles);
+    const uint32_t chunk = __builtin_amdgcn_readfirstlane(tile / static_cast<uint32_t>(p.n_groups));
+    const uint32_t ctile = (tile - chunk * static_cast<uint32_t>(p.n_groups)) * COLS + static_cast<uint32_t>(c.wcol);
     const uint32_t batch = __builtin_amdgcn_readfirstlane(ctile / static_cast<uint32_t>(p.tiles_per_row));
     const uint32_t coltile = ctile - batch * static_cast<uint32_t>(p.tiles_per_row);
     c.chunk = static_cast<int>(chunk);
@@ -503,6 +519,7 @@ __global__ __launch_bounds__(1024) void scan_kernel(const ScanArgs p, const Stat
 
     const int64_t col0 = static_cast<int64_t>(coltile) * kLaneSlots;  // first channel of the tile
     c.col_ok = col0 + c.lane * VEC < p.d;
+    c.lane_off = static_cast<uint32_t>(c.lane * Row<E, VEC>::kBytes) | (c.col_ok ? 0u : kRowsLimit);
     c.tile_base = (static_cast<int64_t>(batch) * c.seq * p.d + col0) * E::kBytes;
     c.chan_row = static_cast<int64_t>(batch) * p.d + col0;
     c.r0 = (static_cast<int64_t>(chunk) * c.n_waves + c.wave) * STEPS;
@@ -534,14 +551,16 @@ __global__ __launch_bounds__(1024) void scan_kernel(const ScanArgs p, const Stat
 
 // ---- launching ---------------------------------------------------------------------
 
-template <typename E, int VEC, int STEPS, bool BWD, bool STATE, bool GATED = false, bool ALT = false>
+template <typename E, int VEC, int STEPS, bool BWD, bool STATE, bool GATED = false, bool ALT = false, int COLS = 1>
 int launch_one(const ScanArgs &args, const StateArgs<true> &state, const Plan &pl, hipStream_t stream) {
   // The kernel's waits are only safe if every workgroup of the grid is resident,
   // so the grid never exceeds what the device holds at once; workgroups loop.
   static int resident[17] = {0};  // workgroups per CU by waves per workgroup
   const int waves = pl.cfg.waves;
-  const size_t lds = lds_bytes(waves, VEC);
-  const int fit = resident_workgroups(scan_kernel<E, VEC, STEPS, BWD, STATE, GATED, ALT>, waves, lds, resident);
+  const size_t lds = lds_bytes(waves, VEC, pl.cfg.cols);
+  constexpr int kMaxW = max_waves(E::kBytes, VEC, STEPS, BWD, GATED);
+  if (waves > kMaxW) return FSS_ERR_BAD_CONFIG;
+  const int fit = resident_workgroups(scan_kernel<E, VEC, STEPS, BWD, STATE, GATED, ALT, COLS, kMaxW>, waves, lds, resident);
   if (fit <= 0) return FSS_ERR_LAUNCH;
   int64_t n_groups = pl.n_tiles < fit ? pl.n_tiles : fit;
   if (pl.cfg.max_groups > 0 && pl.cfg.max_groups < n_groups) n_groups = pl.cfg.max_groups;
@@ -549,7 +568,7 @@ int launch_one(const ScanArgs &args, const StateArgs<true> &state, const Plan &p
   const dim3 block(static_cast<uint32_t>(waves) * 64);
   StateArgs<STATE> st;
   if constexpr (STATE) st = state;
-  hipLaunchKernelGGL((scan_kernel<E, VEC, STEPS, BWD, STATE, GATED, ALT>), grid, block, lds, stream, args, st);
+  hipLaunchKernelGGL((scan_kernel<E, VEC, STEPS, BWD, STATE, GATED, ALT, COLS, kMaxW>), grid, block, lds, stream, args, st);
   const hipError_t e = hipGetLastError();
   if (e != hipSuccess) {
     tls_hip_error = static_cast<int>(e);
@@ -558,9 +577,39 @@ int launch_one(const ScanArgs &args, const StateArgs<true> &state, const Plan &p
   return FSS_OK;
 }
 
+// Two column tiles per workgroup exist for the plain scan's 4-byte-per-lane kernels (the ones
+// large shapes run); config_supported_cols says the same to the planner.
+template <typename E, bool BWD>
+int launch_two_columns(const ScanArgs &args, const StateArgs<true> &state, const Plan &pl, hipStream_t stream) {
+  constexpr int V = E::kBytes == 2 ? 2 : 1;
+  if (pl.cfg.vec != V) return FSS_ERR_BAD_CONFIG;
+  switch (pl.cfg.steps) {
+#define FSS_CASE2(S)                                                                                   \
+  case S:                                                                                              \
+    if (pl.alt_policy) return launch_one<E, V, S, BWD, false, false, true, 2>(args, state, pl, stream); \
+    return launch_one<E, V, S, BWD, false, false, false, 2>(args, state, pl, stream);
+    FSS_CASE2(16)
+    default:
+      break;
+  }
+  if constexpr (!BWD) {
+    switch (pl.cfg.steps) {
+      FSS_CASE2(32)
+      default:
+        break;
+    }
+  }
+#undef FSS_CASE2
+  return FSS_ERR_BAD_CONFIG;
+}
+
 template <typename E, bool BWD, bool STATE>
 int launch_typed(const ScanArgs &args, const StateArgs<true> &state, const Plan &pl, hipStream_t stream) {
   constexpr bool is_16bit = E::kBytes == 2;
+  if (pl.cfg.cols == 2) {
+    if constexpr (STATE) return FSS_ERR_BAD_CONFIG;
+    else return launch_two_columns<E, BWD>(args, state, pl, stream);
+  }
   const int key = pl.cfg.vec * 100 + pl.cfg.steps;
   switch (key) {
 #define FSS_CASE(V, S)                                                                            \
@@ -595,6 +644,7 @@ int launch_typed(const ScanArgs &args, const StateArgs<true> &state, const Plan 
 template <typename E, bool BWD, bool STATE>
 int launch_gated(const ScanArgs &args, const StateArgs<true> &none, const Plan &pl, hipStream_t stream) {
   constexpr bool is_16bit = E::kBytes == 2;
+  if (pl.cfg.cols != 1) return FSS_ERR_BAD_CONFIG;
   const int key = pl.cfg.vec * 100 + pl.cfg.steps;
   switch (key) {
 #define FSS_CASE(V, S) \

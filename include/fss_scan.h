@@ -90,11 +90,18 @@ typedef enum fss_dir { FSS_FWD = 0, FSS_BWD = 1, FSS_GATED_FWD = 2, FSS_GATED_BW
  *          tensors aligned to vec elements
  *   steps  timesteps each lane keeps in registers (8, 16 or 32; vec*steps bounded
  *          by the register budget of the direction)
- *   waves  wavefronts per workgroup (1..16); one workgroup scans waves*steps
- *          consecutive timesteps of 64*vec channels at a time
+ *   waves  wavefronts per workgroup: 1..16; at most 8 with vec = 4 and wherever a lane with
+ *          vec = 2 holds more than 64 dwords of rows (the plain backward at 32 steps); at most
+ *          4 with vec = 8 (the kernels are compiled so that what a lane holds fits its registers)
  *   max_groups  upper bound on the workgroups launched; 0 = as many as the device
  *          holds resident at once (the grid is persistent: workgroups loop over
  *          tiles, and never more are launched than are resident together)
+ *   cols   adjacent column tiles (of 64*vec channels each) a workgroup covers side by
+ *          side, 1 or 2 (row-major kernels only; must divide waves, and with 2 the row
+ *          must hold an even number of column tiles).  A workgroup scans
+ *          (waves/cols)*steps consecutive timesteps of 64*vec*cols channels at a time;
+ *          two column tiles side by side make every row a workgroup touches 512
+ *          contiguous bytes instead of 256, which the memory system serves faster
  * Results do not depend on the configuration beyond fp32 rounding of the
  * carries handed between chunks.
  */
@@ -103,6 +110,7 @@ typedef struct fss_config {
   int32_t steps;
   int32_t waves;
   int32_t max_groups;
+  int32_t cols;
 } fss_config;
 
 int fss_abi_version(void);

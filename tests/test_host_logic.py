@@ -34,7 +34,7 @@ def plan_bytes(lib, bs, seq, d, dtype, direction, align):
     channel slot and tile when the sequence is chained)."""
     cfg = _native.FssConfig()
     assert lib.fss_choose_config(bs, seq, d, dtype, direction, align, ctypes.byref(cfg)) == 0
-    chunks = -(-seq // (cfg.steps * cfg.waves))
+    chunks = -(-seq // (cfg.steps * (cfg.waves // cfg.cols)))
     tiles = bs * -(-d // (64 * cfg.vec)) * chunks
     return 4096 + (tiles * 3 * 64 * cfg.vec * 8 if chunks > 1 else 0), cfg
 

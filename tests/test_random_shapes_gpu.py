@@ -35,8 +35,11 @@ def _draw_config(rng, dtype, d, backward, gated=False):
     budget = (64 if wide else 32) // vec
     steps = [s for s in (8, 16, 32) if s <= budget and not (gated and backward and s > 16)]
     step = int(rng.choice(steps))
+    # wide lanes and the 32-step backward are built for 8 (4) waves at most: what a lane holds must fit its registers
+    dwords = max(1, vec * (2 if wide else 4) // 4)
+    most = 4 if vec >= 8 else 8 if (vec >= 4 or (not gated and vec >= 2 and dwords * step * (3 if backward else 2) > 64)) else 16
     for _ in range(20):
-        waves = int(rng.integers(1, 17))
+        waves = int(rng.integers(1, most + 1))
         look = min(waves, 16)
         while look > 1 and (2 * waves + look + 1) * vec * 512 > 60 * 1024:
             look -= 1

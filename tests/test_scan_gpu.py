@@ -49,10 +49,18 @@ def rel_l2(x: np.ndarray, y: np.ndarray) -> float:
     return float(np.linalg.norm((x - y).ravel()) / max(np.linalg.norm(y.ravel()), 1e-30))
 
 
+def for_backward(config):
+    """The same tiling for the backward: its 32-step kernels with two channels per lane hold three
+    tensors and are built for 8 waves at most."""
+    if config is not None and config[0] == 2 and config[1] == 32 and config[2] > 8:
+        return (config[0], config[1], 8) + tuple(config[3:])
+    return config
+
+
 def run_bf16(alpha, beta, dout, config=None):
     a, b, do = alpha.to(DEV), beta.to(DEV), dout.to(DEV)
     h = ext._forward(torch.bfloat16, a, b, config)
-    ga, gb = ext._backward(torch.bfloat16, a, h, do, config)
+    ga, gb = ext._backward(torch.bfloat16, a, h, do, for_backward(config))
     torch.cuda.synchronize()
     return h, ga, gb
 
@@ -107,8 +115,8 @@ def test_bf16_default_config(oracle, recipe, seq, d):
 CONFIGS = [
     (1, 8, 1), (1, 16, 3), (1, 32, 16),
     (2, 8, 2), (2, 16, 8), (2, 32, 4), (2, 32, 16),
-    (4, 8, 5), (4, 16, 8), (4, 8, 12),
-    (8, 8, 1), (8, 8, 6),
+    (4, 8, 5), (4, 16, 8), (4, 8, 7),
+    (8, 8, 1), (8, 8, 3),
 ]
 
 
@@ -119,8 +127,76 @@ def test_bf16_result_does_not_depend_on_chunking(oracle, config):
     check_bf16(oracle, alpha, beta, dout, config=config, what=str(config))
 
 
+# (forward config, backward config): two column tiles per workgroup exist for 4 bytes per lane with
+# 16 steps (both directions) and 32 steps (forward)
+TWO_COLUMN_CONFIGS = [
+    ((2, 32, 16, 0, 2), (2, 16, 16, 0, 2)), ((2, 16, 8, 0, 2), (2, 16, 8, 0, 2)), ((2, 32, 4, 3, 2), (2, 16, 4, 3, 2)),
+    ((2, 16, 2, 0, 2), (2, 16, 2, 0, 2)), ((2, 32, 2, 5, 2), (2, 16, 2, 5, 2)), ((2, 16, 6, 0, 2), (2, 16, 12, 0, 2)),
+]
+
+
+@pytest.mark.parametrize("fwd_cfg,bwd_cfg", TWO_COLUMN_CONFIGS, ids=lambda c: "v%d_s%d_w%d_g%d_c%d" % c)
+def test_bf16_two_column_tiles_per_workgroup(oracle, fwd_cfg, bwd_cfg):
+    """Workgroups that cover two adjacent column tiles (512 contiguous bytes per row) run two
+    look-backs side by side behind shared barriers.  Short chains resolve in one round; with one
+    wave per column tile the sequence is ~49 chunks, so the two look-backs take several rounds and
+    must agree on when to leave.  Capped grids make workgroups walk many tiles."""
+    alpha, beta, dout = make_inputs("hawk", 2, 777, 512, seed=19)
+    a, b, do = alpha.to(DEV), beta.to(DEV), dout.to(DEV)
+    h = ext._forward(torch.bfloat16, a, b, fwd_cfg)
+    ga, gb = ext._backward(torch.bfloat16, a, h, do, bwd_cfg)
+    ext.workspace_status()
+    a_bits, b_bits, d_bits = bits(alpha), bits(beta), bits(dout)
+    h32 = oracle.scan_fwd_bf16_f32out(a_bits, b_bits)
+    ga32, gb32 = oracle.scan_bwd_bf16_f32out(a_bits, h32, d_bits)
+    assert_close_f32(h, h32, "h")
+    assert_close_f32(gb, gb32, "grad_beta")
+    assert_close_f32(ga, ga32, "grad_alpha")
+    # the same bits as one column tile per workgroup with the same time slicing
+    one = lambda c: (c[0], c[1], c[2] // 2, c[3], 1)  # noqa: E731
+    h1 = ext._forward(torch.bfloat16, a, b, one(fwd_cfg))
+    ga1, gb1 = ext._backward(torch.bfloat16, a, h, do, one(bwd_cfg))
+    assert torch.equal(h, h1) and torch.equal(ga, ga1) and torch.equal(gb, gb1)
+
+
+def test_two_column_tiles_f32_and_refusals(oracle):
+    import ctypes
+
+    alpha, beta, dout = make_inputs("sigmoid", 3, 515, 256, dtype=torch.float32, seed=23)
+    a, b, do = alpha.to(DEV), beta.to(DEV), dout.to(DEV)
+    for fwd_cfg, bwd_cfg in [((1, 32, 8, 0, 2), (1, 16, 8, 0, 2)), ((1, 16, 16, 0, 2), (1, 16, 2, 0, 2))]:
+        h = ext._forward(torch.float32, a, b, fwd_cfg)
+        ga, gb = ext._backward(torch.float32, a, h, do, bwd_cfg)
+        h_or = oracle.scan_fwd_f32(alpha.numpy(), beta.numpy(), fused=True)
+        ga_or, gb_or = oracle.scan_bwd_f32(alpha.numpy(), h.cpu().numpy(), dout.numpy(), fused=True)
+        np.testing.assert_allclose(h.cpu().numpy(), h_or, rtol=1e-4, atol=1e-5)
+        np.testing.assert_allclose(gb.cpu().numpy(), gb_or, rtol=1e-4, atol=1e-5)
+        np.testing.assert_allclose(ga.cpu().numpy(), ga_or, rtol=1e-4, atol=1e-5)
+    ext.workspace_status()
+    # what has no two-column kernel is refused, never run wrongly
+    lib = _native.lib()
+    sp = torch.cuda.current_stream().cuda_stream
+    t = torch.zeros(2, 64, 328, dtype=torch.bfloat16, device=DEV)
+    ws = torch.zeros(1 << 20, dtype=torch.uint8, device=DEV)
+
+    def fwd(cfg, d=256):
+        return lib.fss_scan_fwd_ex(0, t.data_ptr(), t.data_ptr(), t.data_ptr(), 2, 64, d, ws.data_ptr(), ws.numel(), sp,
+                                   ctypes.byref(_native.FssConfig(*cfg)))
+
+    assert fwd((2, 16, 4, 0, 2)) == 0
+    assert fwd((2, 16, 4, 0, 2), d=328) == 5      # three column tiles per row cannot be paired
+    assert fwd((2, 16, 3, 0, 2)) == 5             # the waves do not split over two columns
+    assert fwd((2, 8, 4, 0, 2)) == 5 and fwd((1, 16, 4, 0, 2)) == 5 and fwd((2, 16, 4, 0, 3)) == 5
+    h0 = torch.zeros(2, 256, device=DEV)
+    assert lib.fss_scan_fwd_state(0, t.data_ptr(), t.data_ptr(), t.data_ptr(), h0.data_ptr(), None, 2, 64, 256,
+                                  ws.data_ptr(), ws.numel(), sp, ctypes.byref(_native.FssConfig(2, 16, 4, 0, 2))) == 5
+    assert lib.fss_gated_scan_fwd(0, t.data_ptr(), t.data_ptr(), t.data_ptr(), 2, 64, 256, ws.data_ptr(), ws.numel(), sp,
+                                  ctypes.byref(_native.FssConfig(2, 16, 4, 0, 2))) == 5
+    torch.cuda.synchronize()
+
+
 @pytest.mark.parametrize("groups", [1, 3, 7, 64])
-@pytest.mark.parametrize("config", [(1, 8, 1), (2, 8, 3), (2, 16, 8), (2, 32, 2), (4, 8, 12)],
+@pytest.mark.parametrize("config", [(1, 8, 1), (2, 8, 3), (2, 16, 8), (2, 32, 2), (4, 8, 6)],
                          ids=lambda c: "v%d_s%d_w%d" % c)
 def test_bf16_few_workgroups_walk_many_tiles(oracle, config, groups):
     """The grid is persistent: cap it far below the tile count, so that every workgroup
