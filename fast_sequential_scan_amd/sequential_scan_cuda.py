@@ -197,8 +197,26 @@ def workspace_status(device: Optional[torch.device] = None) -> None:
                 ws.flag_word.value = 0
 
 
+def _same_kind(dtype: torch.dtype, first, *others) -> bool:
+    """The common case of _validate in a few attribute reads: GPU tensors of `dtype`, rank 3, one
+    shape, one device.  Anything else goes through _validate, which names what is wrong."""
+    try:
+        if first.dtype is not dtype or not first.is_cuda or first.dim() != 3:
+            return False
+        shape, device = first.shape, first.device
+        for t in others:
+            if t.dtype is not dtype or t.shape != shape or t.device != device:
+                return False
+        return True
+    except AttributeError:  # not a tensor
+        return False
+
+
 def _forward(dtype: torch.dtype, alpha: torch.Tensor, beta: torch.Tensor, config=None) -> torch.Tensor:
-    bs, seq, d = _validate(dtype, alpha=alpha, beta=beta)
+    if _same_kind(dtype, alpha, beta):
+        bs, seq, d = alpha.shape
+    else:
+        bs, seq, d = _validate(dtype, alpha=alpha, beta=beta)
     alpha, beta = _contiguous(alpha), _contiguous(beta)
     out = torch.empty_like(alpha)
     if out.numel() == 0:
@@ -219,7 +237,10 @@ def _forward(dtype: torch.dtype, alpha: torch.Tensor, beta: torch.Tensor, config
 def _backward(
     dtype: torch.dtype, alpha_saved: torch.Tensor, h_saved: torch.Tensor, grad_out: torch.Tensor, config=None
 ) -> List[torch.Tensor]:
-    bs, seq, d = _validate(dtype, alpha_saved=alpha_saved, h_saved=h_saved, grad_out=grad_out)
+    if _same_kind(dtype, alpha_saved, h_saved, grad_out):
+        bs, seq, d = alpha_saved.shape
+    else:
+        bs, seq, d = _validate(dtype, alpha_saved=alpha_saved, h_saved=h_saved, grad_out=grad_out)
     alpha_saved, h_saved, grad_out = _contiguous(alpha_saved), _contiguous(h_saved), _contiguous(grad_out)
     grad_alpha = torch.empty_like(alpha_saved)
     grad_beta = torch.empty_like(alpha_saved)
