@@ -129,60 +129,6 @@ struct DwordIO<4, NT> {
   }
 };
 
-// The kernels of the row-major layout address row segments through buffer descriptors: four
-// scalar registers per tensor and slice, the row as a scalar byte offset that all tensors share,
-// and the lane's channels as the only vector offset.  No 64-bit vector address exists per row
-// (the compiler forms one per access from a scalar base plus a lane offset otherwise, and
-// keeps dozens of them alive).  The hardware compares lane offset + row offset with the
-// descriptor's size, kRowsLimit: the offsets of a slice stay below it (the planner sees to
-// that), and a lane that must not touch memory - its channels lie beyond the end of the
-// row - carries kRowsLimit in its offset: it reads zeros and stores nothing.
-typedef __amdgpu_buffer_rsrc_t rows_t;
-constexpr int kRowsFlags = 0x00020000;  // raw 32-bit data, no swizzling
-constexpr uint32_t kRowsLimit = 0x80000000u;
-__device__ __forceinline__ rows_t make_rows(const void *first_row) {
-  return __builtin_amdgcn_make_buffer_rsrc(const_cast<void *>(uniform_ptr(first_row)), 0,
-                                           static_cast<int>(kRowsLimit), kRowsFlags);
-}
-
-template <int N, bool NT>
-struct RowsIO;
-template <bool NT>
-struct RowsIO<1, NT> {
-  static __device__ __forceinline__ void load(uint32_t *dst, rows_t r, uint32_t lane_off, int32_t row_off) {
-    dst[0] = __builtin_amdgcn_raw_buffer_load_b32(r, lane_off, row_off, NT ? 2 : 0);
-  }
-  static __device__ __forceinline__ void store(rows_t r, uint32_t lane_off, int32_t row_off, const uint32_t *src) {
-    __builtin_amdgcn_raw_buffer_store_b32(src[0], r, lane_off, row_off, NT ? 2 : 0);
-  }
-};
-template <bool NT>
-struct RowsIO<2, NT> {
-  static __device__ __forceinline__ void load(uint32_t *dst, rows_t r, uint32_t lane_off, int32_t row_off) {
-    const u32x2 v = __builtin_amdgcn_raw_buffer_load_b64(r, lane_off, row_off, NT ? 2 : 0);
-    dst[0] = v.x;
-    dst[1] = v.y;
-  }
-  static __device__ __forceinline__ void store(rows_t r, uint32_t lane_off, int32_t row_off, const uint32_t *src) {
-    const u32x2 v = {src[0], src[1]};
-    __builtin_amdgcn_raw_buffer_store_b64(v, r, lane_off, row_off, NT ? 2 : 0);
-  }
-};
-template <bool NT>
-struct RowsIO<4, NT> {
-  static __device__ __forceinline__ void load(uint32_t *dst, rows_t r, uint32_t lane_off, int32_t row_off) {
-    const u32x4 v = __builtin_amdgcn_raw_buffer_load_b128(r, lane_off, row_off, NT ? 2 : 0);
-    dst[0] = v.x;
-    dst[1] = v.y;
-    dst[2] = v.z;
-    dst[3] = v.w;
-  }
-  static __device__ __forceinline__ void store(rows_t r, uint32_t lane_off, int32_t row_off, const uint32_t *src) {
-    const u32x4 v = {src[0], src[1], src[2], src[3]};
-    __builtin_amdgcn_raw_buffer_store_b128(v, r, lane_off, row_off, NT ? 2 : 0);
-  }
-};
-
 // One row segment owned by a lane: VEC channels of element type E, kept packed.
 template <typename E, int VEC, int BYTES = E::kBytes>
 struct Row;
@@ -200,14 +146,6 @@ struct Row<E, VEC, 2> {
   template <bool NT = false>
   __device__ __forceinline__ void store(gptr_t p) const {
     DwordIO<kDwords, NT>::store(p, dw);
-  }
-  template <bool NT = false>
-  __device__ __forceinline__ void load(rows_t r, uint32_t lane_off, int32_t row_off) {
-    RowsIO<kDwords, NT>::load(dw, r, lane_off, row_off);
-  }
-  template <bool NT = false>
-  __device__ __forceinline__ void store(rows_t r, uint32_t lane_off, int32_t row_off) const {
-    RowsIO<kDwords, NT>::store(r, lane_off, row_off, dw);
   }
   __device__ __forceinline__ float get(int i) const { return (i & 1) ? E::hi(dw[i >> 1]) : E::lo(dw[i >> 1]); }
   __device__ __forceinline__ void fill(float x) {  // x exactly representable in E
@@ -239,14 +177,6 @@ struct Row<E, 1, 2> {
     else
       *q = static_cast<uint16_t>(dw[0]);
   }
-  template <bool NT = false>
-  __device__ __forceinline__ void load(rows_t r, uint32_t lane_off, int32_t row_off) {
-    dw[0] = __builtin_amdgcn_raw_buffer_load_b16(r, lane_off, row_off, NT ? 2 : 0);
-  }
-  template <bool NT = false>
-  __device__ __forceinline__ void store(rows_t r, uint32_t lane_off, int32_t row_off) const {
-    __builtin_amdgcn_raw_buffer_store_b16(static_cast<uint16_t>(dw[0]), r, lane_off, row_off, NT ? 2 : 0);
-  }
   __device__ __forceinline__ float get(int) const { return E::lo(dw[0]); }
   __device__ __forceinline__ void fill(float x) { dw[0] = E::bits(x); }
   __device__ __forceinline__ void pack(const float *f) { dw[0] = E::pack2(f[0], 0.0f) & 0xffffu; }
@@ -266,14 +196,6 @@ struct Row<E, VEC, 4> {
   __device__ __forceinline__ void store(gptr_t p) const {
     DwordIO<kDwords, NT>::store(p, dw);
   }
-  template <bool NT = false>
-  __device__ __forceinline__ void load(rows_t r, uint32_t lane_off, int32_t row_off) {
-    RowsIO<kDwords, NT>::load(dw, r, lane_off, row_off);
-  }
-  template <bool NT = false>
-  __device__ __forceinline__ void store(rows_t r, uint32_t lane_off, int32_t row_off) const {
-    RowsIO<kDwords, NT>::store(r, lane_off, row_off, dw);
-  }
   __device__ __forceinline__ float get(int i) const { return as_f32(dw[i]); }
   __device__ __forceinline__ void fill(float x) {
 #pragma unroll
@@ -284,6 +206,16 @@ struct Row<E, VEC, 4> {
     for (int i = 0; i < kDwords; ++i) dw[i] = as_u32(f[i]);
   }
 };
+
+// seq - r0 clamped to [-1, cap] as a wave-uniform 32-bit integer: how many steps of a slice
+// that starts at scan-order index r0 lie inside the sequence.  With it, "r0 + s < seq" is
+// "s < n", "r0 + s <= seq" is "s <= n" and so on for every step s >= 0 of the slice; -1
+// (the slice starts beyond index seq) keeps "s <= n" false where 0 would make it true for s = 0.
+__device__ __forceinline__ int slice_steps_inside(int64_t seq, int64_t r0, int cap) {
+  const int64_t left = seq - r0;
+  const int n = left < 0 ? -1 : (left >= cap ? cap : static_cast<int>(left));
+  return __builtin_amdgcn_readfirstlane(n);
+}
 
 // Makes the compiler forget what it derived from a packed row: the rows stay
 // packed in registers across the chaining phase and are unpacked again after
@@ -373,8 +305,10 @@ struct ScanArgs {
   int32_t wg_cols;        // adjacent column tiles a workgroup covers side by side (1 or 2)
   int32_t look_waves;     // waves per column tile that look back in parallel (1..kMaxLookWaves)
   uint32_t spin_limit;    // polls before a look-back gives up (kSpinLimit unless a test lowered it)
+  int32_t block_chunks;   // chunks per block of the two-level chain; n_chunks or more: one level
   uint32_t *hdr;          // workspace header
   uint64_t *words;        // tagged words
+  uint64_t *block_words;  // tagged words of the blocks' maps, [block][column tile][A, B][VEC][64]
   const char *in_x;       // gated backward only: the scan's input x (in_a is the gate there)
 #ifdef FSS_TRACE
   uint64_t *trace;        // debug build: 8 timestamps per tile, written by lane 0 of every wave 0
@@ -463,7 +397,7 @@ struct TileCtx {
   int64_t chan_row;      // index of (batch, first channel of the tile) in a (bs, d) array; wave-uniform
   int64_t r0;            // first scan-order index of this wave's slice
   int64_t seq, row_bytes;
-  uint32_t lane_off;     // byte offset of the lane's channels inside the tile's row segment (kRowsLimit set: no such channels)
+  uint32_t lane_off;     // byte offset of the lane's channels inside the tile's row segment
   bool col_ok;           // the lane's channels exist (d % VEC == 0, so all or none)
   float2 *lds_map;       // [wave][v][lane] = (A, B) of this tile
   float2 *lds_pred;      // [look wave][v][lane] = what an earlier chunk offers
@@ -475,41 +409,80 @@ struct TileCtx {
 #endif
 };
 
-// Chunks one look-back wave covers, one after the other.  Only the chunks of a column group
+// Places one look-back wave covers, one after the other.  Only the chunks of a column group
 // that the grid works on at once (gridDim / n_groups of them, tiles being numbered chunk-major)
 // can still lack an outgoing state; whatever lies before them was finished in an earlier round
 // of the grid, so the first look there ends the walk.  One round of the look-back should reach
-// across those chunks; a chain it does not reach simply takes another round.
-__device__ __forceinline__ int look_span(int n_chunks, int n_groups, int look) {
+// across those chunks (with blocks: across the rest of the tile's own block and the blocks in
+// flight before it); a chain it does not reach simply takes another round.
+__device__ __forceinline__ int look_span(int n_chunks, int n_groups, int look, int block_chunks) {
   const int in_flight = (static_cast<int>(gridDim.x) + n_groups - 1) / n_groups;
-  const int need = n_chunks - 1 < in_flight ? n_chunks - 1 : in_flight;
+  int need = n_chunks - 1 < in_flight ? n_chunks - 1 : in_flight;
+  if (block_chunks < n_chunks) {
+    const int in_block = block_chunks - 1 < in_flight ? block_chunks - 1 : in_flight;
+    const int blocks = (n_chunks + block_chunks - 1) / block_chunks - 1;
+    const int blocks_in_flight = in_flight / block_chunks + 1;
+    need = in_block + (blocks < blocks_in_flight ? blocks : blocks_in_flight);
+  }
   const int span = (need + look - 1) / look;
   return span < 1 ? 1 : (span > kMaxSpan ? kMaxSpan : span);
 }
 
-// One look at what chunk `j` of this column tile offers: its outgoing state if it
-// has published one, else (j > 0) its map.  Split in two so that other work can be
-// placed between the loads and the use of what they return.
+// What a look-back can learn from one place: the state leaving a chunk, if that chunk has
+// published it, else a map that leads to it from further back.  Two kinds of places exist:
+//   chunk j    its outgoing state, else (j > 0) its own map;
+//   block h    (chains of many chunks are cut into blocks of block_chunks chunks) the state
+//              leaving the block's last chunk, else the block's map: the composition of all its
+//              chunks' maps, published by its last chunk once it has seen the maps of the others.
+// Split in two so that other work can be placed between the loads and the use of what they return.
 template <int VEC>
 struct ChunkWords {
   uint64_t a[VEC], b[VEC], s[VEC];
 };
 
+// Where the words of look-back item `item` of this tile lie.  Items are numbered in the order
+// of the walk back: first the chunks of the tile's own block, nearest first, then the earlier
+// blocks, nearest first.
+struct LookItem {
+  const uint64_t *state;  // [VEC][64] words of the state
+  const uint64_t *map;    // [2][VEC][64] words of the map, A then B
+  bool map_ok;            // a map may be taken (chunk 0 of a sequence has none: its state is there at once)
+};
+
 template <int VEC>
-__device__ __forceinline__ void poll_issue(const ScanArgs &p, const TileCtx &c, int j, ChunkWords<VEC> &w) {
-  const uint64_t *theirs = p.words + (static_cast<size_t>(j) * p.n_ctiles + c.ctile) * 3 * (64 * VEC) + c.lane;
+__device__ __forceinline__ LookItem look_item(const ScanArgs &p, const TileCtx &c, int n_in, int block, int item) {
+  constexpr size_t kLaneSlots = 64 * VEC;
+  LookItem it;
+  if (item < n_in) {
+    const int j = c.chunk - 1 - item;
+    const uint64_t *w = p.words + (static_cast<size_t>(j) * p.n_ctiles + c.ctile) * 3 * kLaneSlots + c.lane;
+    it.state = w + 2 * kLaneSlots;
+    it.map = w;
+    it.map_ok = j > 0;
+  } else {
+    const int h = block - 1 - (item - n_in);
+    const int j = h * p.block_chunks + p.block_chunks - 1;  // the block's last chunk
+    it.state = p.words + (static_cast<size_t>(j) * p.n_ctiles + c.ctile) * 3 * kLaneSlots + 2 * kLaneSlots + c.lane;
+    it.map = p.block_words + (static_cast<size_t>(h) * p.n_ctiles + c.ctile) * 2 * kLaneSlots + c.lane;
+    it.map_ok = true;
+  }
+  return it;
+}
+
+template <int VEC>
+__device__ __forceinline__ void poll_issue(const LookItem &it, ChunkWords<VEC> &w) {
 #pragma unroll
   for (int v = 0; v < VEC; ++v) {
-    w.s[v] = ld_word(theirs + (2 * VEC + v) * 64);
-    w.a[v] = ld_word(theirs + (0 * VEC + v) * 64);
-    w.b[v] = ld_word(theirs + (1 * VEC + v) * 64);
+    w.s[v] = ld_word(it.state + v * 64);
+    w.a[v] = ld_word(it.map + (0 * VEC + v) * 64);
+    w.b[v] = ld_word(it.map + (1 * VEC + v) * 64);
   }
 }
 
 // The answer is taken for the whole wave, so that one word per wave can describe
 // it.  Returns kPredNone when neither a state nor a map is there yet.
 template <int VEC>
-__device__ __forceinline__ uint32_t poll_eval(const TileCtx &c, int j, const ChunkWords<VEC> &w, float *qA,
+__device__ __forceinline__ uint32_t poll_eval(const TileCtx &c, const LookItem &it, const ChunkWords<VEC> &w, float *qA,
                                               float *qB) {
   bool have_state = true, have_map = true;
 #pragma unroll
@@ -525,7 +498,7 @@ __device__ __forceinline__ uint32_t poll_eval(const TileCtx &c, int j, const Chu
     }
     return kPredState;
   }
-  if (j > 0 && __builtin_amdgcn_ballot_w64(have_map) == ~0ull) {
+  if (it.map_ok && __builtin_amdgcn_ballot_w64(have_map) == ~0ull) {
 #pragma unroll
     for (int v = 0; v < VEC; ++v) {
       qA[v] = word_val(w.a[v]);
@@ -537,11 +510,10 @@ __device__ __forceinline__ uint32_t poll_eval(const TileCtx &c, int j, const Chu
 }
 
 template <int VEC>
-__device__ __forceinline__ uint32_t poll_chunk(const ScanArgs &p, const TileCtx &c, int j, float *qA,
-                                               float *qB) {
+__device__ __forceinline__ uint32_t poll_item(const TileCtx &c, const LookItem &it, float *qA, float *qB) {
   ChunkWords<VEC> w;
-  poll_issue<VEC>(p, c, j, w);
-  return poll_eval<VEC>(c, j, w, qA, qB);
+  poll_issue<VEC>(it, w);
+  return poll_eval<VEC>(c, it, w, qA, qB);
 }
 
 // (A, B) <- map[count-1] o ... o map[0] for this lane's channels: the maps of the
@@ -646,8 +618,31 @@ __device__ __forceinline__ void chain_chunks(const ScanArgs &p, const TileCtx &c
     accA[v] = 1.0f;
     accB[v] = hin[v] = 0.0f;
   }
-  int nearest = c.chunk - 1;  // nearest earlier chunk not folded yet
-  int other_nearest = nearest;
+  // The walk back.  Its places ("items"): the chunks before this one in its own block, nearest
+  // first (n_in of them), then the earlier blocks, nearest first.  With one level the whole
+  // sequence is one block.  Look-back wave w takes entry first_entry + w of the walk: `span`
+  // consecutive items that it asks one after the other (an entry never crosses from the chunks
+  // to the blocks, so that what the chunks of the own block do is known apart: the block's map
+  // is that composed with this chunk's map).
+  const int block = c.chunk / p.block_chunks;
+  const int n_in = c.chunk - block * p.block_chunks;
+  const int span = c.span;
+  const int entries_in = (n_in + span - 1) / span;
+  const int entries = entries_in + (block + span - 1) / span;
+  // this chunk closes its block and later blocks exist: it owes them the block's map
+  const bool owes_block_map = n_in == p.block_chunks - 1 && !c.last && block > 0;
+  int first_entry = 0;  // first entry not folded yet
+  // (item range of an entry)
+  auto entry_items = [&](int e, int &first_item, int &count) {
+    if (e < entries_in) {
+      first_item = e * span;
+      count = n_in - first_item < span ? n_in - first_item : span;
+    } else {
+      const int f = (e - entries_in) * span;
+      first_item = n_in + f;
+      count = block - f < span ? block - f : span;
+    }
+  };
   // The first look goes out ahead of the loop, with `mid` in a straight line between the
   // issue of its loads and their use: only so does the compiler wait for exactly those
   // loads and not for the ones `mid` has issued behind them.
@@ -656,11 +651,14 @@ __device__ __forceinline__ void chain_chunks(const ScanArgs &p, const TileCtx &c
 #pragma unroll
   for (int v = 0; v < VEC; ++v) q0A[v] = q0B[v] = 0.0f;
   if constexpr (HAS_MID) {
-    if (wave < c.look && nearest - wave * c.span >= 0) {
+    if (wave < c.look && wave < entries) {
+      int first_item, count;
+      entry_items(wave, first_item, count);
+      const LookItem it = look_item<VEC>(p, c, n_in, block, first_item);
       ChunkWords<VEC> w;
-      poll_issue<VEC>(p, c, nearest - wave * c.span, w);
+      poll_issue<VEC>(it, w);
       mid();
-      kind0 = poll_eval<VEC>(c, nearest - wave * c.span, w, q0A, q0B);
+      kind0 = poll_eval<VEC>(c, it, w, q0A, q0B);
     } else {
       mid();
     }
@@ -671,11 +669,13 @@ __device__ __forceinline__ void chain_chunks(const ScanArgs &p, const TileCtx &c
   // same barrier, so all waves of the workgroup see the same two answers and agree.
   bool done = false;
   bool other_done = p.wg_cols <= 1;  // (wg_cols is 1 wherever the kernel was compiled for one column)
+  int other_first_entry = 0;
   for (;;) {
-    const int j = nearest - wave * c.span;
-    if (!done && wave < c.look && j >= 0) {
+    const int e = first_entry + wave;
+    if (!done && wave < c.look && e < entries) {
+      int first_item, count;
+      entry_items(e, first_item, count);
       float qA[VEC], qB[VEC];
-      uint32_t polls = 0;
       uint32_t kind = kind0;  // what the first look found (nothing, in later rounds)
 #pragma unroll
       for (int v = 0; v < VEC; ++v) {
@@ -684,50 +684,52 @@ __device__ __forceinline__ void chain_chunks(const ScanArgs &p, const TileCtx &c
       }
       kind0 = kPredNone;
       if (p.spin_limit == 0) kind = kPredNone;
-      while (kind == kPredNone) {
-        if (polls >= p.spin_limit) {
-          // give up, so that the grid still drains: a NaN state poisons what follows
-          if (lane == 0) report_timeout(p.hdr);
-          kind = kPredState;
-#pragma unroll
-          for (int v = 0; v < VEC; ++v) {
-            qA[v] = 0.0f;
-            qB[v] = __builtin_nanf("");
-          }
-          break;
-        }
-        kind = poll_chunk<VEC>(p, c, j, qA, qB);
-        if (kind != kPredNone) break;
-        ++polls;
-        __builtin_amdgcn_s_sleep(2);
-      }
-      // long chains: the wave also takes the chunks before that one (by now they have nearly
-      // always published), so that one round of the look-back reaches `span` times as far
-      for (int k = 1; k < c.span && kind == kPredMap && j - k >= 0; ++k) {
+      // the entry's items one after the other, as long as they answer with maps (by the time
+      // the first has answered, the ones behind it nearly always have published too)
+      for (int k = 0; k < count && (k == 0 || kind == kPredMap); ++k) {
         float rA[VEC], rB[VEC];
-        polls = 0;
-        for (;;) {
-          if (polls >= p.spin_limit) {
-            if (lane == 0) report_timeout(p.hdr);
-            kind = kPredState;
-#pragma unroll
-            for (int v = 0; v < VEC; ++v) {
-              rA[v] = 0.0f;
-              rB[v] = __builtin_nanf("");
-            }
-            break;
-          }
-          kind = poll_chunk<VEC>(p, c, j - k, rA, rB);
-          if (kind != kPredNone) break;
-          ++polls;
-          __builtin_amdgcn_s_sleep(2);
-        }
-        // (a state is the map x -> 0*x + value)
+        uint32_t got = k == 0 ? kind : kPredNone;
 #pragma unroll
         for (int v = 0; v < VEC; ++v) {
-          qB[v] = fma0(qA[v], rB[v], qB[v]);
-          qA[v] *= rA[v];
+          rA[v] = qA[v];
+          rB[v] = qB[v];
         }
+        if (got == kPredNone) {
+          const LookItem it = look_item<VEC>(p, c, n_in, block, first_item + k);
+          uint32_t polls = 0;
+          for (;;) {
+            if (polls >= p.spin_limit) {
+              // give up, so that the grid still drains: a NaN state poisons what follows
+              if (lane == 0) report_timeout(p.hdr);
+              got = kPredState;
+#pragma unroll
+              for (int v = 0; v < VEC; ++v) {
+                rA[v] = 0.0f;
+                rB[v] = __builtin_nanf("");
+              }
+              break;
+            }
+            got = poll_item<VEC>(c, it, rA, rB);
+            if (got != kPredNone) break;
+            ++polls;
+            __builtin_amdgcn_s_sleep(2);
+          }
+        }
+        if (k == 0) {
+#pragma unroll
+          for (int v = 0; v < VEC; ++v) {
+            qA[v] = rA[v];
+            qB[v] = rB[v];
+          }
+        } else {
+          // (a state is the map x -> 0*x + value)
+#pragma unroll
+          for (int v = 0; v < VEC; ++v) {
+            qB[v] = fma0(qA[v], rB[v], qB[v]);
+            qA[v] *= rA[v];
+          }
+        }
+        kind = got;
       }
 #pragma unroll
       for (int v = 0; v < VEC; ++v) c.lds_pred[(wave * VEC + v) * 64 + lane] = make_float2(qA[v], qB[v]);
@@ -738,7 +740,7 @@ __device__ __forceinline__ void chain_chunks(const ScanArgs &p, const TileCtx &c
     // cost less than a second barrier and a broadcast by wave 0)
     if (!done) {
       bool resolved = false;
-      for (int w = 0; w < c.look && nearest - w * c.span >= 0 && !resolved; ++w) {
+      for (int w = 0; w < c.look && first_entry + w < entries && !resolved; ++w) {
         const bool is_state = c.s_kind[w] == kPredState;
 #pragma unroll
         for (int v = 0; v < VEC; ++v) {
@@ -751,6 +753,16 @@ __device__ __forceinline__ void chain_chunks(const ScanArgs &p, const TileCtx &c
           }
         }
         resolved = is_state;
+        // all chunks of the own block have answered with maps: the block's map is theirs
+        // composed with this chunk's, and it goes out at once
+        if (owes_block_map && wave == 0 && !is_state && first_entry + w == entries_in - 1) {
+          uint64_t *blk = p.block_words + (static_cast<size_t>(block) * p.n_ctiles + c.ctile) * 2 * kLaneSlots + lane;
+#pragma unroll
+          for (int v = 0; v < VEC; ++v) {
+            st_word(blk + (0 * VEC + v) * 64, c.tag, cA[v] * accA[v]);
+            st_word(blk + (1 * VEC + v) * 64, c.tag, fma0(cA[v], accB[v], cB[v]));
+          }
+        }
       }
       if (resolved) {  // chunk 0 always offers a state, so this is reached
         done = true;
@@ -760,8 +772,8 @@ __device__ __forceinline__ void chain_chunks(const ScanArgs &p, const TileCtx &c
             st_word(mine + (2 * VEC + v) * 64, c.tag, fma0(cA[v], hin[v], cB[v]));
         }
       } else {
-        nearest -= c.look * c.span;
-        if (nearest < 0) {  // cannot happen; never spin on a logic error
+        first_entry += c.look;
+        if (first_entry >= entries) {  // cannot happen; never spin on a logic error
           if (lane == 0 && wave == 0) report_timeout(p.hdr);
           done = true;
         }
@@ -769,11 +781,11 @@ __device__ __forceinline__ void chain_chunks(const ScanArgs &p, const TileCtx &c
     }
     if (!other_done) {
       // (the other column is at the same chunk and in the same round, so the same slots count)
-      for (int w = 0; w < c.look && other_nearest - w * c.span >= 0 && !other_done; ++w)
+      for (int w = 0; w < c.look && other_first_entry + w < entries && !other_done; ++w)
         other_done = c.s_kind_other[w] == kPredState;
       if (!other_done) {
-        other_nearest -= c.look * c.span;
-        if (other_nearest < 0) other_done = true;  // as above: cannot happen
+        other_first_entry += c.look;
+        if (other_first_entry >= entries) other_done = true;  // as above: cannot happen
       }
     }
     if (done && other_done) break;

@@ -196,8 +196,26 @@ struct Plan {
   int64_t tiles_per_row, n_ctiles, n_chunks;
   int64_t n_groups;  // column groups per chunk: n_ctiles / cfg.cols
   int64_t n_tiles;   // what the workgroups walk: n_groups * n_chunks
+  int64_t block_chunks;  // chunks per block of the two-level chain (n_chunks: one level)
+  size_t block_words_offset;  // where the blocks' words start in the workspace (0: none)
   size_t ws_bytes;
 };
+
+// Chunks per block.  A look-back walks over the chunks before its own, as far as to the first
+// that has published its outgoing state; the chunks of a sequence that are in flight together
+// have none yet, so with c of them each walk reads up to c maps: c^2/2 in all.  Cut into
+// blocks of b chunks whose last chunk publishes the block's map, a walk reads at most b - 1
+// chunk maps and c/b block maps.  Worth its extra round trip (the block's map comes one look
+// after the chunks' maps) only where many chunks of a sequence are in flight: few columns,
+// long sequences.  0 from the debug knob means this choice.
+extern int g_block_chunks;  // fss_debug_set_block_chunks
+inline int64_t choose_block_chunks(int64_t n_chunks, int64_t n_groups) {
+  const int forced = __atomic_load_n(&g_block_chunks, __ATOMIC_RELAXED);
+  if (forced >= 2) return forced < n_chunks ? forced : n_chunks;
+  const int64_t in_flight = ceil_div(kCus, n_groups);  // chunks of one column group the grid holds at once
+  if (n_chunks <= 24 || in_flight <= 12) return n_chunks;
+  return n_chunks <= 160 ? 8 : 16;
+}
 
 inline int make_plan(Plan &pl, int64_t bs, int64_t seq, int64_t d, int dtype, int dir, size_t align,
               const fss_config *user) {
@@ -218,8 +236,6 @@ inline int make_plan(Plan &pl, int64_t bs, int64_t seq, int64_t d, int dtype, in
   const int64_t dd = d > 0 ? d : 1, ss = seq > 0 ? seq : 1, bb = bs > 0 ? bs : 1;
   complete_config(c, bb, ss, dd, dtype, dir, align, gated);
   if (!config_valid(c, dtype, gated, dir)) return FSS_ERR_BAD_CONFIG;
-  // the kernels address the rows of a slice (steps + 1 of them at most) by 32-bit byte offsets
-  if (static_cast<__int128>(c.steps + 1) * dd * esize >= (static_cast<__int128>(1) << 31)) return FSS_ERR_BAD_SHAPE;
   if (dd % c.vec != 0) return FSS_ERR_BAD_CONFIG;
   if (align % (static_cast<size_t>(c.vec) * esize) != 0) return FSS_ERR_MISALIGNED;
   pl.cfg = c;
@@ -231,8 +247,16 @@ inline int make_plan(Plan &pl, int64_t bs, int64_t seq, int64_t d, int dtype, in
   pl.n_tiles = pl.n_groups * pl.n_chunks;
   if (pl.n_ctiles > INT32_MAX || pl.n_chunks > INT32_MAX || pl.n_ctiles * pl.n_chunks > INT32_MAX) return FSS_ERR_BAD_SHAPE;
   pl.ws_bytes = kHeaderBytes;
-  if (pl.n_chunks > 1)
+  pl.block_chunks = pl.n_chunks;
+  pl.block_words_offset = 0;
+  if (pl.n_chunks > 1) {
     pl.ws_bytes += static_cast<size_t>(pl.n_ctiles * pl.n_chunks) * 3 * 64 * c.vec * sizeof(uint64_t);
+    pl.block_chunks = choose_block_chunks(pl.n_chunks, pl.n_groups);
+    if (pl.block_chunks < pl.n_chunks) {
+      pl.block_words_offset = pl.ws_bytes;
+      pl.ws_bytes += static_cast<size_t>(ceil_div(pl.n_chunks, pl.block_chunks) * pl.n_ctiles) * 2 * 64 * c.vec * sizeof(uint64_t);
+    }
+  }
   return FSS_OK;
 }
 

@@ -90,15 +90,19 @@ __device__ __forceinline__ void scan_tile(const ScanArgs &p, const StateArgs<STA
   RowT a[STEPS], b[STEPS];
   RowT hp[BWD ? STEPS : 1];
 
+  // How many steps of the slice lie inside the sequence, as a small wave-uniform integer (capped
+  // one above the slice), and whether the slice starts the scan: the guards of the ragged variant
+  // are then 32-bit scalar compares against constants (a 64-bit "r < seq" per row is a
+  // vector compare whose lane mask the compiler keeps for phase 3, one register pair per row).
+  const int valid = FULL ? STEPS + 1 : slice_steps_inside(seq, r0, STEPS + 1);
+  const bool at_start = r0 == 0;
+
   // scan-order index r -> row: forward t = r; backward t = seq-1-r, with alpha taken
-  // from row t+1 and the saved h from row t-1.  In memory the rows of a slice run upwards
-  // from row `low`; step s of the scan is row row_off(s) / row_bytes of them, whatever the tensor.
+  // from row t+1 and the saved h from row t-1
   const int64_t t_first = BWD ? seq - 1 - r0 : r0;
-  const int64_t low = BWD ? t_first - (STEPS - 1) : t_first;
-  const int32_t rb = static_cast<int32_t>(row_bytes);  // (the planner keeps a slice below 2^31 bytes)
-  auto row_off = [rb](int s) -> int32_t { return (BWD ? STEPS - 1 - s : s) * rb; };
-  const rows_t rows_a = make_rows(p.in_a + c.tile_base + (low + (BWD ? 1 : 0)) * row_bytes);
-  const rows_t rows_b = make_rows(p.in_b + c.tile_base + low * row_bytes);
+  gcptr_t pa = (gcptr_t)p.in_a + c.tile_base + (BWD ? t_first + 1 : t_first) * row_bytes;
+  gcptr_t pb = (gcptr_t)p.in_b + c.tile_base + t_first * row_bytes;
+  const int64_t step_bytes = BWD ? -row_bytes : row_bytes;  // one step in scan order
 
   FSS_STAMP(c, p, 0);
   // ---- phase 1a: issue every load of the slice -------------------------------------
@@ -108,25 +112,24 @@ __device__ __forceinline__ void scan_tile(const ScanArgs &p, const StateArgs<STA
       // The scan's very first step (r = 0) has no predecessor: its coefficient is replaced
       // below, whatever is loaded here.  The backward would find it one row past the end
       // of the sequence, so it loads the row before instead.
-      const int32_t off_a = (BWD && s == 0 && r0 == 0) ? row_off(s) - rb : row_off(s);
-      a[s].template load<(BWD ? kNtABwd : kNtAFwd)>(rows_a, lane_off, off_a);
-      b[s].template load<(BWD ? (kNtBBwd || ALT) : kNtBFwd)>(rows_b, lane_off, row_off(s));
+      const int row = (BWD && s == 0 && at_start) ? 1 : s;
+      a[s].template load<(BWD ? kNtABwd : kNtAFwd)>(uniform_ptr(pa + row * step_bytes) + lane_off);
+      b[s].template load<(BWD ? (kNtBBwd || ALT) : kNtBFwd)>(uniform_ptr(pb + s * step_bytes) + lane_off);
     } else {
-      const int64_t r = r0 + s;
       // Outside the sequence the step is the identity map (a=1, b=0).  The first step
       // of the plain scan has no predecessor (a=0), whatever alpha holds there; with a
       // state coming in, the forward applies alpha[0] to it and the backward adds it (a=1).
-      a[s].fill((r >= seq || (STATE && BWD && r == 0 && st.state_in)) ? 1.0f : 0.0f);
+      a[s].fill((s >= valid || (STATE && BWD && s == 0 && at_start && st.state_in)) ? 1.0f : 0.0f);
       b[s].fill(0.0f);
-      if (r < seq) {  // (wave-uniform; a lane without channels reads zeros through its offset)
-        if (r >= 1 || (STATE && !BWD && st.state_in))
-          a[s].template load<(BWD ? kNtABwd : kNtAFwd)>(rows_a, lane_off, row_off(s));
-        b[s].template load<(BWD ? (kNtBBwd || ALT) : kNtBFwd)>(rows_b, lane_off, row_off(s));
+      if (c.col_ok && s < valid) {
+        if (s >= 1 || !at_start || (STATE && !BWD && st.state_in))
+          a[s].template load<(BWD ? kNtABwd : kNtAFwd)>(uniform_ptr(pa + s * step_bytes) + lane_off);
+        b[s].template load<(BWD ? (kNtBBwd || ALT) : kNtBFwd)>(uniform_ptr(pb + s * step_bytes) + lane_off);
       }
     }
   }
 
-  if (FULL && r0 == 0) {
+  if (FULL && at_start) {
     // no predecessor: coefficient 0 - or, with a state coming in, alpha[0] as loaded
     // (forward) resp. 1, since the incoming gradient is added (backward)
     if (BWD)
@@ -140,14 +143,14 @@ __device__ __forceinline__ void scan_tile(const ScanArgs &p, const StateArgs<STA
   // the registers that the steps already done have released, which is what lets a
   // lane of the backward hold as many timesteps as one of the forward.
   constexpr int kHEarly = (BWD && STEPS * Row<E, VEC>::kDwords > 16) ? STEPS / 2 : STEPS;
-  const rows_t rows_h = make_rows(BWD ? p.in_h + c.tile_base + (low - 1) * row_bytes : p.in_a);
+  gcptr_t ph = BWD ? (gcptr_t)p.in_h + c.tile_base + (t_first - 1) * row_bytes : (gcptr_t) nullptr;
   auto load_h = [&](int s) {
     if (FULL) {
-      hp[s].template load<kNtH>(rows_h, lane_off, row_off(s));
+      hp[s].template load<kNtH>(uniform_ptr(ph + s * step_bytes) + lane_off);
     } else {
       hp[s].fill(0.0f);
-      if (r0 + s < seq - 1)  // t - 1 >= 0
-        hp[s].template load<kNtH>(rows_h, lane_off, row_off(s));
+      if (c.col_ok && s + 1 < valid)  // t - 1 >= 0
+        hp[s].template load<kNtH>(uniform_ptr(ph + s * step_bytes) + lane_off);
     }
   };
   auto load_h_early = [&] {
@@ -200,8 +203,8 @@ __device__ __forceinline__ void scan_tile(const ScanArgs &p, const StateArgs<STA
     keep_packed(b[s]);
     if (BWD && s < kHEarly) keep_packed(hp[s]);
   }
-  const rows_t rows_o0 = make_rows(p.out0 + c.tile_base + low * row_bytes);
-  const rows_t rows_o1 = make_rows(BWD ? p.out1 + c.tile_base + low * row_bytes : p.out0);
+  gptr_t po0 = (gptr_t)p.out0 + c.tile_base + t_first * row_bytes;
+  gptr_t po1 = BWD ? (gptr_t)p.out1 + c.tile_base + t_first * row_bytes : (gptr_t) nullptr;
 #pragma unroll
   for (int s = 0; s < STEPS; ++s) {
     float ga[VEC];
@@ -210,20 +213,19 @@ __device__ __forceinline__ void scan_tile(const ScanArgs &p, const StateArgs<STA
       state[v] = __builtin_fmaf(a[s].get(v), state[v], b[s].get(v));
       if (BWD) ga[v] = state[v] * hp[s].get(v);
     }
-    const int64_t r = r0 + s;
-    if (FULL || r < seq) {  // (a lane without channels stores nothing: its offset says so)
+    if (FULL || (c.col_ok && s < valid)) {
       RowT o;
       o.pack(state);
-      o.template store<(BWD ? kNtOutBwd : (kNtOutFwd && !ALT))>(rows_o0, lane_off, row_off(s));
+      o.template store<(BWD ? kNtOutBwd : (kNtOutFwd && !ALT))>(uniform_ptr(po0 + s * step_bytes) + lane_off);
       if (BWD) {
-        if (!FULL && r == seq - 1) {  // t = 0: grad_alpha[0] = g[0] * h[-1], 0 in the plain scan
+        if (!FULL && s + 1 == valid) {  // t = 0: grad_alpha[0] = g[0] * h[-1], 0 in the plain scan
 #pragma unroll
           for (int v = 0; v < VEC; ++v)
             ga[v] = (STATE && st.h_before) ? state[v] * st.h_before[c.chan_row + c.lane * VEC + v] : 0.0f;
         }
         RowT oa;
         oa.pack(ga);
-        oa.template store<kNtOutBwd>(rows_o1, lane_off, row_off(s));
+        oa.template store<kNtOutBwd>(uniform_ptr(po1 + s * step_bytes) + lane_off);
       }
     }
     if (BWD && s + kHEarly < STEPS) load_h(s + kHEarly);
@@ -231,10 +233,10 @@ __device__ __forceinline__ void scan_tile(const ScanArgs &p, const StateArgs<STA
   // The wave whose slice holds the last step of the scan hands out the final state: the
   // forward as it is (the steps past the end are identity maps), the backward times
   // alpha[0] (the gradient with respect to h[-1]).
-  if (STATE && st.state_out && c.col_ok && r0 <= seq - 1 && seq - 1 < r0 + STEPS) {
+  if (STATE && st.state_out && c.col_ok && r0 <= seq - 1 && seq - 1 < r0 + STEPS) {  // (once per tile)
     if (BWD) {
       RowT a0;
-      a0.template load<false>((gcptr_t)p.in_a + c.tile_base + (lane_off & ~kRowsLimit));
+      a0.template load<false>((gcptr_t)p.in_a + c.tile_base + lane_off);
 #pragma unroll
       for (int v = 0; v < VEC; ++v) st.state_out[c.chan_row + c.lane * VEC + v] = a0.get(v) * state[v];
     } else {
@@ -279,45 +281,43 @@ __device__ __forceinline__ void gated_tile(const ScanArgs &p, const StateArgs<ST
 
   RowT a[kARows], b[STEPS];
   RowT hp[BWD ? STEPS : 1], xs[BWD ? STEPS : 1];
+  // (steps of the slice inside the sequence, capped two above the slice; see scan_tile)
+  const int valid = FULL ? STEPS + 2 : slice_steps_inside(seq, r0, STEPS + 2);
+  const bool at_start = r0 == 0;
 
-  // forward: a[s] = gate row t = r0+s.  backward: a[s] = gate row t+1 = seq-(r0+s), s = 0..STEPS.
-  // In memory the rows of the slice run upwards from row `low` (the gate of the backward: one
-  // row more at the top); step s is row row_off(s, rows of the tensor) / row_bytes of them.
+  // forward: a[s] = gate row t = r0+s.  backward: a[s] = gate row t+1 = seq-(r0+s), s = 0..STEPS
   const int64_t t_first = BWD ? seq - 1 - r0 : r0;
-  const int64_t low = BWD ? t_first - (STEPS - 1) : t_first;
-  const int32_t rb = static_cast<int32_t>(row_bytes);  // (the planner keeps a slice below 2^31 bytes)
-  auto row_off = [rb](int s, int n_rows) -> int32_t { return (BWD ? n_rows - 1 - s : s) * rb; };
-  const rows_t rows_a = make_rows(p.in_a + c.tile_base + low * row_bytes);
-  const rows_t rows_b = make_rows(p.in_b + c.tile_base + low * row_bytes);
+  gcptr_t pa = (gcptr_t)p.in_a + c.tile_base + (BWD ? t_first + 1 : t_first) * row_bytes;
+  gcptr_t pb = (gcptr_t)p.in_b + c.tile_base + t_first * row_bytes;
+  const int64_t step_bytes = BWD ? -row_bytes : row_bytes;
 
   // ---- phase 1a: loads ---------------------------------------------------------------
 #pragma unroll
   for (int s = 0; s < kARows; ++s) {
-    const int64_t r = r0 + s;
-    // the gate row of a[s] exists: forward r < seq; backward 1 <= r <= seq
-    const bool a_ok = FULL || (BWD ? (r >= 1 && r <= seq) : (r < seq));  // (lanes without channels read zeros)
+    // the gate row of a[s] exists: forward r < seq; backward 1 <= r <= seq  (r = r0 + s)
+    const bool a_ok = FULL || (c.col_ok && (BWD ? ((s >= 1 || !at_start) && s <= valid) : (s < valid)));
     if (!FULL) a[s].fill(0.0f);
-    if (a_ok) a[s].template load<(BWD ? kNtABwd : kNtAFwd)>(rows_a, lane_off, row_off(s, kARows));
+    if (a_ok) a[s].template load<(BWD ? kNtABwd : kNtAFwd)>(uniform_ptr(pa + s * step_bytes) + lane_off);
     if (s < STEPS) {
       if (!FULL) b[s].fill(0.0f);
-      if (FULL || r < seq) b[s].template load<(BWD ? kNtBBwd : kNtBFwd)>(rows_b, lane_off, row_off(s, STEPS));
+      if (FULL || (c.col_ok && s < valid)) b[s].template load<(BWD ? kNtBBwd : kNtBFwd)>(uniform_ptr(pb + s * step_bytes) + lane_off);
     }
   }
   // x and the saved h only feed phase 3 of the backward: half of their rows now, the
   // rest during phase 3 into registers that finished steps have released
   constexpr int kEarly = BWD ? (STEPS >= 16 ? STEPS / 2 : STEPS) : 0;
-  const rows_t rows_h = make_rows(BWD ? p.in_h + c.tile_base + (low - 1) * row_bytes : p.in_a);
-  const rows_t rows_x = make_rows(BWD ? p.in_x + c.tile_base + low * row_bytes : p.in_a);
+  gcptr_t ph = BWD ? (gcptr_t)p.in_h + c.tile_base + (t_first - 1) * row_bytes : (gcptr_t) nullptr;
+  gcptr_t px = BWD ? (gcptr_t)p.in_x + c.tile_base + t_first * row_bytes : (gcptr_t) nullptr;
   auto load_hx = [&](int s) {
     if (FULL) {
-      hp[s].template load<kNtH>(rows_h, lane_off, row_off(s, STEPS));
-      xs[s].template load<kNtH>(rows_x, lane_off, row_off(s, STEPS));
+      hp[s].template load<kNtH>(uniform_ptr(ph + s * step_bytes) + lane_off);
+      xs[s].template load<kNtH>(uniform_ptr(px + s * step_bytes) + lane_off);
     } else {
       hp[s].fill(0.0f);
       xs[s].fill(0.0f);
-      if (r0 + s < seq - 1)  // t - 1 >= 0
-        hp[s].template load<kNtH>(rows_h, lane_off, row_off(s, STEPS));
-      if (r0 + s < seq) xs[s].template load<kNtH>(rows_x, lane_off, row_off(s, STEPS));
+      if (c.col_ok && s + 1 < valid)  // t - 1 >= 0
+        hp[s].template load<kNtH>(uniform_ptr(ph + s * step_bytes) + lane_off);
+      if (c.col_ok && s < valid) xs[s].template load<kNtH>(uniform_ptr(px + s * step_bytes) + lane_off);
     }
   };
   if (BWD) {
@@ -337,12 +337,11 @@ __device__ __forceinline__ void gated_tile(const ScanArgs &p, const StateArgs<ST
   }
 #pragma unroll
   for (int s = 0; s < kARows; ++s) {
-    const int64_t r = r0 + s;
     float al[VEC];
 #pragma unroll
     for (int v = 0; v < VEC; ++v) al[v] = sigmoid_f32(a[s].get(v));
     // (backward with a gradient coming in through the last state: it is added, coefficient 1)
-    if (!FULL && (r >= seq + (BWD ? 1 : 0) || !c.col_ok || (STATE && BWD && r == 0 && st.state_in))) {
+    if (!FULL && (s >= valid + (BWD ? 1 : 0) || !c.col_ok || (STATE && BWD && s == 0 && at_start && st.state_in))) {
 #pragma unroll
       for (int v = 0; v < VEC; ++v) al[v] = 1.0f;
     }
@@ -361,7 +360,7 @@ __device__ __forceinline__ void gated_tile(const ScanArgs &p, const StateArgs<ST
       // (for the latency of exp2/rcp/sqrt) and runs out of registers at 32 steps per lane
       keep_packed(a[s]);
       keep_packed(b[s]);
-      const bool ident = !FULL && BWD && r >= seq;  // backward: a[s] with r == seq is alpha[0], not a coefficient
+      const bool ident = !FULL && BWD && s >= valid;  // backward: a[s] with r == seq is alpha[0], not a coefficient
 #pragma unroll
       for (int v = 0; v < VEC; ++v) {
         const float av = ident ? 1.0f : a[s].get(v);
@@ -398,15 +397,14 @@ __device__ __forceinline__ void gated_tile(const ScanArgs &p, const StateArgs<ST
       keep_packed(xs[s]);
     }
   }
-  const rows_t rows_o0 = make_rows(p.out0 + c.tile_base + low * row_bytes);
-  const rows_t rows_o1 = make_rows(BWD ? p.out1 + c.tile_base + low * row_bytes : p.out0);
+  gptr_t po0 = (gptr_t)p.out0 + c.tile_base + t_first * row_bytes;
+  gptr_t po1 = BWD ? (gptr_t)p.out1 + c.tile_base + t_first * row_bytes : (gptr_t) nullptr;
 #pragma unroll
   for (int s = 0; s < STEPS; ++s) {
-    const int64_t r = r0 + s;
-    const bool ident = !FULL && BWD && r >= seq;
+    const bool ident = !FULL && BWD && s >= valid;
     float o0[VEC], o1[VEC];
     // t = 0 with a state coming in: h[-1] is that state, and alpha[0]*g[0] goes out
-    const bool t_zero = STATE && BWD && !FULL && r == seq - 1;
+    const bool t_zero = STATE && BWD && !FULL && s + 1 == valid;
 #pragma unroll
     for (int v = 0; v < VEC; ++v) {
       state[v] = __builtin_fmaf(ident ? 1.0f : a[s].get(v), state[v], b[s].get(v));
@@ -429,14 +427,14 @@ __device__ __forceinline__ void gated_tile(const ScanArgs &p, const StateArgs<ST
         o0[v] = state[v];
       }
     }
-    if (FULL || r < seq) {
+    if (FULL || (c.col_ok && s < valid)) {
       RowT o;
       o.pack(o0);
-      o.template store<(BWD ? kNtOutBwd : kNtOutFwd)>(rows_o0, lane_off, row_off(s, STEPS));
+      o.template store<(BWD ? kNtOutBwd : kNtOutFwd)>(uniform_ptr(po0 + s * step_bytes) + lane_off);
       if (BWD) {
         RowT oz;
         oz.pack(o1);
-        oz.template store<kNtOutBwd>(rows_o1, lane_off, row_off(s, STEPS));
+        oz.template store<kNtOutBwd>(uniform_ptr(po1 + s * step_bytes) + lane_off);
       }
     }
     if (BWD && s + kEarly < STEPS) load_hx(s + kEarly);
@@ -475,7 +473,7 @@ __global__ __launch_bounds__(MAXW * 64) void scan_kernel(const ScanArgs p, const
   c.wcol = COLS > 1 ? (wave_in_group & 1) : 0;
   c.wave = COLS > 1 ? (wave_in_group >> 1) : wave_in_group;
   c.look = p.look_waves;
-  c.span = look_span(p.n_chunks, p.n_groups, p.look_waves);
+  c.span = look_span(p.n_chunks, p.n_groups, p.look_waves, p.block_chunks);
   // LDS: two sets of per-wave maps (tiles alternate between them, so a wave that runs
   // ahead into the next tile cannot overwrite a map a slower wave still reads), then
   // the slots the look-back waves fill
@@ -519,7 +517,7 @@ __global__ __launch_bounds__(MAXW * 64) void scan_kernel(const ScanArgs p, const
 
     const int64_t col0 = static_cast<int64_t>(coltile) * kLaneSlots;  // first channel of the tile
     c.col_ok = col0 + c.lane * VEC < p.d;
-    c.lane_off = static_cast<uint32_t>(c.lane * Row<E, VEC>::kBytes) | (c.col_ok ? 0u : kRowsLimit);
+    c.lane_off = static_cast<uint32_t>(c.lane * Row<E, VEC>::kBytes);
     c.tile_base = (static_cast<int64_t>(batch) * c.seq * p.d + col0) * E::kBytes;
     c.chan_row = static_cast<int64_t>(batch) * p.d + col0;
     c.r0 = (static_cast<int64_t>(chunk) * c.n_waves + c.wave) * STEPS;
