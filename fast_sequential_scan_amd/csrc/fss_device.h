@@ -413,17 +413,13 @@ struct TileCtx {
 // that the grid works on at once (gridDim / n_groups of them, tiles being numbered chunk-major)
 // can still lack an outgoing state; whatever lies before them was finished in an earlier round
 // of the grid, so the first look there ends the walk.  One round of the look-back should reach
-// across those chunks (with blocks: across the rest of the tile's own block and the blocks in
-// flight before it); a chain it does not reach simply takes another round.
+// across those chunks (with blocks: across the rest of the tile's own block); a chain it does
+// not reach simply takes another round.
 __device__ __forceinline__ int look_span(int n_chunks, int n_groups, int look, int block_chunks) {
   const int in_flight = (static_cast<int>(gridDim.x) + n_groups - 1) / n_groups;
   int need = n_chunks - 1 < in_flight ? n_chunks - 1 : in_flight;
-  if (block_chunks < n_chunks) {
-    const int in_block = block_chunks - 1 < in_flight ? block_chunks - 1 : in_flight;
-    const int blocks = (n_chunks + block_chunks - 1) / block_chunks - 1;
-    const int blocks_in_flight = in_flight / block_chunks + 1;
-    need = in_block + (blocks < blocks_in_flight ? blocks : blocks_in_flight);
-  }
+  if (block_chunks < n_chunks)  // (blocks are asked one per wave and round)
+    need = block_chunks - 1 < in_flight ? block_chunks - 1 : in_flight;
   const int span = (need + look - 1) / look;
   return span < 1 ? 1 : (span > kMaxSpan ? kMaxSpan : span);
 }
@@ -621,28 +617,24 @@ __device__ __forceinline__ void chain_chunks(const ScanArgs &p, const TileCtx &c
   // The walk back.  Its places ("items"): the chunks before this one in its own block, nearest
   // first (n_in of them), then the earlier blocks, nearest first.  With one level the whole
   // sequence is one block.  Look-back wave w takes entry first_entry + w of the walk: `span`
-  // consecutive items that it asks one after the other (an entry never crosses from the chunks
-  // to the blocks, so that what the chunks of the own block do is known apart: the block's map
-  // is that composed with this chunk's map).
+  // consecutive chunks that it asks one after the other, or one block.
+  //
+  // A chunk answers as soon as it has its map, so a look at a chunk waits for the answer.  A
+  // block answers one look later (its last chunk must have seen the maps of the others), and
+  // that last chunk publishes the block's map behind its own look-back's barrier: a wave that
+  // waited for a block there would hold up its own workgroup's block map, and every block
+  // would wait for the one before.  So a block is asked once per round; the walk stops at the
+  // first entry without an answer and the next round starts there.
   const int block = c.chunk / p.block_chunks;
   const int n_in = c.chunk - block * p.block_chunks;
   const int span = c.span;
   const int entries_in = (n_in + span - 1) / span;
-  const int entries = entries_in + (block + span - 1) / span;
-  // this chunk closes its block and later blocks exist: it owes them the block's map
+  const int entries = entries_in + block;
+  // this chunk closes its block and later blocks exist: it owes them the block's map (the
+  // first block has none: its first chunk has no map, but a state at once)
   const bool owes_block_map = n_in == p.block_chunks - 1 && !c.last && block > 0;
   int first_entry = 0;  // first entry not folded yet
-  // (item range of an entry)
-  auto entry_items = [&](int e, int &first_item, int &count) {
-    if (e < entries_in) {
-      first_item = e * span;
-      count = n_in - first_item < span ? n_in - first_item : span;
-    } else {
-      const int f = (e - entries_in) * span;
-      first_item = n_in + f;
-      count = block - f < span ? block - f : span;
-    }
-  };
+  uint32_t block_polls = 0;  // looks at blocks by this wave, over all rounds (bounded like any wait)
   // The first look goes out ahead of the loop, with `mid` in a straight line between the
   // issue of its loads and their use: only so does the compiler wait for exactly those
   // loads and not for the ones `mid` has issued behind them.
@@ -650,15 +642,16 @@ __device__ __forceinline__ void chain_chunks(const ScanArgs &p, const TileCtx &c
   float q0A[VEC], q0B[VEC];
 #pragma unroll
   for (int v = 0; v < VEC; ++v) q0A[v] = q0B[v] = 0.0f;
+  bool looked = false;  // the first look has been taken (it counts as this round's look at a block)
   if constexpr (HAS_MID) {
     if (wave < c.look && wave < entries) {
-      int first_item, count;
-      entry_items(wave, first_item, count);
-      const LookItem it = look_item<VEC>(p, c, n_in, block, first_item);
+      const int item = wave < entries_in ? wave * span : n_in + (wave - entries_in);
+      const LookItem it = look_item<VEC>(p, c, n_in, block, item);
       ChunkWords<VEC> w;
       poll_issue<VEC>(it, w);
       mid();
       kind0 = poll_eval<VEC>(c, it, w, q0A, q0B);
+      looked = true;
     } else {
       mid();
     }
@@ -673,8 +666,9 @@ __device__ __forceinline__ void chain_chunks(const ScanArgs &p, const TileCtx &c
   for (;;) {
     const int e = first_entry + wave;
     if (!done && wave < c.look && e < entries) {
-      int first_item, count;
-      entry_items(e, first_item, count);
+      const bool chunks = e < entries_in;  // an entry of chunks (waited for) or one block (asked once per round)
+      const int first_item = chunks ? e * span : n_in + (e - entries_in);
+      const int count = chunks ? (n_in - first_item < span ? n_in - first_item : span) : 1;
       float qA[VEC], qB[VEC];
       uint32_t kind = kind0;  // what the first look found (nothing, in later rounds)
 #pragma unroll
@@ -694,9 +688,9 @@ __device__ __forceinline__ void chain_chunks(const ScanArgs &p, const TileCtx &c
           rA[v] = qA[v];
           rB[v] = qB[v];
         }
-        if (got == kPredNone) {
+        if (got == kPredNone && !(looked && !chunks && p.spin_limit != 0)) {
           const LookItem it = look_item<VEC>(p, c, n_in, block, first_item + k);
-          uint32_t polls = 0;
+          uint32_t polls = chunks ? 0u : block_polls;
           for (;;) {
             if (polls >= p.spin_limit) {
               // give up, so that the grid still drains: a NaN state poisons what follows
@@ -710,10 +704,11 @@ __device__ __forceinline__ void chain_chunks(const ScanArgs &p, const TileCtx &c
               break;
             }
             got = poll_item<VEC>(c, it, rA, rB);
-            if (got != kPredNone) break;
             ++polls;
+            if (got != kPredNone || !chunks) break;
             __builtin_amdgcn_s_sleep(2);
           }
+          if (!chunks) block_polls = polls;
         }
         if (k == 0) {
 #pragma unroll
@@ -735,13 +730,17 @@ __device__ __forceinline__ void chain_chunks(const ScanArgs &p, const TileCtx &c
       for (int v = 0; v < VEC; ++v) c.lds_pred[(wave * VEC + v) * 64 + lane] = make_float2(qA[v], qB[v]);
       if (lane == 0) c.s_kind[wave] = kind;
     }
+    looked = false;
     __syncthreads();
     // every wave folds what the look-back waves found (the same few LDS reads in each wave
     // cost less than a second barrier and a broadcast by wave 0)
     if (!done) {
       bool resolved = false;
-      for (int w = 0; w < c.look && first_entry + w < entries && !resolved; ++w) {
-        const bool is_state = c.s_kind[w] == kPredState;
+      int w = 0;
+      for (; w < c.look && first_entry + w < entries; ++w) {
+        const uint32_t kind = c.s_kind[w];
+        if (kind == kPredNone) break;  // a block without an answer yet: the next round starts here
+        const bool is_state = kind == kPredState;
 #pragma unroll
         for (int v = 0; v < VEC; ++v) {
           const float2 m = c.lds_pred[(w * VEC + v) * 64 + lane];
@@ -752,7 +751,6 @@ __device__ __forceinline__ void chain_chunks(const ScanArgs &p, const TileCtx &c
             accA[v] *= m.x;
           }
         }
-        resolved = is_state;
         // all chunks of the own block have answered with maps: the block's map is theirs
         // composed with this chunk's, and it goes out at once
         if (owes_block_map && wave == 0 && !is_state && first_entry + w == entries_in - 1) {
@@ -763,6 +761,10 @@ __device__ __forceinline__ void chain_chunks(const ScanArgs &p, const TileCtx &c
             st_word(blk + (1 * VEC + v) * 64, c.tag, fma0(cA[v], accB[v], cB[v]));
           }
         }
+        if (is_state) {
+          resolved = true;
+          break;
+        }
       }
       if (resolved) {  // chunk 0 always offers a state, so this is reached
         done = true;
@@ -772,7 +774,7 @@ __device__ __forceinline__ void chain_chunks(const ScanArgs &p, const TileCtx &c
             st_word(mine + (2 * VEC + v) * 64, c.tag, fma0(cA[v], hin[v], cB[v]));
         }
       } else {
-        first_entry += c.look;
+        first_entry += w;
         if (first_entry >= entries) {  // cannot happen; never spin on a logic error
           if (lane == 0 && wave == 0) report_timeout(p.hdr);
           done = true;
@@ -780,11 +782,18 @@ __device__ __forceinline__ void chain_chunks(const ScanArgs &p, const TileCtx &c
       }
     }
     if (!other_done) {
-      // (the other column is at the same chunk and in the same round, so the same slots count)
-      for (int w = 0; w < c.look && other_first_entry + w < entries && !other_done; ++w)
-        other_done = c.s_kind_other[w] == kPredState;
+      // (the other column is at the same chunk, so its walk has the same entries)
+      int w = 0;
+      for (; w < c.look && other_first_entry + w < entries; ++w) {
+        const uint32_t kind = c.s_kind_other[w];
+        if (kind == kPredNone) break;
+        if (kind == kPredState) {
+          other_done = true;
+          break;
+        }
+      }
       if (!other_done) {
-        other_first_entry += c.look;
+        other_first_entry += w;
         if (other_first_entry >= entries) other_done = true;  // as above: cannot happen
       }
     }

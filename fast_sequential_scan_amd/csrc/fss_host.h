@@ -203,18 +203,20 @@ struct Plan {
 
 // Chunks per block.  A look-back walks over the chunks before its own, as far as to the first
 // that has published its outgoing state; the chunks of a sequence that are in flight together
-// have none yet, so with c of them each walk reads up to c maps: c^2/2 in all.  Cut into
-// blocks of b chunks whose last chunk publishes the block's map, a walk reads at most b - 1
-// chunk maps and c/b block maps.  Worth its extra round trip (the block's map comes one look
-// after the chunks' maps) only where many chunks of a sequence are in flight: few columns,
-// long sequences.  0 from the debug knob means this choice.
+// have none yet.  One round of the look-back reaches kMaxLookWaves * kMaxSpan = 64 chunks; where
+// more chunks of a sequence are in flight (one or two column tiles in all, hundreds of
+// chunks) the walk takes several rounds, and cutting the sequence into blocks of 8 chunks whose
+// last chunk publishes the block's map pays for the extra look that map costs: bf16, forward +
+// backward, bs 1 seq 262144 d 64 100.6 -> 91.1 us, d 128 138.3 -> 131.5 us.  With 64 chunks in
+// flight or fewer it measured between 6 % faster and 7 % slower (bs 1 seq 65521 d 256: 70.5 ->
+// 70.9 us; seq 131072: 117.7 -> 125.9 us) and is left off.  0 from the debug knob means this choice.
 extern int g_block_chunks;  // fss_debug_set_block_chunks
 inline int64_t choose_block_chunks(int64_t n_chunks, int64_t n_groups) {
   const int forced = __atomic_load_n(&g_block_chunks, __ATOMIC_RELAXED);
   if (forced >= 2) return forced < n_chunks ? forced : n_chunks;
   const int64_t in_flight = ceil_div(kCus, n_groups);  // chunks of one column group the grid holds at once
-  if (n_chunks <= 24 || in_flight <= 12) return n_chunks;
-  return n_chunks <= 160 ? 8 : 16;
+  const int64_t reach = static_cast<int64_t>(kMaxLookWaves) * kMaxSpan;
+  return (n_chunks > reach && in_flight > reach) ? 8 : n_chunks;
 }
 
 inline int make_plan(Plan &pl, int64_t bs, int64_t seq, int64_t d, int dtype, int dir, size_t align,
