@@ -20,7 +20,7 @@ FSS_OK = 0
 FSS_CACHE_AUTO, FSS_CACHE_STREAMING = 0, 1
 FSS_ERR_CHAIN_TIMEOUT = 7
 FSS_ERR_TOO_LARGE = 9
-FSS_ABI_VERSION = 2
+FSS_ABI_VERSION = 3
 FSS_NOALLOC_SCRATCH_BYTES = 16 << 20
 
 EXPORTED_SYMBOLS = (
@@ -33,7 +33,6 @@ EXPORTED_SYMBOLS = (
     "fss_workspace_status",
     "fss_workspace_attach_flag",
     "fss_debug_set_spin_limit",
-    "fss_debug_set_block_chunks",
     "fss_scan_fwd_noalloc",
     "fss_choose_config",
     "fss_scan_fwd_bf16",
@@ -102,8 +101,6 @@ def _declare(lib: ctypes.CDLL) -> None:
     lib.fss_workspace_attach_flag.argtypes = [_vp, _vp, _vp]
     lib.fss_debug_set_spin_limit.restype = ctypes.c_uint32
     lib.fss_debug_set_spin_limit.argtypes = [ctypes.c_uint32]
-    lib.fss_debug_set_block_chunks.restype = _int
-    lib.fss_debug_set_block_chunks.argtypes = [_int]
     lib.fss_scan_fwd_noalloc.restype = _int
     lib.fss_scan_fwd_noalloc.argtypes = [_int, _vp, _vp, _vp, _i64, _i64, _i64, _vp]
     lib.fss_choose_config.restype = _int

@@ -29,7 +29,6 @@ __global__ void copy_kernel(const u32x4 *__restrict__ src, u32x4 *__restrict__ d
 }
 
 int g_cache_policy = FSS_CACHE_AUTO;  // fss_set_cache_policy
-int g_block_chunks = 0;               // fss_debug_set_block_chunks
 uint32_t g_spin_limit = kSpinLimit;    // fss_debug_set_spin_limit
 
 // ---- the chaining scratch of the entry point that allocates nothing ----------------------
@@ -134,10 +133,6 @@ int run_scan(int dtype, int dir, const void *alpha, const void *in_b, const void
   const StateArgs<true> state = {state_in, state_out, h_before};
   args.hdr = static_cast<uint32_t *>(workspace);
   args.words = workspace ? reinterpret_cast<uint64_t *>(static_cast<char *>(workspace) + kHeaderBytes) : nullptr;
-  args.block_chunks = static_cast<int32_t>(pl.block_chunks > 0 ? pl.block_chunks : 1);
-  args.block_words = pl.block_words_offset
-                         ? reinterpret_cast<uint64_t *>(static_cast<char *>(workspace) + pl.block_words_offset)
-                         : nullptr;
 #ifdef FSS_TRACE
   args.trace = g_trace;
 #endif
@@ -251,10 +246,6 @@ int fss_workspace_attach_flag(void *workspace, uint32_t *flag, void *stream) {
     return FSS_ERR_LAUNCH;
   }
   return FSS_OK;
-}
-
-int fss_debug_set_block_chunks(int chunks) {
-  return __atomic_exchange_n(&fss::g_block_chunks, chunks >= 2 ? chunks : 0, __ATOMIC_RELAXED);
 }
 
 uint32_t fss_debug_set_spin_limit(uint32_t polls) {

@@ -305,10 +305,8 @@ struct ScanArgs {
   int32_t wg_cols;        // adjacent column tiles a workgroup covers side by side (1 or 2)
   int32_t look_waves;     // waves per column tile that look back in parallel (1..kMaxLookWaves)
   uint32_t spin_limit;    // polls before a look-back gives up (kSpinLimit unless a test lowered it)
-  int32_t block_chunks;   // chunks per block of the two-level chain; n_chunks or more: one level
   uint32_t *hdr;          // workspace header
   uint64_t *words;        // tagged words
-  uint64_t *block_words;  // tagged words of the blocks' maps, [block][column tile][A, B][VEC][64]
   const char *in_x;       // gated backward only: the scan's input x (in_a is the gate there)
 #ifdef FSS_TRACE
   uint64_t *trace;        // debug build: 8 timestamps per tile, written by lane 0 of every wave 0
@@ -409,76 +407,41 @@ struct TileCtx {
 #endif
 };
 
-// Places one look-back wave covers, one after the other.  Only the chunks of a column group
+// Chunks one look-back wave covers, one after the other.  Only the chunks of a column group
 // that the grid works on at once (gridDim / n_groups of them, tiles being numbered chunk-major)
 // can still lack an outgoing state; whatever lies before them was finished in an earlier round
 // of the grid, so the first look there ends the walk.  One round of the look-back should reach
-// across those chunks (with blocks: across the rest of the tile's own block); a chain it does
-// not reach simply takes another round.
-__device__ __forceinline__ int look_span(int n_chunks, int n_groups, int look, int block_chunks) {
+// across those chunks; a chain it does not reach simply takes another round.
+__device__ __forceinline__ int look_span(int n_chunks, int n_groups, int look) {
   const int in_flight = (static_cast<int>(gridDim.x) + n_groups - 1) / n_groups;
-  int need = n_chunks - 1 < in_flight ? n_chunks - 1 : in_flight;
-  if (block_chunks < n_chunks)  // (blocks are asked one per wave and round)
-    need = block_chunks - 1 < in_flight ? block_chunks - 1 : in_flight;
+  const int need = n_chunks - 1 < in_flight ? n_chunks - 1 : in_flight;
   const int span = (need + look - 1) / look;
   return span < 1 ? 1 : (span > kMaxSpan ? kMaxSpan : span);
 }
 
-// What a look-back can learn from one place: the state leaving a chunk, if that chunk has
-// published it, else a map that leads to it from further back.  Two kinds of places exist:
-//   chunk j    its outgoing state, else (j > 0) its own map;
-//   block h    (chains of many chunks are cut into blocks of block_chunks chunks) the state
-//              leaving the block's last chunk, else the block's map: the composition of all its
-//              chunks' maps, published by its last chunk once it has seen the maps of the others.
-// Split in two so that other work can be placed between the loads and the use of what they return.
+// One look at what chunk `j` of this column tile offers: its outgoing state if it
+// has published one, else (j > 0) its map.  Split in two so that other work can be
+// placed between the loads and the use of what they return.
 template <int VEC>
 struct ChunkWords {
   uint64_t a[VEC], b[VEC], s[VEC];
 };
 
-// Where the words of look-back item `item` of this tile lie.  Items are numbered in the order
-// of the walk back: first the chunks of the tile's own block, nearest first, then the earlier
-// blocks, nearest first.
-struct LookItem {
-  const uint64_t *state;  // [VEC][64] words of the state
-  const uint64_t *map;    // [2][VEC][64] words of the map, A then B
-  bool map_ok;            // a map may be taken (chunk 0 of a sequence has none: its state is there at once)
-};
-
 template <int VEC>
-__device__ __forceinline__ LookItem look_item(const ScanArgs &p, const TileCtx &c, int n_in, int block, int item) {
-  constexpr size_t kLaneSlots = 64 * VEC;
-  LookItem it;
-  if (item < n_in) {
-    const int j = c.chunk - 1 - item;
-    const uint64_t *w = p.words + (static_cast<size_t>(j) * p.n_ctiles + c.ctile) * 3 * kLaneSlots + c.lane;
-    it.state = w + 2 * kLaneSlots;
-    it.map = w;
-    it.map_ok = j > 0;
-  } else {
-    const int h = block - 1 - (item - n_in);
-    const int j = h * p.block_chunks + p.block_chunks - 1;  // the block's last chunk
-    it.state = p.words + (static_cast<size_t>(j) * p.n_ctiles + c.ctile) * 3 * kLaneSlots + 2 * kLaneSlots + c.lane;
-    it.map = p.block_words + (static_cast<size_t>(h) * p.n_ctiles + c.ctile) * 2 * kLaneSlots + c.lane;
-    it.map_ok = true;
-  }
-  return it;
-}
-
-template <int VEC>
-__device__ __forceinline__ void poll_issue(const LookItem &it, ChunkWords<VEC> &w) {
+__device__ __forceinline__ void poll_issue(const ScanArgs &p, const TileCtx &c, int j, ChunkWords<VEC> &w) {
+  const uint64_t *theirs = p.words + (static_cast<size_t>(j) * p.n_ctiles + c.ctile) * 3 * (64 * VEC) + c.lane;
 #pragma unroll
   for (int v = 0; v < VEC; ++v) {
-    w.s[v] = ld_word(it.state + v * 64);
-    w.a[v] = ld_word(it.map + (0 * VEC + v) * 64);
-    w.b[v] = ld_word(it.map + (1 * VEC + v) * 64);
+    w.s[v] = ld_word(theirs + (2 * VEC + v) * 64);
+    w.a[v] = ld_word(theirs + (0 * VEC + v) * 64);
+    w.b[v] = ld_word(theirs + (1 * VEC + v) * 64);
   }
 }
 
 // The answer is taken for the whole wave, so that one word per wave can describe
 // it.  Returns kPredNone when neither a state nor a map is there yet.
 template <int VEC>
-__device__ __forceinline__ uint32_t poll_eval(const TileCtx &c, const LookItem &it, const ChunkWords<VEC> &w, float *qA,
+__device__ __forceinline__ uint32_t poll_eval(const TileCtx &c, int j, const ChunkWords<VEC> &w, float *qA,
                                               float *qB) {
   bool have_state = true, have_map = true;
 #pragma unroll
@@ -494,7 +457,7 @@ __device__ __forceinline__ uint32_t poll_eval(const TileCtx &c, const LookItem &
     }
     return kPredState;
   }
-  if (it.map_ok && __builtin_amdgcn_ballot_w64(have_map) == ~0ull) {
+  if (j > 0 && __builtin_amdgcn_ballot_w64(have_map) == ~0ull) {
 #pragma unroll
     for (int v = 0; v < VEC; ++v) {
       qA[v] = word_val(w.a[v]);
@@ -506,10 +469,11 @@ __device__ __forceinline__ uint32_t poll_eval(const TileCtx &c, const LookItem &
 }
 
 template <int VEC>
-__device__ __forceinline__ uint32_t poll_item(const TileCtx &c, const LookItem &it, float *qA, float *qB) {
+__device__ __forceinline__ uint32_t poll_chunk(const ScanArgs &p, const TileCtx &c, int j, float *qA,
+                                               float *qB) {
   ChunkWords<VEC> w;
-  poll_issue<VEC>(it, w);
-  return poll_eval<VEC>(c, it, w, qA, qB);
+  poll_issue<VEC>(p, c, j, w);
+  return poll_eval<VEC>(c, j, w, qA, qB);
 }
 
 // (A, B) <- map[count-1] o ... o map[0] for this lane's channels: the maps of the
@@ -614,27 +578,8 @@ __device__ __forceinline__ void chain_chunks(const ScanArgs &p, const TileCtx &c
     accA[v] = 1.0f;
     accB[v] = hin[v] = 0.0f;
   }
-  // The walk back.  Its places ("items"): the chunks before this one in its own block, nearest
-  // first (n_in of them), then the earlier blocks, nearest first.  With one level the whole
-  // sequence is one block.  Look-back wave w takes entry first_entry + w of the walk: `span`
-  // consecutive chunks that it asks one after the other, or one block.
-  //
-  // A chunk answers as soon as it has its map, so a look at a chunk waits for the answer.  A
-  // block answers one look later (its last chunk must have seen the maps of the others), and
-  // that last chunk publishes the block's map behind its own look-back's barrier: a wave that
-  // waited for a block there would hold up its own workgroup's block map, and every block
-  // would wait for the one before.  So a block is asked once per round; the walk stops at the
-  // first entry without an answer and the next round starts there.
-  const int block = c.chunk / p.block_chunks;
-  const int n_in = c.chunk - block * p.block_chunks;
-  const int span = c.span;
-  const int entries_in = (n_in + span - 1) / span;
-  const int entries = entries_in + block;
-  // this chunk closes its block and later blocks exist: it owes them the block's map (the
-  // first block has none: its first chunk has no map, but a state at once)
-  const bool owes_block_map = n_in == p.block_chunks - 1 && !c.last && block > 0;
-  int first_entry = 0;  // first entry not folded yet
-  uint32_t block_polls = 0;  // looks at blocks by this wave, over all rounds (bounded like any wait)
+  int nearest = c.chunk - 1;  // nearest earlier chunk not folded yet
+  int other_nearest = nearest;
   // The first look goes out ahead of the loop, with `mid` in a straight line between the
   // issue of its loads and their use: only so does the compiler wait for exactly those
   // loads and not for the ones `mid` has issued behind them.
@@ -642,16 +587,12 @@ __device__ __forceinline__ void chain_chunks(const ScanArgs &p, const TileCtx &c
   float q0A[VEC], q0B[VEC];
 #pragma unroll
   for (int v = 0; v < VEC; ++v) q0A[v] = q0B[v] = 0.0f;
-  bool looked = false;  // the first look has been taken (it counts as this round's look at a block)
   if constexpr (HAS_MID) {
-    if (wave < c.look && wave < entries) {
-      const int item = wave < entries_in ? wave * span : n_in + (wave - entries_in);
-      const LookItem it = look_item<VEC>(p, c, n_in, block, item);
+    if (wave < c.look && nearest - wave * c.span >= 0) {
       ChunkWords<VEC> w;
-      poll_issue<VEC>(it, w);
+      poll_issue<VEC>(p, c, nearest - wave * c.span, w);
       mid();
-      kind0 = poll_eval<VEC>(c, it, w, q0A, q0B);
-      looked = true;
+      kind0 = poll_eval<VEC>(c, nearest - wave * c.span, w, q0A, q0B);
     } else {
       mid();
     }
@@ -662,14 +603,11 @@ __device__ __forceinline__ void chain_chunks(const ScanArgs &p, const TileCtx &c
   // same barrier, so all waves of the workgroup see the same two answers and agree.
   bool done = false;
   bool other_done = p.wg_cols <= 1;  // (wg_cols is 1 wherever the kernel was compiled for one column)
-  int other_first_entry = 0;
   for (;;) {
-    const int e = first_entry + wave;
-    if (!done && wave < c.look && e < entries) {
-      const bool chunks = e < entries_in;  // an entry of chunks (waited for) or one block (asked once per round)
-      const int first_item = chunks ? e * span : n_in + (e - entries_in);
-      const int count = chunks ? (n_in - first_item < span ? n_in - first_item : span) : 1;
+    const int j = nearest - wave * c.span;
+    if (!done && wave < c.look && j >= 0) {
       float qA[VEC], qB[VEC];
+      uint32_t polls = 0;
       uint32_t kind = kind0;  // what the first look found (nothing, in later rounds)
 #pragma unroll
       for (int v = 0; v < VEC; ++v) {
@@ -678,69 +616,62 @@ __device__ __forceinline__ void chain_chunks(const ScanArgs &p, const TileCtx &c
       }
       kind0 = kPredNone;
       if (p.spin_limit == 0) kind = kPredNone;
-      // the entry's items one after the other, as long as they answer with maps (by the time
-      // the first has answered, the ones behind it nearly always have published too)
-      for (int k = 0; k < count && (k == 0 || kind == kPredMap); ++k) {
+      while (kind == kPredNone) {
+        if (polls >= p.spin_limit) {
+          // give up, so that the grid still drains: a NaN state poisons what follows
+          if (lane == 0) report_timeout(p.hdr);
+          kind = kPredState;
+#pragma unroll
+          for (int v = 0; v < VEC; ++v) {
+            qA[v] = 0.0f;
+            qB[v] = __builtin_nanf("");
+          }
+          break;
+        }
+        kind = poll_chunk<VEC>(p, c, j, qA, qB);
+        if (kind != kPredNone) break;
+        ++polls;
+        __builtin_amdgcn_s_sleep(2);
+      }
+      // long chains: the wave also takes the chunks before that one (by now they have nearly
+      // always published), so that one round of the look-back reaches `span` times as far
+      for (int k = 1; k < c.span && kind == kPredMap && j - k >= 0; ++k) {
         float rA[VEC], rB[VEC];
-        uint32_t got = k == 0 ? kind : kPredNone;
+        polls = 0;
+        for (;;) {
+          if (polls >= p.spin_limit) {
+            if (lane == 0) report_timeout(p.hdr);
+            kind = kPredState;
+#pragma unroll
+            for (int v = 0; v < VEC; ++v) {
+              rA[v] = 0.0f;
+              rB[v] = __builtin_nanf("");
+            }
+            break;
+          }
+          kind = poll_chunk<VEC>(p, c, j - k, rA, rB);
+          if (kind != kPredNone) break;
+          ++polls;
+          __builtin_amdgcn_s_sleep(2);
+        }
+        // (a state is the map x -> 0*x + value)
 #pragma unroll
         for (int v = 0; v < VEC; ++v) {
-          rA[v] = qA[v];
-          rB[v] = qB[v];
+          qB[v] = fma0(qA[v], rB[v], qB[v]);
+          qA[v] *= rA[v];
         }
-        if (got == kPredNone && !(looked && !chunks && p.spin_limit != 0)) {
-          const LookItem it = look_item<VEC>(p, c, n_in, block, first_item + k);
-          uint32_t polls = chunks ? 0u : block_polls;
-          for (;;) {
-            if (polls >= p.spin_limit) {
-              // give up, so that the grid still drains: a NaN state poisons what follows
-              if (lane == 0) report_timeout(p.hdr);
-              got = kPredState;
-#pragma unroll
-              for (int v = 0; v < VEC; ++v) {
-                rA[v] = 0.0f;
-                rB[v] = __builtin_nanf("");
-              }
-              break;
-            }
-            got = poll_item<VEC>(c, it, rA, rB);
-            ++polls;
-            if (got != kPredNone || !chunks) break;
-            __builtin_amdgcn_s_sleep(2);
-          }
-          if (!chunks) block_polls = polls;
-        }
-        if (k == 0) {
-#pragma unroll
-          for (int v = 0; v < VEC; ++v) {
-            qA[v] = rA[v];
-            qB[v] = rB[v];
-          }
-        } else {
-          // (a state is the map x -> 0*x + value)
-#pragma unroll
-          for (int v = 0; v < VEC; ++v) {
-            qB[v] = fma0(qA[v], rB[v], qB[v]);
-            qA[v] *= rA[v];
-          }
-        }
-        kind = got;
       }
 #pragma unroll
       for (int v = 0; v < VEC; ++v) c.lds_pred[(wave * VEC + v) * 64 + lane] = make_float2(qA[v], qB[v]);
       if (lane == 0) c.s_kind[wave] = kind;
     }
-    looked = false;
     __syncthreads();
     // every wave folds what the look-back waves found (the same few LDS reads in each wave
     // cost less than a second barrier and a broadcast by wave 0)
     if (!done) {
       bool resolved = false;
-      int w = 0;
-      for (; w < c.look && first_entry + w < entries; ++w) {
-        const uint32_t kind = c.s_kind[w];
-        if (kind == kPredNone) break;  // a block without an answer yet: the next round starts here
-        const bool is_state = kind == kPredState;
+      for (int w = 0; w < c.look && nearest - w * c.span >= 0 && !resolved; ++w) {
+        const bool is_state = c.s_kind[w] == kPredState;
 #pragma unroll
         for (int v = 0; v < VEC; ++v) {
           const float2 m = c.lds_pred[(w * VEC + v) * 64 + lane];
@@ -751,20 +682,7 @@ __device__ __forceinline__ void chain_chunks(const ScanArgs &p, const TileCtx &c
             accA[v] *= m.x;
           }
         }
-        // all chunks of the own block have answered with maps: the block's map is theirs
-        // composed with this chunk's, and it goes out at once
-        if (owes_block_map && wave == 0 && !is_state && first_entry + w == entries_in - 1) {
-          uint64_t *blk = p.block_words + (static_cast<size_t>(block) * p.n_ctiles + c.ctile) * 2 * kLaneSlots + lane;
-#pragma unroll
-          for (int v = 0; v < VEC; ++v) {
-            st_word(blk + (0 * VEC + v) * 64, c.tag, cA[v] * accA[v]);
-            st_word(blk + (1 * VEC + v) * 64, c.tag, fma0(cA[v], accB[v], cB[v]));
-          }
-        }
-        if (is_state) {
-          resolved = true;
-          break;
-        }
+        resolved = is_state;
       }
       if (resolved) {  // chunk 0 always offers a state, so this is reached
         done = true;
@@ -774,27 +692,20 @@ __device__ __forceinline__ void chain_chunks(const ScanArgs &p, const TileCtx &c
             st_word(mine + (2 * VEC + v) * 64, c.tag, fma0(cA[v], hin[v], cB[v]));
         }
       } else {
-        first_entry += w;
-        if (first_entry >= entries) {  // cannot happen; never spin on a logic error
+        nearest -= c.look * c.span;
+        if (nearest < 0) {  // cannot happen; never spin on a logic error
           if (lane == 0 && wave == 0) report_timeout(p.hdr);
           done = true;
         }
       }
     }
     if (!other_done) {
-      // (the other column is at the same chunk, so its walk has the same entries)
-      int w = 0;
-      for (; w < c.look && other_first_entry + w < entries; ++w) {
-        const uint32_t kind = c.s_kind_other[w];
-        if (kind == kPredNone) break;
-        if (kind == kPredState) {
-          other_done = true;
-          break;
-        }
-      }
+      // (the other column is at the same chunk and in the same round, so the same slots count)
+      for (int w = 0; w < c.look && other_nearest - w * c.span >= 0 && !other_done; ++w)
+        other_done = c.s_kind_other[w] == kPredState;
       if (!other_done) {
-        other_first_entry += w;
-        if (other_first_entry >= entries) other_done = true;  // as above: cannot happen
+        other_nearest -= c.look * c.span;
+        if (other_nearest < 0) other_done = true;  // as above: cannot happen
       }
     }
     if (done && other_done) break;

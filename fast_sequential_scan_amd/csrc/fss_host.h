@@ -196,28 +196,8 @@ struct Plan {
   int64_t tiles_per_row, n_ctiles, n_chunks;
   int64_t n_groups;  // column groups per chunk: n_ctiles / cfg.cols
   int64_t n_tiles;   // what the workgroups walk: n_groups * n_chunks
-  int64_t block_chunks;  // chunks per block of the two-level chain (n_chunks: one level)
-  size_t block_words_offset;  // where the blocks' words start in the workspace (0: none)
   size_t ws_bytes;
 };
-
-// Chunks per block.  A look-back walks over the chunks before its own, as far as to the first
-// that has published its outgoing state; the chunks of a sequence that are in flight together
-// have none yet.  One round of the look-back reaches kMaxLookWaves * kMaxSpan = 64 chunks; where
-// more chunks of a sequence are in flight (one or two column tiles in all, hundreds of
-// chunks) the walk takes several rounds, and cutting the sequence into blocks of 8 chunks whose
-// last chunk publishes the block's map pays for the extra look that map costs: bf16, forward +
-// backward, bs 1 seq 262144 d 64 100.6 -> 91.1 us, d 128 138.3 -> 131.5 us.  With 64 chunks in
-// flight or fewer it measured between 6 % faster and 7 % slower (bs 1 seq 65521 d 256: 70.5 ->
-// 70.9 us; seq 131072: 117.7 -> 125.9 us) and is left off.  0 from the debug knob means this choice.
-extern int g_block_chunks;  // fss_debug_set_block_chunks
-inline int64_t choose_block_chunks(int64_t n_chunks, int64_t n_groups) {
-  const int forced = __atomic_load_n(&g_block_chunks, __ATOMIC_RELAXED);
-  if (forced >= 2) return forced < n_chunks ? forced : n_chunks;
-  const int64_t in_flight = ceil_div(kCus, n_groups);  // chunks of one column group the grid holds at once
-  const int64_t reach = static_cast<int64_t>(kMaxLookWaves) * kMaxSpan;
-  return (n_chunks > reach && in_flight > reach) ? 8 : n_chunks;
-}
 
 inline int make_plan(Plan &pl, int64_t bs, int64_t seq, int64_t d, int dtype, int dir, size_t align,
               const fss_config *user) {
@@ -249,16 +229,8 @@ inline int make_plan(Plan &pl, int64_t bs, int64_t seq, int64_t d, int dtype, in
   pl.n_tiles = pl.n_groups * pl.n_chunks;
   if (pl.n_ctiles > INT32_MAX || pl.n_chunks > INT32_MAX || pl.n_ctiles * pl.n_chunks > INT32_MAX) return FSS_ERR_BAD_SHAPE;
   pl.ws_bytes = kHeaderBytes;
-  pl.block_chunks = pl.n_chunks;
-  pl.block_words_offset = 0;
-  if (pl.n_chunks > 1) {
+  if (pl.n_chunks > 1)
     pl.ws_bytes += static_cast<size_t>(pl.n_ctiles * pl.n_chunks) * 3 * 64 * c.vec * sizeof(uint64_t);
-    pl.block_chunks = choose_block_chunks(pl.n_chunks, pl.n_groups);
-    if (pl.block_chunks < pl.n_chunks) {
-      pl.block_words_offset = pl.ws_bytes;
-      pl.ws_bytes += static_cast<size_t>(ceil_div(pl.n_chunks, pl.block_chunks) * pl.n_ctiles) * 2 * 64 * c.vec * sizeof(uint64_t);
-    }
-  }
   return FSS_OK;
 }
 

@@ -204,7 +204,7 @@ __global__ __launch_bounds__(1024) void cm_scan_kernel(const ScanArgs p) {
   c.wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   c.n_waves = blockDim.x >> 6;
   c.look = p.look_waves;
-  c.span = look_span(p.n_chunks, p.n_groups, p.look_waves, p.block_chunks);
+  c.span = look_span(p.n_chunks, p.n_groups, p.look_waves);
   float2 *const lds_maps = reinterpret_cast<float2 *>(lds);  // laid out as in scan_kernel with one slot per lane
   c.lds_pred = lds_maps + 2 * c.n_waves * 64;
   c.s_kind = s_kind;
@@ -302,8 +302,6 @@ int run_cm_scan(int dtype, int dir, const void *alpha, const void *in_b, const v
   args.n_tiles = static_cast<int32_t>(pl.n_tiles);
   args.n_groups = static_cast<int32_t>(pl.n_rowtiles);
   args.wg_cols = 1;
-  args.block_chunks = args.n_chunks > 0 ? args.n_chunks : 1;  // one level
-  args.block_words = nullptr;
   args.look_waves = look_waves(pl.waves, 1);
   args.spin_limit = __atomic_load_n(&g_spin_limit, __ATOMIC_RELAXED);
   args.hdr = static_cast<uint32_t *>(workspace);

@@ -473,7 +473,7 @@ __global__ __launch_bounds__(MAXW * 64) void scan_kernel(const ScanArgs p, const
   c.wcol = COLS > 1 ? (wave_in_group & 1) : 0;
   c.wave = COLS > 1 ? (wave_in_group >> 1) : wave_in_group;
   c.look = p.look_waves;
-  c.span = look_span(p.n_chunks, p.n_groups, p.look_waves, p.block_chunks);
+  c.span = look_span(p.n_chunks, p.n_groups, p.look_waves);
   // LDS: two sets of per-wave maps (tiles alternate between them, so a wave that runs
   // ahead into the next tile cannot overwrite a map a slower wave still reads), then
   // the slots the look-back waves fill

@@ -64,7 +64,7 @@
 extern "C" {
 #endif
 
-#define FSS_ABI_VERSION 2
+#define FSS_ABI_VERSION 3
 
 typedef enum fss_status {
   FSS_OK = 0,
@@ -149,17 +149,6 @@ int fss_workspace_attach_flag(void *workspace, uint32_t *flag, void *stream);
  * Process-wide; returns the previous value.
  */
 uint32_t fss_debug_set_spin_limit(uint32_t polls);
-/*
- * Test hook: chunks per block of the two-level chain of the row-major kernels.  Sequences of
- * many chunks with few column tiles (hundreds of chunks of one sequence in flight at once) are
- * cut into blocks whose last chunk publishes the composition of the block's maps, so that a
- * look-back reads a few chunk maps and a few block maps instead of every map back to the last
- * published state.  0 (default): the library decides by shape; >= 2: that many chunks per block
- * wherever a sequence has more chunks than that.  Changes the workspace a shape needs
- * (fss_workspace_bytes follows).  Process-wide; returns the previous value.  No counterpart in
- * the reference.
- */
-int fss_debug_set_block_chunks(int chunks);
 
 /* The configuration the library would choose for this shape (for reporting). */
 int fss_choose_config(int64_t bs, int64_t seq, int64_t d, int dtype, int dir,

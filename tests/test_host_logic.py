@@ -31,18 +31,12 @@ def test_library_exports_every_declared_symbol():
 def plan_bytes(lib, bs, seq, d, dtype, direction, align):
     """Workspace bytes of the launch the library plans for tensors of this common alignment,
     recomputed from the configuration it reports (4 KiB header + 3 tagged 64-bit words per
-    channel slot and tile when the sequence is chained; where more chunks of a sequence are in
-    flight at once than one look-back round reaches - more than 64 chunks, more than 64 of them
-    resident together on 256 CUs - 2 more words per channel slot for every block of 8 chunks)."""
+    channel slot and tile when the sequence is chained)."""
     cfg = _native.FssConfig()
     assert lib.fss_choose_config(bs, seq, d, dtype, direction, align, ctypes.byref(cfg)) == 0
     chunks = -(-seq // (cfg.steps * (cfg.waves // cfg.cols)))
-    ctiles = bs * -(-d // (64 * cfg.vec))
-    tiles = ctiles * chunks
-    need = 4096 + (tiles * 3 * 64 * cfg.vec * 8 if chunks > 1 else 0)
-    if chunks > 64 and -(-256 // (ctiles // cfg.cols)) > 64:
-        need += -(-chunks // 8) * ctiles * 2 * 64 * cfg.vec * 8
-    return need, cfg
+    tiles = bs * -(-d // (64 * cfg.vec)) * chunks
+    return 4096 + (tiles * 3 * 64 * cfg.vec * 8 if chunks > 1 else 0), cfg
 
 
 def test_workspace_sizing_and_config_choice():

@@ -195,35 +195,6 @@ def test_two_column_tiles_f32_and_refusals(oracle):
     torch.cuda.synchronize()
 
 
-@pytest.mark.parametrize("block", [2, 3, 8, 16])
-def test_two_level_chain(oracle, block):
-    """Long chains cut into blocks of `block` chunks whose last chunk publishes the block's map:
-    single waves (98 chunks per sequence), small workgroups, two column tiles per workgroup, capped
-    grids (several rounds of the grid) and full ones (every chunk of a sequence in flight at once)."""
-    lib = _native.lib()
-    alpha, beta, dout = make_inputs("hawk", 2, 777, 256, seed=29)
-    previous = lib.fss_debug_set_block_chunks(block)
-    ext._need_cache.clear()
-    try:
-        for config in [(1, 8, 1), (2, 8, 2), (2, 16, 3, 5), (2, 16, 4, 0, 2), (1, 8, 2, 3), (4, 8, 1)]:
-            check_bf16(oracle, alpha, beta, dout, config=config, what=f"block {block} {config}")
-        ext.workspace_status()
-        # fp32 and a single long sequence (every look-back crosses many blocks)
-        a32, b32, d32 = make_inputs("sigmoid", 1, 3001, 64, dtype=torch.float32, seed=31)
-        a, b, do = a32.to(DEV), b32.to(DEV), d32.to(DEV)
-        h = ext._forward(torch.float32, a, b, (1, 8, 2))
-        ga, gb = ext._backward(torch.float32, a, h, do, (1, 8, 2))
-        ext.workspace_status()
-        h_or = oracle.scan_fwd_f32(a32.numpy(), b32.numpy(), fused=True)
-        ga_or, gb_or = oracle.scan_bwd_f32(a32.numpy(), h.cpu().numpy(), d32.numpy(), fused=True)
-        np.testing.assert_allclose(h.cpu().numpy(), h_or, rtol=1e-4, atol=1e-5)
-        np.testing.assert_allclose(gb.cpu().numpy(), gb_or, rtol=1e-4, atol=1e-5)
-        np.testing.assert_allclose(ga.cpu().numpy(), ga_or, rtol=1e-4, atol=1e-5)
-    finally:
-        lib.fss_debug_set_block_chunks(previous)
-        ext._need_cache.clear()
-
-
 @pytest.mark.parametrize("groups", [1, 3, 7, 64])
 @pytest.mark.parametrize("config", [(1, 8, 1), (2, 8, 3), (2, 16, 8), (2, 32, 2), (4, 8, 6)],
                          ids=lambda c: "v%d_s%d_w%d" % c)
