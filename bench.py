@@ -66,6 +66,9 @@ def parse_args():
                          "tensors, as the reference's benchmark does, so part of them sits in the 256 MB "
                          "memory-side cache; 8: 3.2 GB in rotation at the headline shape, nothing reused)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline / parity leg")
+    ap.add_argument("--no-autograd", action="store_true",
+                    help="skip the timing of the public autograd path (profiler runs: its launches would be "
+                         "averaged into the kernels' statistics)")
     ap.add_argument("--cpu-seconds", type=float, default=12.0, help="budget of the CPU baseline leg")
     ap.add_argument("--flush-mb", type=int, default=1024, help="size of the cache-flush read for the cold timings")
     ap.add_argument("--cache-policy", default="auto", choices=("auto", "streaming"),
@@ -448,23 +451,25 @@ def main() -> int:
         del junk
 
     # ---- the public autograd path (allocates its outputs, goes through torch.autograd) ----
-    a_req = alpha.detach().clone().requires_grad_(True)
-    b_req = beta.detach().clone().requires_grad_(True)
-    # (the allocator and the autograd engine take a few dozen steps to settle: with ten timed steps
-    # after five the figure read 25 % above what the same loop reaches from step 50 on)
-    for _ in range(50):
-        scan_fn(a_req, b_req).backward(dout)
-        a_req.grad = b_req.grad = None
-    torch.cuda.synchronize()
-    n_auto = max(200, K)
-    t0 = time.perf_counter()
-    for _ in range(n_auto):
-        scan_fn(a_req, b_req).backward(dout)
-        a_req.grad = b_req.grad = None
-    t_enqueued = time.perf_counter()
-    torch.cuda.synchronize()
-    autograd_ms = (time.perf_counter() - t0) * 1e3 / n_auto
-    autograd_cpu_ms = (t_enqueued - t0) * 1e3 / n_auto  # host time to issue a step; the GPU may lag behind it
+    autograd_ms = autograd_cpu_ms = None
+    if not args.no_autograd:
+        a_req = alpha.detach().clone().requires_grad_(True)
+        b_req = beta.detach().clone().requires_grad_(True)
+        # (the allocator and the autograd engine take a few dozen steps to settle: with ten timed steps
+        # after five the figure read 25 % above what the same loop reaches from step 50 on)
+        for _ in range(50):
+            scan_fn(a_req, b_req).backward(dout)
+            a_req.grad = b_req.grad = None
+        torch.cuda.synchronize()
+        n_auto = max(200, K)
+        t0 = time.perf_counter()
+        for _ in range(n_auto):
+            scan_fn(a_req, b_req).backward(dout)
+            a_req.grad = b_req.grad = None
+        t_enqueued = time.perf_counter()
+        torch.cuda.synchronize()
+        autograd_ms = (time.perf_counter() - t0) * 1e3 / n_auto
+        autograd_cpu_ms = (t_enqueued - t0) * 1e3 / n_auto  # host time to issue a step; the GPU may lag behind it
 
     # ---- CPU baseline + parity of this very run ----
     cpu = None
@@ -622,8 +627,8 @@ def main() -> int:
         },
         "cold_cache": cold,
         "rotating_sets": rotating,
-        "autograd_path_ms_per_step": round(autograd_ms, 5),
-        "autograd_path_host_ms_per_step": round(autograd_cpu_ms, 5),
+        "autograd_path_ms_per_step": None if autograd_ms is None else round(autograd_ms, 5),
+        "autograd_path_host_ms_per_step": None if autograd_cpu_ms is None else round(autograd_cpu_ms, 5),
         "parity": parity,
         "cpu_baseline": cpu,
     }

@@ -235,7 +235,8 @@ def _forward(dtype: torch.dtype, alpha: torch.Tensor, beta: torch.Tensor, config
 
 
 def _backward(
-    dtype: torch.dtype, alpha_saved: torch.Tensor, h_saved: torch.Tensor, grad_out: torch.Tensor, config=None
+    dtype: torch.dtype, alpha_saved: torch.Tensor, h_saved: torch.Tensor, grad_out: torch.Tensor, config=None,
+    overwrite_grad_out: bool = False,
 ) -> List[torch.Tensor]:
     if _same_kind(dtype, alpha_saved, h_saved, grad_out):
         bs, seq, d = alpha_saved.shape
@@ -243,7 +244,9 @@ def _backward(
         bs, seq, d = _validate(dtype, alpha_saved=alpha_saved, h_saved=h_saved, grad_out=grad_out)
     alpha_saved, h_saved, grad_out = _contiguous(alpha_saved), _contiguous(h_saved), _contiguous(grad_out)
     grad_alpha = torch.empty_like(alpha_saved)
-    grad_beta = torch.empty_like(alpha_saved)
+    # grad_beta over grad_out itself is the one overlap the kernels allow (every lane reads its rows
+    # of dout before it stores them): one allocation per backward, as in the reference
+    grad_beta = grad_out if overwrite_grad_out else torch.empty_like(alpha_saved)
     if grad_alpha.numel() == 0:
         return [grad_alpha, grad_beta]
     code = _DTYPE_CODE[dtype]
@@ -265,9 +268,12 @@ def scan_forward(alpha: torch.Tensor, beta: torch.Tensor) -> torch.Tensor:
     return _forward(torch.float32, alpha, beta)
 
 
-def scan_backward(alpha_saved: torch.Tensor, h_saved: torch.Tensor, grad_out: torch.Tensor) -> List[torch.Tensor]:
-    """fp32 backward -> [grad_alpha, grad_beta]: csrc/sequential_scan.cpp:17 / sequential_scan_kernel.cu:60-124."""
-    return _backward(torch.float32, alpha_saved, h_saved, grad_out)
+def scan_backward(alpha_saved: torch.Tensor, h_saved: torch.Tensor, grad_out: torch.Tensor,
+                  overwrite_grad_out: bool = False) -> List[torch.Tensor]:
+    """fp32 backward -> [grad_alpha, grad_beta]: csrc/sequential_scan.cpp:17 / sequential_scan_kernel.cu:60-124.
+    ``overwrite_grad_out=True`` writes grad_beta over a contiguous ``grad_out`` (not for use inside
+    autograd, which owns the gradients it hands to a backward)."""
+    return _backward(torch.float32, alpha_saved, h_saved, grad_out, overwrite_grad_out=overwrite_grad_out)
 
 
 def scan_forward_half(alpha: torch.Tensor, beta: torch.Tensor) -> torch.Tensor:
@@ -275,9 +281,13 @@ def scan_forward_half(alpha: torch.Tensor, beta: torch.Tensor) -> torch.Tensor:
     return _forward(torch.bfloat16, alpha, beta)
 
 
-def scan_backward_half(alpha_saved: torch.Tensor, h_saved: torch.Tensor, grad_out: torch.Tensor) -> List[torch.Tensor]:
-    """bf16 backward -> [grad_alpha, grad_beta]: csrc/sequential_scan.cpp:21 / sequential_scan_kernel.cu:189-268."""
-    return _backward(torch.bfloat16, alpha_saved, h_saved, grad_out)
+def scan_backward_half(alpha_saved: torch.Tensor, h_saved: torch.Tensor, grad_out: torch.Tensor,
+                       overwrite_grad_out: bool = False) -> List[torch.Tensor]:
+    """bf16 backward -> [grad_alpha, grad_beta]: csrc/sequential_scan.cpp:21 / sequential_scan_kernel.cu:189-268.
+    The reference returns ``h_saved`` overwritten with grad_beta (sequential_scan_kernel.cu:197), i.e. it
+    allocates one tensor; ``overwrite_grad_out=True`` gets the same footprint here by writing grad_beta
+    over a contiguous ``grad_out`` (not for use inside autograd, which owns the gradients it hands out)."""
+    return _backward(torch.bfloat16, alpha_saved, h_saved, grad_out, overwrite_grad_out=overwrite_grad_out)
 
 
 def scan_forward_fp16(alpha: torch.Tensor, beta: torch.Tensor) -> torch.Tensor:

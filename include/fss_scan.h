@@ -167,11 +167,16 @@ int fss_scan_fwd_bf16(const void *alpha, const void *beta, void *h, int64_t bs,
  * bf16 backward.  Replaces scan_backward_half
  * (csrc/sequential_scan.cpp:21, csrc/sequential_scan_kernel.cu:189-268, kernel
  * csrc/include/sequential_scan_kernel_bf16.cuh:169-390).  `h` is the stored
- * forward output.  The five tensors must not overlap: the reference writes
- * grad_beta over `h` (csrc/sequential_scan_kernel.cu:197), which is only safe
- * when one thread walks a channel's whole sequence in order; here neighbouring
- * chunks of a sequence run concurrently and each reads the last row of `h`
- * before its own chunk.
+ * forward output.  The tensors must not overlap, with one exception: grad_beta may
+ * be dout itself (the same address: the gradient is then computed in place, and the
+ * backward allocates one tensor, as the reference's does) - every lane has read the
+ * rows of dout it owns before it stores one of them, and no other lane touches them.
+ * The reference writes grad_beta over `h` instead (csrc/sequential_scan_kernel.cu:197),
+ * which is only safe when one thread walks a channel's whole sequence in order; here
+ * neighbouring chunks of a sequence run concurrently and each reads the last row of
+ * `h` before its own chunk, so grad_beta over `h` (or any partial overlap) stays
+ * forbidden.  The same holds for fss_scan_bwd_f32, fss_scan_bwd_ex and
+ * fss_scan_bwd_state (row-major layout only).
  */
 int fss_scan_bwd_bf16(const void *alpha, const void *h, const void *dout,
                       void *grad_alpha, void *grad_beta, int64_t bs, int64_t seq,

@@ -195,6 +195,30 @@ def test_two_column_tiles_f32_and_refusals(oracle):
     torch.cuda.synchronize()
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32], ids=["bf16", "f32"])
+def test_grad_beta_in_place_over_dout(dtype):
+    """grad_beta written over dout itself - the one overlap the kernels allow, which gives the
+    backward the reference's footprint of one allocation (it aliases grad_beta onto the saved h,
+    csrc/sequential_scan_kernel.cu:197): bit-identical to the out-of-place result, for chained,
+    ragged and capped launches and for two column tiles per workgroup."""
+    narrow = dtype != torch.float32
+    for shape, config in [((2, 777, 328), None), ((3, 1000, 256), (2 if narrow else 1, 16, 4)), ((2, 515, 204), (1, 8, 2, 3)),
+                          ((1, 2049, 512), (2 if narrow else 1, 16, 8, 0, 2)), ((8, 4096, 1024), None), ((2, 5, 7), None)]:
+        alpha, beta, dout = make_inputs("hawk", *shape, dtype=dtype, seed=41)
+        a, b, do = alpha.to(DEV), beta.to(DEV), dout.to(DEV)
+        h = ext._forward(dtype, a, b)
+        ga_ref, gb_ref = ext._backward(dtype, a, h, do, config)
+        work = do.clone()
+        ga, gb = ext._backward(dtype, a, h, work, config, overwrite_grad_out=True)
+        ext.workspace_status()
+        assert gb.data_ptr() == work.data_ptr()
+        assert torch.equal(gb, gb_ref) and torch.equal(ga, ga_ref), (shape, config)
+    # the public callee of the reference's name takes the option too
+    ga, gb = ext.scan_backward_half(a.bfloat16(), h.bfloat16(), do.bfloat16().clone(), overwrite_grad_out=True) if not narrow else \
+        ext.scan_backward_half(a, h, do.clone(), overwrite_grad_out=True)
+    assert ga.shape == gb.shape == a.shape
+
+
 @pytest.mark.parametrize("groups", [1, 3, 7, 64])
 @pytest.mark.parametrize("config", [(1, 8, 1), (2, 8, 3), (2, 16, 8), (2, 32, 2), (4, 8, 6)],
                          ids=lambda c: "v%d_s%d_w%d" % c)
