@@ -98,8 +98,10 @@ int run_scan(int dtype, int dir, const void *alpha, const void *in_b, const void
   if ((reinterpret_cast<uintptr_t>(state_in) | reinterpret_cast<uintptr_t>(state_out) |
        reinterpret_cast<uintptr_t>(h_before)) % 4 != 0)
     return FSS_ERR_MISALIGNED;
+  const bool streaming = __atomic_load_n(&g_cache_policy, __ATOMIC_RELAXED) == FSS_CACHE_STREAMING;
+  const bool with_state = state_in || state_out || h_before;
   Plan pl;
-  int rc = make_plan(pl, bs, seq, d, dtype, plan_dir, align, cfg);
+  int rc = make_plan(pl, bs, seq, d, dtype, plan_dir, align, cfg, streaming && !with_state);
   if (rc != FSS_OK) return rc;
   if (pl.n_chunks > 1) {
     if (!workspace || workspace_bytes < pl.ws_bytes) return FSS_ERR_WORKSPACE_SMALL;
@@ -126,7 +128,7 @@ int run_scan(int dtype, int dir, const void *alpha, const void *in_b, const void
   args.look_waves = look_waves(pl.cfg.waves, pl.cfg.vec, pl.cfg.cols);
   args.spin_limit = __atomic_load_n(&g_spin_limit, __ATOMIC_RELAXED);
   const int64_t tensor_bytes = bs * seq * d * static_cast<int64_t>(esize);
-  if (__atomic_load_n(&g_cache_policy, __ATOMIC_RELAXED) == FSS_CACHE_STREAMING)
+  if (streaming)
     pl.alt_policy = !gated && dir == FSS_BWD;
   else
     pl.alt_policy = !gated && (dir == FSS_FWD ? tensor_bytes <= kKeepOutBytes : tensor_bytes > kStreamDoutBytes);
@@ -137,7 +139,7 @@ int run_scan(int dtype, int dir, const void *alpha, const void *in_b, const void
   args.trace = g_trace;
 #endif
   hipStream_t s = static_cast<hipStream_t>(stream);
-  const bool st = state_in || state_out || h_before;
+  const bool st = with_state;
   const bool bwd = dir == FSS_BWD;
   const ScanOrderGuard ordered(s);
   if (dtype == FSS_BF16)
@@ -188,11 +190,15 @@ size_t fss_workspace_bytes(int64_t bs, int64_t seq, int64_t d, int dtype, int di
   // The tensors' alignment is unknown here and changes the plan (less aligned tensors take
   // fewer channels per lane, which can mean more, smaller tiles and more chaining words):
   // the answer covers every alignment.
+  // ... and either cache policy (the streaming one may take two column tiles per workgroup, whose
+  // chunks are half as long)
   size_t best = fss::kHeaderBytes;
-  for (size_t align = 2; align <= 16; align <<= 1) {
-    fss::Plan pl;
-    if (fss::make_plan(pl, bs, seq, d, dtype, dir, align, cfg) == FSS_OK && pl.ws_bytes > best) best = pl.ws_bytes;
-  }
+  for (size_t align = 2; align <= 16; align <<= 1)
+    for (int two = 0; two < 2; ++two) {
+      fss::Plan pl;
+      if (fss::make_plan(pl, bs, seq, d, dtype, dir, align, cfg, two != 0) == FSS_OK && pl.ws_bytes > best)
+        best = pl.ws_bytes;
+    }
   return best;
 }
 
@@ -200,11 +206,12 @@ size_t fss_workspace_bytes_max(int64_t bs, int64_t seq, int64_t d) {
   size_t best = fss::kHeaderBytes;
   for (int dtype = FSS_BF16; dtype <= FSS_F16; ++dtype)
     for (int dir = FSS_FWD; dir <= FSS_GATED_BWD; ++dir)
-      for (size_t align = 2; align <= 16; align <<= 1) {
-        fss::Plan pl;
-        if (fss::make_plan(pl, bs, seq, d, dtype, dir, align, nullptr) == FSS_OK && pl.ws_bytes > best)
-          best = pl.ws_bytes;
-      }
+      for (size_t align = 2; align <= 16; align <<= 1)
+        for (int two = 0; two < 2; ++two) {
+          fss::Plan pl;
+          if (fss::make_plan(pl, bs, seq, d, dtype, dir, align, nullptr, two != 0) == FSS_OK && pl.ws_bytes > best)
+            best = pl.ws_bytes;
+        }
   return best;
 }
 
@@ -212,7 +219,8 @@ int fss_choose_config(int64_t bs, int64_t seq, int64_t d, int dtype, int dir, si
                       fss_config *out) {
   if (!out) return FSS_ERR_NULL_POINTER;
   fss::Plan pl;
-  const int rc = fss::make_plan(pl, bs, seq, d, dtype, dir, align_bytes ? align_bytes : 16, nullptr);
+  const bool streaming = __atomic_load_n(&fss::g_cache_policy, __ATOMIC_RELAXED) == FSS_CACHE_STREAMING;
+  const int rc = fss::make_plan(pl, bs, seq, d, dtype, dir, align_bytes ? align_bytes : 16, nullptr, streaming);
   if (rc == FSS_OK) *out = pl.cfg;
   return rc;
 }

@@ -51,9 +51,28 @@ def test_workspace_sizing_and_config_choice():
                 need = lib.fss_workspace_bytes(bs, seq, d, dtype, direction, None)
                 assert need >= 4096 and need % 256 == 0
                 assert need <= lib.fss_workspace_bytes_max(bs, seq, d)
-                # the answer covers every alignment the tensors may have
-                per_align = [plan_bytes(lib, bs, seq, d, dtype, direction, a)[0] for a in (2, 4, 8, 16) if a >= esize]
-                assert need == max(per_align)
+                # the answer covers every alignment the tensors may have and either cache policy (under
+                # the streaming one a forward of at most two tiles per CU takes two column tiles per
+                # workgroup, whose chunks are half as long)
+                per_plan = []
+                for policy in (_native.FSS_CACHE_AUTO, _native.FSS_CACHE_STREAMING):
+                    previous = lib.fss_set_cache_policy(policy)
+                    try:
+                        per_plan += [plan_bytes(lib, bs, seq, d, dtype, direction, a)[0] for a in (2, 4, 8, 16) if a >= esize]
+                    finally:
+                        lib.fss_set_cache_policy(previous)
+                assert need == max(per_plan)
+    # the forward at the headline shape (512 tiles: two per CU): two column tiles per workgroup under the
+    # streaming policy, one otherwise; never in the backward
+    for policy, cols in ((_native.FSS_CACHE_STREAMING, 2), (_native.FSS_CACHE_AUTO, 1)):
+        previous = lib.fss_set_cache_policy(policy)
+        try:
+            assert lib.fss_choose_config(8, 4096, 1024, 0, 0, 16, ctypes.byref(cfg)) == 0
+            assert (cfg.vec, cfg.steps, cfg.waves, cfg.cols) == (2, 32, 16, cols)
+            assert lib.fss_choose_config(8, 4096, 1024, 0, 1, 16, ctypes.byref(cfg)) == 0 and cfg.cols == 1
+            assert lib.fss_choose_config(8, 8192, 1024, 0, 0, 16, ctypes.byref(cfg)) == 0 and cfg.cols == 1
+        finally:
+            lib.fss_set_cache_policy(previous)
     # odd d forces the scalar path; 2-byte alignment too
     assert lib.fss_choose_config(2, 100, 77, 0, 0, 16, ctypes.byref(cfg)) == 0 and cfg.vec == 1
     assert lib.fss_choose_config(2, 100, 64, 0, 0, 2, ctypes.byref(cfg)) == 0 and cfg.vec == 1
