@@ -217,6 +217,15 @@ __device__ __forceinline__ int slice_steps_inside(int64_t seq, int64_t r0, int c
   return __builtin_amdgcn_readfirstlane(n);
 }
 
+// A constant the compiler materialises where it is used.  Constants it recognises as
+// loop-invariant are otherwise put into registers ahead of the tile loop and kept there for
+// the whole kernel (or spilled, and reloaded in the middle of the look-back): four to six
+// registers in kernels that have none to spare.
+__device__ __forceinline__ float local_const(float x) {
+  asm volatile("" : "+v"(x));
+  return x;
+}
+
 // Makes the compiler forget what it derived from a packed row: the rows stay
 // packed in registers across the chaining phase and are unpacked again after
 // it, instead of keeping an fp32 copy of every element alive next to them.
@@ -575,8 +584,9 @@ __device__ __forceinline__ void chain_chunks(const ScanArgs &p, const TileCtx &c
   float hin[VEC], accA[VEC], accB[VEC];
 #pragma unroll
   for (int v = 0; v < VEC; ++v) {
-    accA[v] = 1.0f;
-    accB[v] = hin[v] = 0.0f;
+    accA[v] = local_const(1.0f);
+    accB[v] = local_const(0.0f);
+    hin[v] = local_const(0.0f);
   }
   int nearest = c.chunk - 1;  // nearest earlier chunk not folded yet
   int other_nearest = nearest;
@@ -586,7 +596,7 @@ __device__ __forceinline__ void chain_chunks(const ScanArgs &p, const TileCtx &c
   uint32_t kind0 = kPredNone;
   float q0A[VEC], q0B[VEC];
 #pragma unroll
-  for (int v = 0; v < VEC; ++v) q0A[v] = q0B[v] = 0.0f;
+  for (int v = 0; v < VEC; ++v) q0A[v] = q0B[v] = local_const(0.0f);
   if constexpr (HAS_MID) {
     if (wave < c.look && nearest - wave * c.span >= 0) {
       ChunkWords<VEC> w;
@@ -624,7 +634,7 @@ __device__ __forceinline__ void chain_chunks(const ScanArgs &p, const TileCtx &c
 #pragma unroll
           for (int v = 0; v < VEC; ++v) {
             qA[v] = 0.0f;
-            qB[v] = __builtin_nanf("");
+            qB[v] = local_const(__builtin_nanf(""));
           }
           break;
         }
@@ -645,7 +655,7 @@ __device__ __forceinline__ void chain_chunks(const ScanArgs &p, const TileCtx &c
 #pragma unroll
             for (int v = 0; v < VEC; ++v) {
               rA[v] = 0.0f;
-              rB[v] = __builtin_nanf("");
+              rB[v] = local_const(__builtin_nanf(""));
             }
             break;
           }
