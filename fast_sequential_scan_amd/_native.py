@@ -33,6 +33,7 @@ EXPORTED_SYMBOLS = (
     "fss_workspace_status",
     "fss_workspace_attach_flag",
     "fss_debug_set_spin_limit",
+    "fss_debug_tile_groups",
     "fss_scan_fwd_noalloc",
     "fss_choose_config",
     "fss_scan_fwd_bf16",
@@ -101,6 +102,7 @@ def _declare(lib: ctypes.CDLL) -> None:
     lib.fss_workspace_attach_flag.argtypes = [_vp, _vp, _vp]
     lib.fss_debug_set_spin_limit.restype = ctypes.c_uint32
     lib.fss_debug_set_spin_limit.argtypes = [ctypes.c_uint32]
+    lib.fss_debug_tile_groups.argtypes = [ctypes.c_int32, ctypes.c_int32, ctypes.c_int32, ctypes.POINTER(ctypes.c_int32)]
     lib.fss_scan_fwd_noalloc.restype = _int
     lib.fss_scan_fwd_noalloc.argtypes = [_int, _vp, _vp, _vp, _i64, _i64, _i64, _vp]
     lib.fss_choose_config.restype = _int

@@ -322,6 +322,35 @@ struct ScanArgs {
 #endif
 };
 
+// Which column group the workgroup that takes slot `slot` of a chunk works on (tiles are
+// numbered chunk-major: tile = chunk * n_groups + slot, and workgroup b takes tiles b,
+// b + grid, ...).  Workgroup b runs on XCD b % 8, so with the groups dealt out in eighths the
+// workgroups of one XCD share consecutive groups: whole rows of a few batch items instead of
+// one 256-byte stripe of every row (`per` groups each; 0: the number of groups does not
+// divide by 8, slot s takes group s).  Within its eighth a workgroup moves on by one group with
+// every tile it takes (`turn` = tiles it has taken so far, modulo per), so that column stripes
+// which the memory system serves more slowly than others (measured on MI355X: by 10-15 %) are
+// shared out evenly; a column's chunks stay on one XCD, and so do the words that chain them.
+// The rotation needs every round of the grid to cover whole chunks - otherwise two slots of
+// one chunk, taken in different rounds, could map to the same group.
+struct TileOrder {
+  uint32_t n_groups, per;
+  bool rotate;
+};
+__host__ __device__ inline TileOrder tile_order(uint32_t n_groups, uint32_t grid) {
+  TileOrder o;
+  o.n_groups = n_groups;
+  o.per = (n_groups & 7u) == 0 ? n_groups >> 3 : 0u;
+  o.rotate = o.per > 1 && grid % n_groups == 0;
+  return o;
+}
+__host__ __device__ inline uint32_t tile_group(const TileOrder &o, uint32_t slot, uint32_t turn) {
+  if (!o.per) return slot;
+  uint32_t k = (slot >> 3) + (o.rotate ? turn : 0u);
+  if (k >= o.per) k -= o.per;
+  return (slot & 7u) * o.per + k;
+}
+
 // Optional (bs, d) fp32 rows of the scans with a state entering/leaving the sequence.
 // The plain scan is compiled against the empty variant, whose members are constant
 // nulls: it carries no kernel arguments for them and every use folds away.

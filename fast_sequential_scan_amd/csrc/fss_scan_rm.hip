@@ -502,33 +502,20 @@ __global__ __launch_bounds__(MAXW * 64) void scan_kernel(const ScanArgs p, const
   // blockIdx, blockIdx + gridDim, ...  Tiles are numbered chunk-major, so a tile
   // only ever waits for tiles with smaller numbers: those belong to a resident
   // workgroup that reaches them no later than this one reaches its own.
-  // Which column group a workgroup takes in a chunk.  Workgroup b runs on XCD b % 8, so with the
-  // groups in eighths the workgroups of one XCD share consecutive groups: whole rows of a few
-  // batch items instead of one 256-byte stripe of every row (`per` groups each; 0: the number
-  // of groups does not divide, slot s takes group s).  Within its eighth a workgroup moves
-  // on by one group with every tile it takes, so that column stripes which the memory system
-  // serves more slowly than others (measured: by up to 15 %) are shared out evenly; a
-  // column's chunks stay on one XCD, and so do the words that chain them.  The rotation
-  // needs every round of the grid to cover whole chunks (or two slots of one chunk could
-  // map to the same group).  bs 8 seq 4096 d 1024 bf16, forward + backward: 96.3 -> 94.3 us
-  // on one set of tensors, 117.7 -> 111.0 us over eight sets in rotation.
-  const uint32_t n_groups = static_cast<uint32_t>(p.n_groups);
-  const uint32_t per = (n_groups & 7u) == 0 ? n_groups >> 3 : 0u;
-  const bool rotate = per > 1 && gridDim.x % n_groups == 0;
-  uint32_t turn = 0;  // tiles this workgroup has taken, modulo per
+  // (which column group a slot of a chunk stands for: tile_order; bs 8 seq 4096 d 1024 bf16, forward +
+  // backward, against slot s = group s: 96.3 -> 94.3 us on one set of tensors, 117.7 -> 111.0 us
+  // over eight sets in rotation)
+  const TileOrder order = tile_order(static_cast<uint32_t>(p.n_groups), gridDim.x);
+  const uint32_t n_groups = order.n_groups;
+  uint32_t turn = 0;  // tiles this workgroup has taken, modulo order.per
   uint32_t parity = 0;
   for (uint32_t tile = blockIdx.x; tile < static_cast<uint32_t>(p.n_tiles); tile += gridDim.x, parity ^= 1u) {
     c.lds_map = lds_maps + (parity * waves_total + c.wcol * c.n_waves) * kLaneSlots;
     // unsigned, wave-uniform arithmetic: stays on the scalar unit
     // (the compiler divides through a vector-unit reciprocal: pin the quotients back)
     const uint32_t chunk = __builtin_amdgcn_readfirstlane(tile / n_groups);
-    uint32_t group = tile - chunk * n_groups;
-    if (per) {
-      uint32_t k = (group >> 3) + turn;
-      if (k >= per) k -= per;
-      group = (group & 7u) * per + k;
-      if (rotate) turn = turn + 1 == per ? 0u : turn + 1;
-    }
+    const uint32_t group = tile_group(order, tile - chunk * n_groups, turn);
+    if (order.rotate) turn = turn + 1 == order.per ? 0u : turn + 1;
     const uint32_t ctile = group * COLS + static_cast<uint32_t>(c.wcol);
     const uint32_t batch = __builtin_amdgcn_readfirstlane(ctile / static_cast<uint32_t>(p.tiles_per_row));
     const uint32_t coltile = ctile - batch * static_cast<uint32_t>(p.tiles_per_row);

@@ -149,6 +149,14 @@ int fss_workspace_attach_flag(void *workspace, uint32_t *flag, void *stream);
  * Process-wide; returns the previous value.
  */
 uint32_t fss_debug_set_spin_limit(uint32_t polls);
+/*
+ * Test hook (host only, no device call): the order in which the row-major kernels take
+ * their tiles.  Tiles are numbered chunk-major (tile = chunk * n_groups + slot) and workgroup b
+ * of a grid of `grid` workgroups takes tiles b, b + grid, ...; groups[tile] receives the column
+ * group that tile stands for, for tile = 0 .. n_tiles-1.  Every chunk's slots must map onto its
+ * groups one to one.  No counterpart in the reference (one block per batch row, no tiles).
+ */
+int fss_debug_tile_groups(int32_t n_groups, int32_t grid, int32_t n_tiles, int32_t *groups);
 
 /* The configuration the library would choose for this shape (for reporting). */
 int fss_choose_config(int64_t bs, int64_t seq, int64_t d, int dtype, int dir,

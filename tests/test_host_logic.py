@@ -373,3 +373,46 @@ def test_chosen_configurations_are_valid_for_random_shapes():
         # shape (any alignment, the library's own choice) covers it
         explicit = _native.FssConfig(cfg.vec, cfg.steps, cfg.waves, 0)
         assert 4096 <= lib.fss_workspace_bytes(bs, seq, d, dtype, direction, ctypes.byref(explicit)) <= need, what
+
+
+def _tile_groups(lib, n_groups, grid, n_chunks):
+    n_tiles = n_groups * n_chunks
+    out = (ctypes.c_int32 * n_tiles)()
+    assert lib.fss_debug_tile_groups(n_groups, grid, n_tiles, out) == 0
+    return np.frombuffer(out, dtype=np.int32).reshape(n_chunks, n_groups)
+
+
+def test_tile_order_covers_every_group_of_every_chunk_once():
+    """The order in which the kernels take their tiles (which column group a slot of a chunk
+    stands for) must be one to one within every chunk, whatever the grid - a collision would
+    leave a tile undone and another done twice.  Where the workgroups of an XCD (workgroup
+    index modulo 8) share consecutive groups, a column's chunks must stay on one XCD, and
+    with the rotation on, a workgroup must meet different groups in successive tiles."""
+    lib = _native.lib()
+    rng = np.random.default_rng(11)
+    cases = [(64, 256, 16), (64, 256, 8), (128, 256, 4), (32, 256, 16), (64, 64, 5), (64, 128, 7), (8, 256, 300),
+             (16, 256, 128), (12, 256, 9), (64, 48, 6), (64, 255, 6), (1, 256, 40), (7, 3, 11), (256, 256, 3), (512, 256, 5)]
+    cases += [(int(rng.integers(1, 300)), int(rng.integers(1, 300)), int(rng.integers(1, 20))) for _ in range(300)]
+    cases += [(8 * int(rng.integers(1, 40)), 8 * int(rng.integers(1, 40)), int(rng.integers(1, 20))) for _ in range(300)]
+    rotated = 0
+    for n_groups, grid, n_chunks in cases:
+        g = _tile_groups(lib, n_groups, grid, n_chunks)
+        for c in range(n_chunks):
+            assert sorted(g[c].tolist()) == list(range(n_groups)), (n_groups, grid, n_chunks, c)
+        if n_groups % 8 == 0:
+            # slot s belongs to XCD s % 8 when the grid is a multiple of 8 too; its group lies in that XCD's eighth
+            per = n_groups // 8
+            assert (g // per == np.arange(n_groups) % 8).all(), (n_groups, grid)
+            if per > 1 and grid % n_groups == 0 and n_chunks * n_groups > grid:
+                rounds = g.reshape(-1)[: (n_chunks * n_groups) // grid * grid].reshape(-1, grid)
+                if rounds.shape[0] > 1:
+                    assert (rounds[0] != rounds[1]).all(), (n_groups, grid)
+                    rotated += 1
+        else:
+            assert (g == np.arange(n_groups)).all()
+    assert rotated > 20
+    # the headline backward: 64 groups, 256 workgroups, 16 chunks - every workgroup meets 4 different stripes
+    g = _tile_groups(lib, 64, 256, 16).reshape(4, 256)
+    assert all(len(set(g[:, b].tolist())) == 4 for b in range(256))
+    assert lib.fss_debug_tile_groups(0, 256, 0, (ctypes.c_int32 * 1)()) != 0
+    assert lib.fss_debug_tile_groups(8, 8, 8, None) != 0
