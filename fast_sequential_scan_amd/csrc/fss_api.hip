@@ -260,11 +260,9 @@ int fss_debug_tile_groups(int32_t n_groups, int32_t grid, int32_t n_tiles, int32
   if (!groups) return FSS_ERR_NULL_POINTER;
   if (n_groups <= 0 || grid <= 0 || n_tiles < 0) return FSS_ERR_BAD_SHAPE;
   const fss::TileOrder order = fss::tile_order(static_cast<uint32_t>(n_groups), static_cast<uint32_t>(grid));
-  for (int32_t tile = 0; tile < n_tiles; ++tile) {
-    // (a workgroup's turn counts the tiles it has taken: tile / grid of them before this one)
-    const uint32_t turn = order.per ? static_cast<uint32_t>(tile / grid) % order.per : 0u;
-    groups[tile] = static_cast<int32_t>(fss::tile_group(order, static_cast<uint32_t>(tile % n_groups), turn));
-  }
+  for (int32_t tile = 0; tile < n_tiles; ++tile)
+    groups[tile] = static_cast<int32_t>(
+        fss::tile_group(order, static_cast<uint32_t>(tile % n_groups), static_cast<uint32_t>(tile / n_groups)));
   return FSS_OK;
 }
 

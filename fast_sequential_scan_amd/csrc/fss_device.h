@@ -322,31 +322,40 @@ struct ScanArgs {
 #endif
 };
 
-// Which column group the workgroup that takes slot `slot` of a chunk works on (tiles are
+// Which column group the workgroup that takes slot `slot` of chunk `chunk` works on (tiles are
 // numbered chunk-major: tile = chunk * n_groups + slot, and workgroup b takes tiles b,
 // b + grid, ...).  Workgroup b runs on XCD b % 8, so with the groups dealt out in eighths the
 // workgroups of one XCD share consecutive groups: whole rows of a few batch items instead of
 // one 256-byte stripe of every row (`per` groups each; 0: the number of groups does not
-// divide by 8, slot s takes group s).  Within its eighth a workgroup moves on by one group with
-// every tile it takes (`turn` = tiles it has taken so far, modulo per), so that column stripes
-// which the memory system serves more slowly than others (measured on MI355X: by 10-15 %) are
-// shared out evenly; a column's chunks stay on one XCD, and so do the words that chain them.
-// The rotation needs every round of the grid to cover whole chunks - otherwise two slots of
-// one chunk, taken in different rounds, could map to the same group.
+// divide by 8, slot s takes group s).  Within its eighth the deal moves on by one group from one
+// round of the grid to the next (`in_flight` chunks make a round), so that a workgroup meets a
+// different column stripe with every tile: the memory system serves some stripes more slowly
+// than others (measured on MI355X: byte offsets 256-511 of every KiB by 12 %), and the kernel ends
+// with its slowest workgroup.  A column's chunks stay on one XCD, and so do the words that
+// chain them.  The turn depends on the chunk alone, so every chunk's slots map onto its groups
+// one to one whatever the grid.
 struct TileOrder {
-  uint32_t n_groups, per;
-  bool rotate;
+  uint32_t n_groups, per, in_flight;
 };
+__host__ __device__ inline uint32_t wave_uniform(uint32_t x) {
+#if defined(__HIP_DEVICE_COMPILE__)
+  return __builtin_amdgcn_readfirstlane(x);  // (divisions run on the vector unit: pin the result back)
+#else
+  return x;
+#endif
+}
 __host__ __device__ inline TileOrder tile_order(uint32_t n_groups, uint32_t grid) {
   TileOrder o;
   o.n_groups = n_groups;
   o.per = (n_groups & 7u) == 0 ? n_groups >> 3 : 0u;
-  o.rotate = o.per > 1 && grid % n_groups == 0;
+  o.in_flight = wave_uniform((grid + n_groups - 1) / n_groups);
+  if (o.in_flight < 1) o.in_flight = 1;
   return o;
 }
-__host__ __device__ inline uint32_t tile_group(const TileOrder &o, uint32_t slot, uint32_t turn) {
-  if (!o.per) return slot;
-  uint32_t k = (slot >> 3) + (o.rotate ? turn : 0u);
+__host__ __device__ inline uint32_t tile_group(const TileOrder &o, uint32_t slot, uint32_t chunk) {
+  if (o.per <= 1) return slot;
+  const uint32_t turn = wave_uniform((chunk / o.in_flight) % o.per);
+  uint32_t k = (slot >> 3) + turn;
   if (k >= o.per) k -= o.per;
   return (slot & 7u) * o.per + k;
 }

@@ -507,15 +507,13 @@ __global__ __launch_bounds__(MAXW * 64) void scan_kernel(const ScanArgs p, const
   // over eight sets in rotation)
   const TileOrder order = tile_order(static_cast<uint32_t>(p.n_groups), gridDim.x);
   const uint32_t n_groups = order.n_groups;
-  uint32_t turn = 0;  // tiles this workgroup has taken, modulo order.per
   uint32_t parity = 0;
   for (uint32_t tile = blockIdx.x; tile < static_cast<uint32_t>(p.n_tiles); tile += gridDim.x, parity ^= 1u) {
     c.lds_map = lds_maps + (parity * waves_total + c.wcol * c.n_waves) * kLaneSlots;
     // unsigned, wave-uniform arithmetic: stays on the scalar unit
     // (the compiler divides through a vector-unit reciprocal: pin the quotients back)
     const uint32_t chunk = __builtin_amdgcn_readfirstlane(tile / n_groups);
-    const uint32_t group = tile_group(order, tile - chunk * n_groups, turn);
-    if (order.rotate) turn = turn + 1 == order.per ? 0u : turn + 1;
+    const uint32_t group = tile_group(order, tile - chunk * n_groups, chunk);
     const uint32_t ctile = group * COLS + static_cast<uint32_t>(c.wcol);
     const uint32_t batch = __builtin_amdgcn_readfirstlane(ctile / static_cast<uint32_t>(p.tiles_per_row));
     const uint32_t coltile = ctile - batch * static_cast<uint32_t>(p.tiles_per_row);

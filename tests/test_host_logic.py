@@ -387,7 +387,7 @@ def test_tile_order_covers_every_group_of_every_chunk_once():
     stands for) must be one to one within every chunk, whatever the grid - a collision would
     leave a tile undone and another done twice.  Where the workgroups of an XCD (workgroup
     index modulo 8) share consecutive groups, a column's chunks must stay on one XCD, and
-    with the rotation on, a workgroup must meet different groups in successive tiles."""
+    a workgroup must meet different groups in successive rounds of the grid."""
     lib = _native.lib()
     rng = np.random.default_rng(11)
     cases = [(64, 256, 16), (64, 256, 8), (128, 256, 4), (32, 256, 16), (64, 64, 5), (64, 128, 7), (8, 256, 300),
@@ -403,11 +403,11 @@ def test_tile_order_covers_every_group_of_every_chunk_once():
             # slot s belongs to XCD s % 8 when the grid is a multiple of 8 too; its group lies in that XCD's eighth
             per = n_groups // 8
             assert (g // per == np.arange(n_groups) % 8).all(), (n_groups, grid)
-            if per > 1 and grid % n_groups == 0 and n_chunks * n_groups > grid:
-                rounds = g.reshape(-1)[: (n_chunks * n_groups) // grid * grid].reshape(-1, grid)
-                if rounds.shape[0] > 1:
-                    assert (rounds[0] != rounds[1]).all(), (n_groups, grid)
-                    rotated += 1
+            in_flight = -(-grid // n_groups)
+            if per > 1 and n_chunks > in_flight:
+                # one round of the grid later, every slot stands for another group of its eighth
+                assert (g[0] != g[in_flight]).all(), (n_groups, grid)
+                rotated += 1
         else:
             assert (g == np.arange(n_groups)).all()
     assert rotated > 20
