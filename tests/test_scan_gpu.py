@@ -288,6 +288,20 @@ def test_baseline_configs_full_size(oracle, case):
     ext.workspace_status()
 
 
+@pytest.mark.parametrize(
+    "bs,seq,d",
+    [(12, 2048, 1024), (8, 1536, 1536), (5, 2048, 1024), (2, 4096, 1792), (16, 1024, 2048)],
+    ids=["96_groups", "96_groups_12_stripes", "40_groups", "28_groups", "256_groups"],
+)
+def test_tile_orders_of_full_grids(oracle, bs, seq, d):
+    """Shapes whose launches fill the device and take their tiles in the different orders the
+    kernels know: column groups in eighths that do not divide the grid (96, 40), that equal it
+    (256), and a number of groups that does not divide by 8 (28)."""
+    alpha, beta, dout = make_inputs("sigmoid", bs, seq, d, seed=bs + d)
+    check_bf16(oracle, alpha, beta, dout, what=f"({bs},{seq},{d})")
+    ext.workspace_status()
+
+
 def test_fp32_at_headline_shape(oracle):
     """fp32 at bs 8, seq 4096, d 1024: 128 MiB per tensor, so the backward runs the instantiation
     that reads dout with the streaming hint.  Against the fp32 oracle, the reference's fp32 bar
