@@ -95,6 +95,33 @@ def test_plain_and_state_scans(oracle, seed):
 
 
 @pytest.mark.parametrize("seed", range(12))
+def test_many_column_groups_under_random_grids(oracle, seed):
+    """Shapes with enough column groups for the tile orders that deal them out by XCD (a multiple
+    of 8 groups: 24 to 128 here), small tiles (many chunks per sequence) and grids capped at random,
+    so that rounds of the grid cut through chunks at every offset."""
+    rng = np.random.default_rng(4000 + seed)
+    dtype = DTYPES[seed % 3]
+    bs = int(rng.choice([3, 5, 8, 12, 16]))
+    d = int(rng.choice([512, 1024]))
+    seq = int(rng.choice([257, 513, 1000]))
+    alpha, beta, dout = _tensors(rng, (bs, seq, d), dtype)
+    vec = 2 if dtype != torch.float32 else 1  # 128 (64) channels per column tile
+    grids = [0, 8, 24, 40, 64, 100, 136]
+    fwd_cfg = (vec, int(rng.choice([8, 16])), int(rng.choice([1, 2, 4])), int(rng.choice(grids)))
+    bwd_cfg = (vec, int(rng.choice([8, 16])), int(rng.choice([1, 2, 4])), int(rng.choice(grids)))
+    what = f"seed {seed} {dtype} {(bs, seq, d)} fwd {fwd_cfg} bwd {bwd_cfg}"
+    a, b, do = alpha.to(DEV), beta.to(DEV), dout.to(DEV)
+    h = ext._forward(dtype, a, b, fwd_cfg)
+    ga, gb = ext._backward(dtype, a, h, do, bwd_cfg)
+    a32, b32, d32 = alpha.float().numpy(), beta.float().numpy(), dout.float().numpy()
+    _check(h, oracle.scan_fwd_f32(a32, b32), dtype, what + " h")
+    ga_or, gb_or = oracle.scan_bwd_f32(a32, h.float().cpu().numpy(), d32)
+    _check(gb, gb_or, dtype, what + " grad_beta")
+    _check(ga, ga_or, dtype, what + " grad_alpha")
+    ext.workspace_status()
+
+
+@pytest.mark.parametrize("seed", range(12))
 def test_gated_scans(oracle, seed):
     rng = np.random.default_rng(2000 + seed)
     dtype = DTYPES[seed % 3]
