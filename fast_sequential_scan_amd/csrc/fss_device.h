@@ -556,17 +556,54 @@ __device__ __forceinline__ void fold_wave_maps(const float2 *lds_map, int lane, 
   }
 }
 
+// The same composition over all `count` waves, by one wave for the whole workgroup: slot w
+// receives what the waves before w do to the chunk's incoming state (the composition of maps
+// 0 .. w-1, in place of map w, which nobody else reads), and (A, B) the chunk's map.  Every
+// other wave then finds its prefix with one LDS read after the next barrier, instead of
+// composing up to 15 maps itself on the way to its last phase.  Same operations in the same
+// order as fold_wave_maps, so the results are bit for bit the same.
+template <int VEC>
+__device__ __forceinline__ void fold_and_leave_prefixes(float2 *lds_map, int lane, int count, float *A, float *B) {
+  constexpr int kBatch = 4;
+#pragma unroll
+  for (int v = 0; v < VEC; ++v) {
+    A[v] = 1.0f;
+    B[v] = 0.0f;
+  }
+  for (int w0 = 0; w0 < count; w0 += kBatch) {
+    float2 m[kBatch][VEC];
+#pragma unroll
+    for (int i = 0; i < kBatch; ++i) {
+      const int w = w0 + i < count ? w0 + i : count - 1;  // clamped: the read stays in bounds
+#pragma unroll
+      for (int v = 0; v < VEC; ++v) m[i][v] = lds_map[(w * VEC + v) * 64 + lane];
+    }
+#pragma unroll
+    for (int i = 0; i < kBatch; ++i) {
+      if (w0 + i < count) {
+#pragma unroll
+        for (int v = 0; v < VEC; ++v) {
+          lds_map[((w0 + i) * VEC + v) * 64 + lane] = make_float2(A[v], B[v]);
+          B[v] = fma0(m[i][v].x, B[v], m[i][v].y);
+          A[v] *= m[i][v].x;
+        }
+      }
+    }
+  }
+}
+
 // Phase 2.  In: this wave's slice as the map x -> mA*x + mB.  Out: the state
 // entering the slice.  Every wave of the workgroup must call it (barriers).
 //
 // After one barrier wave 0 composes all the waves' maps into the chunk's map and
-// publishes it.  Meanwhile wave w (w < look) fetches what chunk-1-w offers - its
+// publishes it, leaving in every wave's slot the composition of the waves before it.  Meanwhile wave w (w < look) fetches what chunk-1-w offers - its
 // outgoing state if it has one, else its map - so a look-back over `look` chunks
 // costs one memory round trip instead of one per chunk.  After a second barrier
 // every wave folds what the look-back waves found into the chunk's incoming state
 // itself (a few multiply-adds: cheaper than a third barrier and a broadcast), wave 0
 // also publishes the chunk's outgoing state, and every wave applies the composition
-// of the waves before it.  Chains longer than `look` repeat the fetch.
+// of the waves before it (one LDS read; the first chunk of a sequence, which has no second
+// barrier to wait at, composes it itself).  Chains longer than `look` repeat the fetch.
 //
 // `mid` (only with HAS_MID) is called once by every wave, by the look-back waves right after their
 // first fetch has been issued: loads it issues travel while the chain is resolved and
@@ -584,17 +621,23 @@ __device__ __forceinline__ void chain_chunks(const ScanArgs &p, const TileCtx &c
   const bool look_back = c.chained && c.chunk > 0;
   uint64_t *mine = nullptr;
   float cA[VEC], cB[VEC];
-  if (wave == 0 && c.chained && !c.last) {
-    // the chunk's own map, needed by later chunks: out as early as possible
-    fold_wave_maps<VEC>(c.lds_map, lane, c.n_waves, cA, cB);
+  if (wave == 0 && look_back) {
+    // the chunk's own map, needed by later chunks: out as early as possible - and on the way
+    // every wave's prefix, left where its map was (the waves read it behind the look-back's barrier)
+    fold_and_leave_prefixes<VEC>(c.lds_map, lane, c.n_waves, cA, cB);
     mine = p.words + (static_cast<size_t>(c.chunk) * p.n_ctiles + c.ctile) * 3 * kLaneSlots + lane;
-    if (c.chunk > 0) {
+    if (!c.last) {
 #pragma unroll
       for (int v = 0; v < VEC; ++v) {
         st_word(mine + (0 * VEC + v) * 64, c.tag, cA[v]);
         st_word(mine + (1 * VEC + v) * 64, c.tag, cB[v]);
       }
     }
+  } else if (wave == 0 && c.chained && !c.last) {
+    // first chunk of a chained sequence: its map is needed for its outgoing state only (the
+    // other waves compose their prefixes themselves: no barrier follows that they could wait at)
+    fold_wave_maps<VEC>(c.lds_map, lane, c.n_waves, cA, cB);
+    mine = p.words + (static_cast<size_t>(c.chunk) * p.n_ctiles + c.ctile) * 3 * kLaneSlots + lane;
   }
   FSS_STAMP(c, p, 3);
 
@@ -760,7 +803,13 @@ __device__ __forceinline__ void chain_chunks(const ScanArgs &p, const TileCtx &c
     __syncthreads();  // the slots are about to be overwritten: wait until every wave has read them
   }
   FSS_STAMP(c, p, 4);
-  fold_wave_maps<VEC>(c.lds_map, lane, wave, pA, pB);  // after the polls: those are what is waited for
+  // (the prefix wave 0 left in this wave's slot, behind the loop's barrier)
+#pragma unroll
+  for (int v = 0; v < VEC; ++v) {
+    const float2 e = c.lds_map[(wave * VEC + v) * 64 + lane];
+    pA[v] = e.x;
+    pB[v] = e.y;
+  }
 #pragma unroll
   for (int v = 0; v < VEC; ++v) state[v] = fma0(pA[v], hin[v], pB[v]);
   FSS_STAMP(c, p, 5);
