@@ -129,8 +129,7 @@ inline void complete_config(fss_config &c, int64_t bs, int64_t seq, int64_t d, i
   auto rung = [&](int v, int s, int w, int64_t need = kCus) { ladder[n++] = Rung{v, s, w, need}; };
   const bool fwd = dir == FSS_FWD;
   if (!gated && fwd) {
-    // (very long sequences: one channel per lane, i.e. twice the independent chains, is 5-16 % faster)
-    if (narrow && seq < 32768) rung(2, 32, 16);
+    if (narrow) rung(2, 32, 16);
     if (wide32) rung(2, 16, 16);
     rung(1, 32, 16);
     if (seq <= 2048) rung(1, 16, 16);
