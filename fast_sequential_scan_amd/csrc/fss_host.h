@@ -120,17 +120,23 @@ inline void complete_config(fss_config &c, int64_t bs, int64_t seq, int64_t d, i
   // two channels per lane: even d, 2-element alignment, and never pad a row to twice its width
   const bool can2 = d % 2 == 0 && align % (2 * static_cast<size_t>(esize)) == 0 &&
                     ceil_div(d, 128) * 128 < 2 * ceil_div(d, 64) * 64;
-  // fp32, very large tensors (from 2^26 elements) with wide rows and sequences of a few
-  // thousand steps: 8 bytes per lane measured 5-15 % faster than 4 (below that size, slower)
-  const bool wide32 = !narrow && !gated && can2 && d >= 512 && seq <= 4096 &&
-                      bs * seq * d >= (static_cast<int64_t>(1) << 26);
-  Rung ladder[6];
+  // fp32, very large tensors with wide rows (56 shapes of 2^24..2^27 elements, d 512..4096, seq
+  // 512..8192, six configurations each).  Forward from 2^26 elements: 16 steps per lane are 2-6 %
+  // faster than 32 up to seq 4096, and 8 bytes per lane another 3-8 % at seq 512 (4-9 % slower
+  // from seq 2048).  Backward: 8 bytes per lane with 8 steps are 4-11 % faster from 2^27 elements
+  // and 3-10 % slower at 2^26.
+  const int64_t elems = bs * seq * d;
+  const bool big32 = !narrow && !gated && d >= 512 && elems >= (static_cast<int64_t>(1) << 26);
+  const bool wide32_fwd = big32 && can2 && seq <= 512;
+  const bool wide32_bwd = big32 && can2 && elems >= (static_cast<int64_t>(1) << 27);
+  Rung ladder[8];
   int n = 0;
   auto rung = [&](int v, int s, int w, int64_t need = kCus) { ladder[n++] = Rung{v, s, w, need}; };
   const bool fwd = dir == FSS_FWD;
   if (!gated && fwd) {
     if (narrow) rung(2, 32, 16);
-    if (wide32) rung(2, 16, 16);
+    if (wide32_fwd) rung(2, 16, 16);
+    else if (big32 && seq <= 4096) rung(1, 16, 16);
     rung(1, 32, 16);
     if (seq <= 2048) rung(1, 16, 16);
     rung(1, 32, 8, 0);
@@ -141,7 +147,7 @@ inline void complete_config(fss_config &c, int64_t bs, int64_t seq, int64_t d, i
       if (seq >= 16384) rung(1, 16, 16); else rung(2, 16, 8);
       if (seq > 256) rung(1, 16, 8); else rung(2, 8, 8);
     } else {
-      if (wide32) rung(2, 8, 16);
+      if (wide32_bwd) rung(2, 8, 16);
       rung(1, 16, 16);
       rung(1, 16, 8);
     }
@@ -150,6 +156,8 @@ inline void complete_config(fss_config &c, int64_t bs, int64_t seq, int64_t d, i
     // The gated kernels spend as much time on arithmetic as on memory and like more, smaller
     // waves; a sequence that 8 waves cover wants two workgroups per CU before it takes them.
     if (narrow) {
+      // (from 8192 steps two 8-wave workgroups per CU are 3-5 % faster than one of 16 waves: 8 shapes of 9)
+      if (seq >= 8192) rung(2, 32, 8, 2 * kCus);
       if (seq > 256) rung(2, 32, 16); else rung(2, 32, 8, 2 * kCus);
       if (seq >= 4096) rung(1, 32, 16); else rung(2, 16, 16);
       if (seq >= 16384) rung(1, 32, 8);
@@ -162,6 +170,8 @@ inline void complete_config(fss_config &c, int64_t bs, int64_t seq, int64_t d, i
   } else {
     // gated backward: four tensors per timestep, at most 16 steps per lane (fp32: 8 are faster)
     if (narrow) {
+      // (many short sequences: two 8-wave workgroups per CU are 3-16 % faster: 6 shapes of 7 at 2^25 elements)
+      if (seq <= 1024) rung(2, 16, 8, 8 * kCus);
       if (seq > 256) rung(2, 16, 16); else rung(2, 16, 8, 4 * kCus);
       rung(2, 8, 16);
       rung(2, 8, 8, seq <= 256 ? 1 : kCus);
@@ -186,11 +196,11 @@ inline void complete_config(fss_config &c, int64_t bs, int64_t seq, int64_t d, i
     pick = fss_config{v, s, w, 0, 0};
     if (bs * ceil_div(d, 64 * static_cast<int64_t>(v)) * ceil_div(seq, static_cast<int64_t>(s) * w) >= ladder[i].need) break;
   }
-  // Forward, 16-wave workgroups (one per CU) whose last round would fill less than 90 % of the
+  // Forward and gated backward, 16-wave workgroups (one per CU) whose last round would fill less than 90 % of the
   // CUs: the same tile shape as 8-wave workgroups, two per CU, spreads that round over all CUs
   // (7-18 % faster on 59 of 182 shapes with lengths and widths that are no powers of two; the
-  // backward measured no gain from it).
-  if (fwd && !c.waves && pick.waves == 16) {
+  // plain backward measured no gain from it, the gated backward 5-16 % on 6 shapes of 6).
+  if ((fwd || gated) && !c.waves && pick.waves == 16) {
     const int64_t tiles = bs * ceil_div(d, 64 * static_cast<int64_t>(pick.vec)) * ceil_div(seq, static_cast<int64_t>(pick.steps) * 16);
     const int64_t rounds = ceil_div(tiles, kCus);
     if (rounds >= 2 && tiles * 10 < rounds * kCus * 9) pick.waves = 8;
