@@ -251,6 +251,22 @@ def test_planning_of_the_gated_fp16_and_channel_major_entry_points():
     assert choose(_native.FSS_F32, _native.FSS_GATED_BWD)[1] <= 16
     assert choose(_native.FSS_BF16, _native.FSS_GATED_BWD, (1, 65521, 256))[1] <= 16
     assert choose(_native.FSS_BF16, _native.FSS_GATED_BWD, (1, 1024, 1024)) == (1, 8, 8)
+    # two 8-wave workgroups per CU: long gated forwards, many short gated backwards, ragged last rounds
+    assert choose(_native.FSS_BF16, _native.FSS_GATED_FWD, (2, 8192, 1024)) == (2, 32, 8)
+    assert choose(_native.FSS_BF16, _native.FSS_GATED_BWD, (2, 8192, 1024)) == (2, 16, 16)
+    assert choose(_native.FSS_BF16, _native.FSS_GATED_BWD, (64, 512, 1024)) == (2, 16, 8)
+    assert choose(_native.FSS_BF16, _native.FSS_GATED_BWD, (5, 2048, 1024)) == (2, 16, 8)
+    assert choose(_native.FSS_BF16, _native.FSS_BWD, (5, 2048, 1024)) == (2, 16, 16)
+    # two channels per lane in the forward at every sequence length
+    assert choose(_native.FSS_BF16, _native.FSS_FWD, (1, 65521, 256)) == (2, 32, 16)
+    assert choose(_native.FSS_BF16, _native.FSS_FWD, (1, 32768, 1024)) == (2, 32, 16)
+    # fp32, very large tensors
+    assert choose(_native.FSS_F32, _native.FSS_FWD) == (1, 32, 16)
+    assert choose(_native.FSS_F32, _native.FSS_FWD, (16, 4096, 1024)) == (1, 16, 16)
+    assert choose(_native.FSS_F32, _native.FSS_FWD, (256, 512, 512)) == (2, 16, 16)
+    assert choose(_native.FSS_F32, _native.FSS_FWD, (8, 8192, 1024)) == (1, 32, 16)
+    assert choose(_native.FSS_F32, _native.FSS_BWD, (16, 4096, 1024)) == (1, 16, 16)
+    assert choose(_native.FSS_F32, _native.FSS_BWD, (32, 4096, 1024)) == (2, 8, 16)
     # fp16 plans like bf16
     for direction in (_native.FSS_FWD, _native.FSS_BWD):
         assert choose(_native.FSS_F16, direction) == choose(_native.FSS_BF16, direction)

@@ -152,6 +152,18 @@ def test_headline_size_against_oracle(oracle):
     _check_all(oracle, "bf16", 1e-2, 1e-2, gate, x, dout, h, grad_gate, grad_x)
 
 
+@pytest.mark.parametrize("shape", [(2, 8192, 1024), (64, 512, 1024), (5, 2048, 1024)])
+def test_shapes_the_library_gives_two_workgroups_per_cu(oracle, shape):
+    """The library's own choices where they are 8-wave workgroups: a forward of 8192 steps, a backward
+    over many short sequences, a backward whose last round of 16-wave tiles would be ragged."""
+    gate, x, dout = _inputs(shape, torch.bfloat16, seed=sum(shape))
+    gd, xd, dd = gate.to(DEV), x.to(DEV), dout.to(DEV)
+    h = ext.gated_scan_forward(gd, xd)
+    grad_gate, grad_x = ext.gated_scan_backward(gd, xd, h, dd)
+    ext.workspace_status()
+    _check_all(oracle, "bf16", 1e-2, 1e-2, gate, x, dout, h, grad_gate, grad_x)
+
+
 def test_autograd_and_validation():
     gate, x, dout = (t.to(DEV) for t in _inputs((2, 50, 24), torch.bfloat16, seed=10))
     g1, x1 = gate.clone().requires_grad_(True), x.clone().requires_grad_(True)

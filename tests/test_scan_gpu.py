@@ -369,6 +369,30 @@ def test_closed_forms_at_headline_shape():
     ext.workspace_status()
 
 
+@pytest.mark.parametrize("shape", [(32, 4096, 1024), (256, 512, 512)], ids=["2^27", "2^26_seq512"])
+def test_fp32_closed_forms_at_the_sizes_that_change_the_launch_configuration(shape):
+    """fp32 tensors of 2^26 and 2^27 elements take other launch configurations (16 steps or 8 bytes per
+    lane).  alpha == 1 and beta, dout powers of two that differ by channel and batch row: every
+    partial sum and product is exact in fp32 whatever the chunking, so the results are known bit for
+    bit: h[t] = (t+1) beta, grad_beta[t] = (seq-t) dout, grad_alpha[t] = h[t-1] grad_beta[t]."""
+    bs, seq, d = shape
+    t = torch.arange(seq, device=DEV, dtype=torch.float32)[None, :, None]
+    c = torch.arange(d, device=DEV)[None, None, :]
+    b = torch.arange(bs, device=DEV)[:, None, None]
+    beta_bc = torch.ldexp(torch.ones((), device=DEV), (c % 4 + b % 2 - 6).to(torch.int32)).to(torch.float32)
+    dout_bc = torch.ldexp(torch.ones((), device=DEV), (c % 2 - 6 + 0 * b).to(torch.int32)).to(torch.float32)
+    alpha = torch.ones(shape, device=DEV)
+    beta = beta_bc.expand(shape).contiguous()
+    h = ext.scan_forward(alpha, beta)
+    assert torch.equal(h, ((t + 1) * beta_bc).expand(shape))
+    del beta
+    dout = dout_bc.expand(shape).contiguous()
+    ga, gb = ext.scan_backward(alpha, h, dout)
+    ext.workspace_status()
+    assert torch.equal(gb, ((seq - t) * dout_bc).expand(shape))
+    assert torch.equal(ga, (t * beta_bc * (seq - t) * dout_bc).expand(shape))
+
+
 # -------------------------------------------------------------------- edge cases
 
 
