@@ -1,0 +1,69 @@
+"""Loads ``_lib/fss_torch_binding.so`` (csrc/fss_torch_binding.cpp): the C++ dispatch of the plain scan.
+
+The module is an accelerator of host-side dispatch only: what it launches are the kernels of
+``libfss_scan.so`` through the same C ABI the ctypes wrappers use, and whatever it does not cover
+goes through those wrappers.  ``FSS_TORCH_BINDING=0`` keeps every call on the Python wrappers.
+"""
+from __future__ import annotations
+
+import ctypes
+import importlib.machinery
+import importlib.util
+import os
+import threading
+from typing import Any, Callable, Optional
+
+from . import _native
+
+NAME = "fss_torch_binding"
+PATH = os.path.join(_native.PKG_DIR, "_lib", NAME + ".so")
+
+_lock = threading.Lock()
+_module: Any = None
+_tried = False
+
+
+class TorchBindingMissing(RuntimeError):
+    pass
+
+
+def _address(function: Any) -> int:
+    return ctypes.cast(function, ctypes.c_void_p).value
+
+
+def load(slow_backward: Callable[..., Any]) -> Optional[Any]:
+    """The initialised module, or None when it is switched off.  A missing file is an error: the
+    package is built with it (``python -m fast_sequential_scan_amd.build``)."""
+    global _module, _tried
+    if _tried:
+        return _module
+    with _lock:
+        if _tried:
+            return _module
+        if os.environ.get("FSS_TORCH_BINDING", "1") == "0":
+            _tried = True
+            return None
+        lib = _native.lib()  # raises if the HIP library is missing
+        if not os.path.exists(PATH):
+            raise TorchBindingMissing(
+                f"{PATH} not found: build it with `python -m fast_sequential_scan_amd.build` "
+                "(or set FSS_TORCH_BINDING=0 to dispatch through the Python wrappers)"
+            )
+        import torch  # noqa: F401  (the module links against torch's libraries)
+
+        loader = importlib.machinery.ExtensionFileLoader(NAME, PATH)
+        spec = importlib.util.spec_from_loader(NAME, loader)
+        module = importlib.util.module_from_spec(spec)
+        loader.exec_module(module)
+        module.init(
+            _address(lib.fss_scan_fwd_ex), _address(lib.fss_scan_bwd_ex), _address(lib.fss_workspace_bytes),
+            _address(lib.fss_strerror), slow_backward,
+        )
+        _module = module
+        _tried = True
+    return _module
+
+
+def loaded() -> Optional[Any]:
+    """The module if `load` has initialised it."""
+    return _module

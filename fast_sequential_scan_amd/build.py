@@ -10,6 +10,9 @@ Translation units (compiled in parallel, then linked):
   csrc/fss_api.hip       the C ABI, planning, small kernels
   csrc/fss_scan_rm.hip   the row-major scan kernels, once per storage type and direction
   csrc/fss_scan_cm.hip   the channel-major scan kernels
+
+``build_torch_binding`` compiles csrc/fss_torch_binding.cpp (host code: the PyTorch-side dispatch of
+``scan_cu`` in C++ over that C ABI) into ``_lib/fss_torch_binding.so`` with the host compiler.
 """
 from __future__ import annotations
 
@@ -61,7 +64,7 @@ def _run(cmd: List[str], verbose: bool) -> None:
     proc = subprocess.run(cmd, capture_output=True, text=True)
     if proc.returncode != 0:
         sys.stderr.write(proc.stdout + proc.stderr)
-        raise RuntimeError(f"hipcc failed with exit code {proc.returncode}: {' '.join(cmd)}")
+        raise RuntimeError(f"{os.path.basename(cmd[0])} failed with exit code {proc.returncode}: {' '.join(cmd)}")
     if verbose and proc.stderr and "-Rpass" in " ".join(cmd):
         sys.stderr.write(proc.stderr)
 
@@ -84,5 +87,36 @@ def build(verbose: bool = False, extra_flags: Sequence[str] = (), output: str = 
     return output
 
 
+BINDING_NAME = "fss_torch_binding"
+BINDING_PATH = os.path.join(LIB_DIR, BINDING_NAME + ".so")
+
+
+def build_torch_binding(verbose: bool = False, output: str = BINDING_PATH) -> str:
+    """Compiles the PyTorch binding (always) against the installed torch's headers and libraries."""
+    import sysconfig
+
+    import torch
+    from torch.utils import cpp_extension
+
+    os.makedirs(os.path.dirname(output), exist_ok=True)
+    rocm = os.environ.get("ROCM_PATH", "/opt/rocm")
+    cxx = os.environ.get("CXX") or shutil.which("g++") or "g++"
+    includes = [*cpp_extension.include_paths(), os.path.join(rocm, "include"), sysconfig.get_paths()["include"]]
+    cmd = [
+        cxx, "-O2", "-std=c++17", "-fPIC", "-shared", "-w",
+        "-D__HIP_PLATFORM_AMD__=1", "-DUSE_ROCM=1", f"-DTORCH_EXTENSION_NAME={BINDING_NAME}",
+        f"-D_GLIBCXX_USE_CXX11_ABI={int(torch._C._GLIBCXX_USE_CXX11_ABI)}",
+        *(f"-I{path}" for path in includes),
+        os.path.join(SRC_DIR, "fss_torch_binding.cpp"), "-o", output + ".tmp",
+        # torch is imported before this module is loaded, so its libraries are resolved already
+        *(f"-L{path}" for path in cpp_extension.library_paths()),
+        "-lc10", "-lc10_hip", "-ltorch", "-ltorch_cpu", "-ltorch_hip", "-ltorch_python",
+    ]
+    _run(cmd, verbose)
+    os.replace(output + ".tmp", output)
+    return output
+
+
 if __name__ == "__main__":
     print(build(verbose=True))
+    print(build_torch_binding(verbose=True))

@@ -77,14 +77,33 @@ class SequentialScanSingle(Function):
         return alpha_grad, beta_grad
 
 
+# The C++ dispatch (csrc/fss_torch_binding.cpp) takes the common call - contiguous GPU tensors of
+# the right type, outside autocast - from here to the launch and records a C++ autograd node; it
+# answers None for anything else, which then goes through the Functions above, as do all errors.
+_UNRESOLVED = object()
+_fast: Any = _UNRESOLVED
+
+
+def _fast_scan(alpha: torch.Tensor, beta: torch.Tensor, code: int) -> Optional[torch.Tensor]:
+    global _fast
+    if _fast is _UNRESOLVED:
+        binding = _ext.fast_dispatch()
+        _fast = binding.scan if binding is not None else None
+    if _fast is None or not isinstance(alpha, torch.Tensor) or not isinstance(beta, torch.Tensor):
+        return None
+    return _fast(alpha, beta, code)
+
+
 def scan(alpha: torch.Tensor, beta: torch.Tensor) -> torch.Tensor:
     """h[:,0] = beta[:,0]; h[:,t] = alpha[:,t]*h[:,t-1] + beta[:,t]  (bf16, fp32 carry)."""
-    return SequentialScan.apply(alpha, beta)
+    h = _fast_scan(alpha, beta, 0)
+    return h if h is not None else SequentialScan.apply(alpha, beta)
 
 
 def scan_single(alpha: torch.Tensor, beta: torch.Tensor) -> torch.Tensor:
     """The same recurrence on fp32 tensors."""
-    return SequentialScanSingle.apply(alpha, beta)
+    h = _fast_scan(alpha, beta, 1)
+    return h if h is not None else SequentialScanSingle.apply(alpha, beta)
 
 
 class SequentialScanFp16(Function):
@@ -106,7 +125,8 @@ class SequentialScanFp16(Function):
 
 def scan_fp16(alpha: torch.Tensor, beta: torch.Tensor) -> torch.Tensor:
     """The same recurrence on fp16 tensors."""
-    return SequentialScanFp16.apply(alpha, beta)
+    h = _fast_scan(alpha, beta, 2)
+    return h if h is not None else SequentialScanFp16.apply(alpha, beta)
 
 
 class SequentialScanState(Function):

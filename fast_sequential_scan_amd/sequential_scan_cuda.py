@@ -21,7 +21,7 @@ from typing import Dict, List, Optional, Tuple
 
 import torch
 
-from . import _native
+from . import _native, _torch_binding
 
 __all__ = [
     "scan_forward", "scan_backward", "scan_forward_half", "scan_backward_half",
@@ -32,6 +32,7 @@ __all__ = [
 ]
 
 _DTYPE_CODE = {torch.bfloat16: _native.FSS_BF16, torch.float32: _native.FSS_F32, torch.float16: _native.FSS_F16}
+_CODE_DTYPE = {code: dtype for dtype, code in _DTYPE_CODE.items()}
 
 # one workspace per (device, stream): calls on one stream are ordered, calls on
 # different streams must not share the chaining words
@@ -57,7 +58,8 @@ class _Workspace:
         self.buf = buf
         self.ptr = buf.data_ptr()
         self.size = buf.numel()
-        self.launches = 0
+        # (a C integer: the C++ dispatch of the plain scan counts its launches into the same word)
+        self.launches = ctypes.c_int64(0)
         self.flag = torch.zeros(1, dtype=torch.int32).pin_memory()
         self.flag_word = ctypes.c_uint32.from_address(self.flag.data_ptr())
         _native.check(lib.fss_workspace_init(self.ptr, self.size, stream_handle))
@@ -67,7 +69,7 @@ class _Workspace:
         lib = _native.lib()
         _native.check(lib.fss_workspace_init(self.ptr, self.size, stream_handle))
         _native.check(lib.fss_workspace_attach_flag(self.ptr, self.flag.data_ptr(), stream_handle))
-        self.launches = 0
+        self.launches.value = 0
 
     def raise_if_flagged(self) -> None:
         if self.flag_word.value:
@@ -146,6 +148,13 @@ def _need(family: str, code: int, direction: int, bs: int, seq: int, d: int, con
     return need
 
 
+def _need_plain(code: int, bs: int, seq: int, d: int, config) -> int:
+    """Workspace bytes of the plain scan, forward or backward: one workspace serves both, and the
+    C++ dispatch of `scan_cu` only takes a call whose backward it can serve too."""
+    return max(_need("rm", code, _native.FSS_FWD, bs, seq, d, config),
+               _need("rm", code, _native.FSS_BWD, bs, seq, d, config))
+
+
 def _workspace(device: torch.device, stream: "_RawStream", need: int) -> "_Workspace":
     """The workspace of (device, stream), grown to `need` bytes; raises if a scan launched through
     it earlier reported a chain time-out."""
@@ -156,13 +165,35 @@ def _workspace(device: torch.device, stream: "_RawStream", need: int) -> "_Works
             ws.raise_if_flagged()
         ws = _Workspace(torch.empty(max(need, 1 << 20), dtype=torch.uint8, device=device), stream.cuda_stream)
         _workspaces[key] = ws
+        binding = _torch_binding.loaded()
+        if binding is not None:
+            binding.register_workspace(
+                key[0], key[1], ws.ptr, ws.size, ws.flag.data_ptr(), ctypes.addressof(ws.launches))
     else:
         if ws.flag_word.value:
             ws.raise_if_flagged()
-        if ws.launches >= _REINIT_AFTER_LAUNCHES:
+        if ws.launches.value >= _REINIT_AFTER_LAUNCHES:
             ws.reinit(stream.cuda_stream)
-    ws.launches += 1
+    ws.launches.value += 1
     return ws
+
+
+def _slow_backward(code: int, alpha_saved: torch.Tensor, h_saved: torch.Tensor, grad_out: torch.Tensor):
+    """What the C++ dispatch calls back for a backward it does not cover."""
+    return _backward(_CODE_DTYPE[code], alpha_saved, h_saved, grad_out)
+
+
+def fast_dispatch():
+    """The C++ dispatch of the plain scan (None when switched off), knowing every workspace that
+    exists so far; later ones are registered as they are made."""
+    binding = _torch_binding.loaded()
+    if binding is None:
+        binding = _torch_binding.load(_slow_backward)
+        if binding is not None:
+            for (device, stream), ws in _workspaces.items():
+                binding.register_workspace(
+                    device, stream, ws.ptr, ws.size, ws.flag.data_ptr(), ctypes.addressof(ws.launches))
+    return binding
 
 
 def _contiguous(t: torch.Tensor) -> torch.Tensor:
@@ -224,7 +255,7 @@ def _forward(dtype: torch.dtype, alpha: torch.Tensor, beta: torch.Tensor, config
     code = _DTYPE_CODE[dtype]
     with _on(alpha.device):
         stream = _current_stream()
-        ws = _workspace(alpha.device, stream, _need("rm", code, _native.FSS_FWD, bs, seq, d, config))
+        ws = _workspace(alpha.device, stream, _need_plain(code, bs, seq, d, config))
         rc = _native.lib().fss_scan_fwd_ex(
             code, alpha.data_ptr(), beta.data_ptr(), out.data_ptr(), bs, seq, d,
             ws.ptr, ws.size, stream.cuda_stream, _native.make_config(config),
@@ -252,7 +283,7 @@ def _backward(
     code = _DTYPE_CODE[dtype]
     with _on(alpha_saved.device):
         stream = _current_stream()
-        ws = _workspace(alpha_saved.device, stream, _need("rm", code, _native.FSS_BWD, bs, seq, d, config))
+        ws = _workspace(alpha_saved.device, stream, _need_plain(code, bs, seq, d, config))
         rc = _native.lib().fss_scan_bwd_ex(
             code, alpha_saved.data_ptr(), h_saved.data_ptr(), grad_out.data_ptr(),
             grad_alpha.data_ptr(), grad_beta.data_ptr(), bs, seq, d,

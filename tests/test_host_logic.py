@@ -229,6 +229,20 @@ def test_public_names():
         pkg.scan_tr(None, None)
 
 
+def test_torch_binding_loads_and_declines_what_it_does_not_cover():
+    """No GPU here: the C++ dispatch loads, and answers None for tensors it does not take."""
+    import torch
+
+    from fast_sequential_scan_amd import sequential_scan_cuda as ext
+
+    binding = ext.fast_dispatch()
+    assert binding is not None
+    for name in ("init", "scan", "register_workspace", "forget_workspaces"):
+        assert callable(getattr(binding, name))
+    x = torch.zeros(2, 3, 4, dtype=torch.bfloat16)
+    assert binding.scan(x, x, 0) is None and binding.scan(x, x, 7) is None
+
+
 def test_missing_library_is_an_error(monkeypatch, tmp_path):
     monkeypatch.setattr(_native, "_lib", None)
     monkeypatch.setattr(_native, "LIB_PATH", str(tmp_path / "nope.so"))
