@@ -1,4 +1,4 @@
-"""Loads ``_lib/fss_torch_binding.so`` (csrc/fss_torch_binding.cpp): the C++ dispatch of the plain scan.
+"""Loads ``_lib/fss_torch_binding.so`` (csrc/fss_torch_binding.cpp): the C++ dispatch of the plain and the gated scan.
 
 The module is an accelerator of host-side dispatch only: what it launches are the kernels of
 ``libfss_scan.so`` through the same C ABI the ctypes wrappers use, and whatever it does not cover
@@ -56,8 +56,8 @@ def load(slow_backward: Callable[..., Any]) -> Optional[Any]:
         module = importlib.util.module_from_spec(spec)
         loader.exec_module(module)
         module.init(
-            _address(lib.fss_scan_fwd_ex), _address(lib.fss_scan_bwd_ex), _address(lib.fss_workspace_bytes),
-            _address(lib.fss_strerror), slow_backward,
+            _address(lib.fss_scan_fwd_ex), _address(lib.fss_scan_bwd_ex), _address(lib.fss_gated_scan_fwd),
+            _address(lib.fss_gated_scan_bwd), _address(lib.fss_workspace_bytes), _address(lib.fss_strerror), slow_backward,
         )
         _module = module
         _tried = True

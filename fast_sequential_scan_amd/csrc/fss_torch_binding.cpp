@@ -1,9 +1,10 @@
-// PyTorch-side dispatch of the plain scan in C++: what the reference's pybind11 module
+// PyTorch-side dispatch of the plain and the gated scan in C++: what the reference's pybind11 module
 // (csrc/sequential_scan.cpp:13-22: scan_forward, scan_backward, scan_forward_half,
 // scan_backward_half) and its two autograd Functions (sequential_scan/scan_cuda.py:13-62) do
 // between `scan_cu(alpha, beta)` and the kernel launch, here between the call and the C ABI of
 // libfss_scan.so.  Host code only: it allocates the outputs, looks up the stream and the chaining
-// workspace, calls fss_scan_fwd_ex / fss_scan_bwd_ex and records the autograd node.  A forward and
+// workspace, calls fss_scan_fwd_ex / fss_scan_bwd_ex (fss_gated_scan_fwd / fss_gated_scan_bwd for
+// `scan_gated`) and records the autograd node.  A forward and
 // a backward through Python Functions and ctypes cost the host 85-120 us, as much as the kernels of
 // the headline shape take and several times those of short sequences.
 //
@@ -36,18 +37,22 @@ using FwdFn = int (*)(int, const void *, const void *, void *, int64_t, int64_t,
                       const void *);
 using BwdFn = int (*)(int, const void *, const void *, const void *, void *, void *, int64_t, int64_t, int64_t,
                       void *, size_t, void *, const void *);
+using GatedBwdFn = int (*)(int, const void *, const void *, const void *, const void *, void *, void *, int64_t,
+                           int64_t, int64_t, void *, size_t, void *, const void *);
 using NeedFn = size_t (*)(int64_t, int64_t, int64_t, int, int, const void *);
 using StrerrorFn = const char *(*)(int);
 
-FwdFn g_fwd = nullptr;
+FwdFn g_fwd = nullptr, g_gated_fwd = nullptr;
 BwdFn g_bwd = nullptr;
+GatedBwdFn g_gated_bwd = nullptr;
 NeedFn g_need = nullptr;
 StrerrorFn g_strerror = nullptr;
-// (code, alpha, h, grad_out) -> [grad_alpha, grad_beta], the Python wrappers'; never destroyed (the
-// interpreter may be gone by the time statics are)
+// (kind, code, saved tensors, grad_out) -> [two gradients], the Python wrappers'; never destroyed
+// (the interpreter may be gone by the time statics are)
 py::object *g_slow_backward = nullptr;
 
-constexpr int kFwd = 0, kBwd = 1;
+// kind of scan: the `dir` values of fss_workspace_bytes for its two directions follow from it
+constexpr int kPlain = 0, kGated = 1;
 // the Python side reinitialises a workspace long before its 32-bit launch counter wraps
 constexpr int64_t kLaunchLimit = (static_cast<int64_t>(1) << 31) - 16;
 
@@ -63,18 +68,18 @@ struct Workspace {
 
 std::mutex g_lock;
 std::map<std::pair<int, uintptr_t>, Workspace> g_workspaces;
-std::map<std::tuple<int, int64_t, int64_t, int64_t>, size_t> g_needs;  // (code, bs, seq, d) -> bytes, both directions
+std::map<std::tuple<int, int, int64_t, int64_t, int64_t>, size_t> g_needs;  // (kind, code, bs, seq, d) -> bytes, both directions
 
 at::ScalarType dtype_of(int64_t code) {
   return code == 0 ? at::kBFloat16 : code == 1 ? at::kFloat : at::kHalf;
 }
 
-size_t workspace_need(int code, int64_t bs, int64_t seq, int64_t d) {
-  const auto key = std::make_tuple(code, bs, seq, d);
+size_t workspace_need(int kind, int code, int64_t bs, int64_t seq, int64_t d) {
+  const auto key = std::make_tuple(kind, code, bs, seq, d);
   std::lock_guard<std::mutex> guard(g_lock);
   auto it = g_needs.find(key);
   if (it != g_needs.end()) return it->second;
-  const size_t fwd = g_need(bs, seq, d, code, kFwd, nullptr), bwd = g_need(bs, seq, d, code, kBwd, nullptr);
+  const size_t fwd = g_need(bs, seq, d, code, 2 * kind, nullptr), bwd = g_need(bs, seq, d, code, 2 * kind + 1, nullptr);
   if (g_needs.size() > 4096) g_needs.clear();
   const size_t need = fwd > bwd ? fwd : bwd;
   g_needs[key] = need;
@@ -103,50 +108,66 @@ bool plain_tensor(const at::Tensor &t, at::ScalarType dtype) {
 }
 
 // (called with everything checked)
-at::Tensor launch_forward(const at::Tensor &alpha, const at::Tensor &beta, int code, const Workspace &ws,
+at::Tensor launch_forward(int kind, const at::Tensor &alpha, const at::Tensor &beta, int code, const Workspace &ws,
                           void *stream) {
   at::Tensor h = at::empty_like(alpha);
-  const int rc = g_fwd(code, alpha.data_ptr(), beta.data_ptr(), h.data_ptr(), alpha.size(0), alpha.size(1),
-                       alpha.size(2), ws.ptr, ws.size, stream, nullptr);
+  const int rc = (kind == kGated ? g_gated_fwd : g_fwd)(code, alpha.data_ptr(), beta.data_ptr(), h.data_ptr(),
+                                                        alpha.size(0), alpha.size(1), alpha.size(2), ws.ptr, ws.size,
+                                                        stream, nullptr);
   if (rc != 0) raise_status(rc);
   return h;
 }
 
 struct ScanNode : public torch::autograd::Function<ScanNode> {
+  // (alpha, beta) of the plain scan or (gate, x) of the gated one
   static at::Tensor forward(torch::autograd::AutogradContext *ctx, const at::Tensor &alpha, const at::Tensor &beta,
-                            int64_t code, int64_t ws_ptr, int64_t ws_size, int64_t stream) {
+                            int64_t code, int64_t kind, int64_t ws_ptr, int64_t ws_size, int64_t stream) {
     Workspace ws;
     ws.ptr = reinterpret_cast<void *>(ws_ptr);
     ws.size = static_cast<size_t>(ws_size);
-    at::Tensor h = launch_forward(alpha, beta, static_cast<int>(code), ws, reinterpret_cast<void *>(stream));
-    // (alpha, h): the output itself, no extra activation memory (reference scan_cuda.py:20,42)
-    ctx->save_for_backward({alpha, h});
+    at::Tensor h = launch_forward(static_cast<int>(kind), alpha, beta, static_cast<int>(code), ws,
+                                  reinterpret_cast<void *>(stream));
+    // (alpha, h): the output itself, no extra activation memory (reference scan_cuda.py:20,42);
+    // the gated backward also needs x
+    if (kind == kGated)
+      ctx->save_for_backward({alpha, beta, h});
+    else
+      ctx->save_for_backward({alpha, h});
     ctx->saved_data["code"] = code;
+    ctx->saved_data["kind"] = kind;
     return h;
   }
 
   static torch::autograd::variable_list backward(torch::autograd::AutogradContext *ctx,
                                                  torch::autograd::variable_list grads) {
     const auto saved = ctx->get_saved_variables();
-    const at::Tensor &alpha = saved[0], &h = saved[1];
     const int code = static_cast<int>(ctx->saved_data["code"].toInt());
+    const int kind = static_cast<int>(ctx->saved_data["kind"].toInt());
+    const at::Tensor &alpha = saved[0], &h = saved.back();
     at::Tensor dout = grads[0];
     at::Tensor grad_alpha, grad_beta;
     bool done = false;
     const at::ScalarType dtype = dtype_of(code);
-    if (dout.defined() && dout.is_cuda() && dout.scalar_type() == dtype && dout.sizes() == alpha.sizes() &&
-        dout.device() == alpha.device() && dout.layout() == at::kStrided && !at::isTensorSubclassLike(dout) &&
-        plain_tensor(alpha, dtype) && plain_tensor(h, dtype) && alpha.device().index() == c10::hip::current_device()) {
+    bool plain = dout.defined() && dout.is_cuda() && dout.scalar_type() == dtype && dout.sizes() == alpha.sizes() &&
+                 dout.device() == alpha.device() && dout.layout() == at::kStrided && !at::isTensorSubclassLike(dout) &&
+                 alpha.device().index() == c10::hip::current_device();
+    for (const auto &t : saved) plain = plain && plain_tensor(t, dtype);
+    if (plain) {
       const int device = alpha.device().index();
       void *stream = c10::hip::getCurrentHIPStream(static_cast<c10::DeviceIndex>(device)).stream();
       Workspace ws;
-      if (usable_workspace(device, stream, workspace_need(code, alpha.size(0), alpha.size(1), alpha.size(2)), ws)) {
+      if (usable_workspace(device, stream, workspace_need(kind, code, alpha.size(0), alpha.size(1), alpha.size(2)), ws)) {
         if (!dout.is_contiguous()) dout = dout.contiguous();
         grad_alpha = at::empty_like(alpha);
         grad_beta = at::empty_like(alpha);
-        const int rc = g_bwd(code, alpha.data_ptr(), h.data_ptr(), dout.data_ptr(), grad_alpha.data_ptr(),
-                             grad_beta.data_ptr(), alpha.size(0), alpha.size(1), alpha.size(2), ws.ptr, ws.size,
-                             stream, nullptr);
+        const int rc =
+            kind == kGated
+                ? g_gated_bwd(code, alpha.data_ptr(), saved[1].data_ptr(), h.data_ptr(), dout.data_ptr(),
+                              grad_alpha.data_ptr(), grad_beta.data_ptr(), alpha.size(0), alpha.size(1), alpha.size(2),
+                              ws.ptr, ws.size, stream, nullptr)
+                : g_bwd(code, alpha.data_ptr(), h.data_ptr(), dout.data_ptr(), grad_alpha.data_ptr(),
+                        grad_beta.data_ptr(), alpha.size(0), alpha.size(1), alpha.size(2), ws.ptr, ws.size, stream,
+                        nullptr);
         if (rc != 0) raise_status(rc);
         done = true;
       }
@@ -154,7 +175,7 @@ struct ScanNode : public torch::autograd::Function<ScanNode> {
     if (!done) {
       py::gil_scoped_acquire gil;
       TORCH_CHECK(g_slow_backward != nullptr, "fss_torch_binding.init was not called");
-      py::object result = (*g_slow_backward)(code, alpha, h, dout);
+      py::object result = (*g_slow_backward)(kind, code, std::vector<at::Tensor>(saved.begin(), saved.end()), dout);
       auto pair = result.cast<std::vector<at::Tensor>>();
       TORCH_CHECK(pair.size() == 2, "the Python backward returned ", pair.size(), " tensors");
       grad_alpha = pair[0];
@@ -173,18 +194,18 @@ struct ScanNode : public torch::autograd::Function<ScanNode> {
           "trying to differentiate twice a function that was marked with @once_differentiable", 2);
       out = (*err)(std::move(out));
     }
-    out.emplace_back();
-    out.emplace_back();
-    out.emplace_back();
-    out.emplace_back();
+    out.resize(7);  // nothing for code, kind, workspace and stream
     return out;
   }
 };
 
-void init(uintptr_t fwd, uintptr_t bwd, uintptr_t need, uintptr_t strerror_fn, py::object slow_backward) {
+void init(uintptr_t fwd, uintptr_t bwd, uintptr_t gated_fwd, uintptr_t gated_bwd, uintptr_t need, uintptr_t strerror_fn,
+          py::object slow_backward) {
   std::lock_guard<std::mutex> guard(g_lock);
   g_fwd = reinterpret_cast<FwdFn>(fwd);
   g_bwd = reinterpret_cast<BwdFn>(bwd);
+  g_gated_fwd = reinterpret_cast<FwdFn>(gated_fwd);
+  g_gated_bwd = reinterpret_cast<GatedBwdFn>(gated_bwd);
   g_need = reinterpret_cast<NeedFn>(need);
   g_strerror = reinterpret_cast<StrerrorFn>(strerror_fn);
   g_slow_backward = new py::object(std::move(slow_backward));
@@ -207,8 +228,9 @@ void forget_workspaces() {
 }
 
 // h of the scan, recorded for autograd when an input asks for it; None when this path does not
-// cover the call.  `code`: 0 bf16, 1 fp32, 2 fp16 (FSS_BF16, FSS_F32, FSS_F16).
-std::optional<at::Tensor> scan(const at::Tensor &alpha, const at::Tensor &beta, int64_t code) {
+// cover the call.  `code`: 0 bf16, 1 fp32, 2 fp16 (FSS_BF16, FSS_F32, FSS_F16); `kind`: 0 the plain
+// scan of (alpha, beta), 1 the gated scan of (gate, x).
+std::optional<at::Tensor> dispatch(const at::Tensor &alpha, const at::Tensor &beta, int64_t code, int kind) {
   if (!g_fwd || code < 0 || code > 2) return std::nullopt;
   const at::ScalarType dtype = dtype_of(code);
   if (!plain_tensor(alpha, dtype) || !plain_tensor(beta, dtype)) return std::nullopt;
@@ -218,20 +240,37 @@ std::optional<at::Tensor> scan(const at::Tensor &alpha, const at::Tensor &beta, 
   if (device != c10::hip::current_device()) return std::nullopt;
   void *stream = c10::hip::getCurrentHIPStream(static_cast<c10::DeviceIndex>(device)).stream();
   Workspace ws;
-  if (!usable_workspace(device, stream, workspace_need(static_cast<int>(code), alpha.size(0), alpha.size(1), alpha.size(2)), ws))
+  if (!usable_workspace(device, stream,
+                        workspace_need(kind, static_cast<int>(code), alpha.size(0), alpha.size(1), alpha.size(2)), ws))
     return std::nullopt;
   if (at::GradMode::is_enabled() && (alpha.requires_grad() || beta.requires_grad()))
-    return ScanNode::apply(alpha, beta, code, static_cast<int64_t>(reinterpret_cast<uintptr_t>(ws.ptr)),
-                           static_cast<int64_t>(ws.size), static_cast<int64_t>(reinterpret_cast<uintptr_t>(stream)));
-  return launch_forward(alpha, beta, static_cast<int>(code), ws, stream);
+    return ScanNode::apply(alpha, beta, code, static_cast<int64_t>(kind),
+                           static_cast<int64_t>(reinterpret_cast<uintptr_t>(ws.ptr)), static_cast<int64_t>(ws.size),
+                           static_cast<int64_t>(reinterpret_cast<uintptr_t>(stream)));
+  return launch_forward(kind, alpha, beta, static_cast<int>(code), ws, stream);
+}
+
+std::optional<at::Tensor> scan(const at::Tensor &alpha, const at::Tensor &beta, int64_t code) {
+  return dispatch(alpha, beta, code, kPlain);
+}
+
+// (the storage type is the gate's: bf16, fp32 or fp16)
+std::optional<at::Tensor> scan_gated(const at::Tensor &gate, const at::Tensor &x) {
+  if (!gate.defined()) return std::nullopt;
+  const at::ScalarType t = gate.scalar_type();
+  const int64_t code = t == at::kBFloat16 ? 0 : t == at::kFloat ? 1 : t == at::kHalf ? 2 : -1;
+  return dispatch(gate, x, code, kGated);
 }
 
 }  // namespace
 
 PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
   m.doc() = "C++ dispatch of the plain scan over the C ABI of libfss_scan.so";
-  m.def("init", &init, "addresses of fss_scan_fwd_ex, fss_scan_bwd_ex, fss_workspace_bytes, fss_strerror; the Python backward");
+  m.def("init", &init,
+        "addresses of fss_scan_fwd_ex, fss_scan_bwd_ex, fss_gated_scan_fwd, fss_gated_scan_bwd, fss_workspace_bytes, "
+        "fss_strerror; the Python backward");
   m.def("register_workspace", &register_workspace, "device, stream, pointer, bytes, address of the flag word, address of the launch count");
   m.def("forget_workspaces", &forget_workspaces);
   m.def("scan", &scan, "h, or None when the call is not the common case");
+  m.def("scan_gated", &scan_gated, "h of the gated scan, or None when the call is not the common case");
 }

@@ -82,6 +82,7 @@ class SequentialScanSingle(Function):
 # answers None for anything else, which then goes through the Functions above, as do all errors.
 _UNRESOLVED = object()
 _fast: Any = _UNRESOLVED
+_fast_gated: Any = _UNRESOLVED
 
 
 def _fast_scan(alpha: torch.Tensor, beta: torch.Tensor, code: int) -> Optional[torch.Tensor]:
@@ -185,6 +186,14 @@ class SequentialScanGated(Function):
 def scan_gated(gate: torch.Tensor, x: torch.Tensor) -> torch.Tensor:
     """The Hawk / RG-LRU style gated recurrence from its pre-activations:
     ``a = sigmoid(gate)``, ``h[t] = a[t]*h[t-1] + sqrt(1 - a[t]**2) * x[t]``."""
+    global _fast_gated
+    if _fast_gated is _UNRESOLVED:
+        binding = _ext.fast_dispatch()
+        _fast_gated = binding.scan_gated if binding is not None else None
+    if _fast_gated is not None and isinstance(gate, torch.Tensor) and isinstance(x, torch.Tensor):
+        h = _fast_gated(gate, x)
+        if h is not None:
+            return h
     return SequentialScanGated.apply(gate, x)
 
 

@@ -155,6 +155,12 @@ def _need_plain(code: int, bs: int, seq: int, d: int, config) -> int:
                _need("rm", code, _native.FSS_BWD, bs, seq, d, config))
 
 
+def _need_gated(code: int, bs: int, seq: int, d: int, config) -> int:
+    """The same for the gated scan."""
+    return max(_need("rm", code, _native.FSS_GATED_FWD, bs, seq, d, config),
+               _need("rm", code, _native.FSS_GATED_BWD, bs, seq, d, config))
+
+
 def _workspace(device: torch.device, stream: "_RawStream", need: int) -> "_Workspace":
     """The workspace of (device, stream), grown to `need` bytes; raises if a scan launched through
     it earlier reported a chain time-out."""
@@ -178,13 +184,16 @@ def _workspace(device: torch.device, stream: "_RawStream", need: int) -> "_Works
     return ws
 
 
-def _slow_backward(code: int, alpha_saved: torch.Tensor, h_saved: torch.Tensor, grad_out: torch.Tensor):
-    """What the C++ dispatch calls back for a backward it does not cover."""
-    return _backward(_CODE_DTYPE[code], alpha_saved, h_saved, grad_out)
+def _slow_backward(kind: int, code: int, saved: List[torch.Tensor], grad_out: torch.Tensor):
+    """What the C++ dispatch calls back for a backward it does not cover (kind 0: the plain scan,
+    saved (alpha, h); kind 1: the gated scan, saved (gate, x, h))."""
+    if kind == 1:
+        return gated_scan_backward(saved[0], saved[1], saved[2], grad_out)
+    return _backward(_CODE_DTYPE[code], saved[0], saved[1], grad_out)
 
 
 def fast_dispatch():
-    """The C++ dispatch of the plain scan (None when switched off), knowing every workspace that
+    """The C++ dispatch of the plain and the gated scan (None when switched off), knowing every workspace that
     exists so far; later ones are registered as they are made."""
     binding = _torch_binding.loaded()
     if binding is None:
@@ -443,7 +452,7 @@ def gated_scan_forward(gate: torch.Tensor, x: torch.Tensor, config=None) -> torc
     cfg = _native.make_config(config)
     with _on(gate.device):
         stream = _current_stream()
-        ws = _workspace(gate.device, stream, _need("rm", code, _native.FSS_GATED_FWD, bs, seq, d, config))
+        ws = _workspace(gate.device, stream, _need_gated(code, bs, seq, d, config))
         _native.check(
             lib.fss_gated_scan_fwd(
                 code, gate.data_ptr(), x.data_ptr(), out.data_ptr(), bs, seq, d,
@@ -469,7 +478,7 @@ def gated_scan_backward(
     cfg = _native.make_config(config)
     with _on(gate.device):
         stream = _current_stream()
-        ws = _workspace(gate.device, stream, _need("rm", code, _native.FSS_GATED_BWD, bs, seq, d, config))
+        ws = _workspace(gate.device, stream, _need_gated(code, bs, seq, d, config))
         _native.check(
             lib.fss_gated_scan_bwd(
                 code, gate.data_ptr(), x.data_ptr(), h_saved.data_ptr(), grad_out.data_ptr(),
@@ -500,7 +509,7 @@ def gated_scan_forward_state(
     cfg = _native.make_config(config)
     with _on(gate.device):
         stream = _current_stream()
-        ws = _workspace(gate.device, stream, _need("rm", code, _native.FSS_GATED_FWD, bs, seq, d, config))
+        ws = _workspace(gate.device, stream, _need_gated(code, bs, seq, d, config))
         _native.check(
             lib.fss_gated_scan_fwd_state(
                 code, gate.data_ptr(), x.data_ptr(), out.data_ptr(),
@@ -538,7 +547,7 @@ def gated_scan_backward_state(
     cfg = _native.make_config(config)
     with _on(gate.device):
         stream = _current_stream()
-        ws = _workspace(gate.device, stream, _need("rm", code, _native.FSS_GATED_BWD, bs, seq, d, config))
+        ws = _workspace(gate.device, stream, _need_gated(code, bs, seq, d, config))
         _native.check(
             lib.fss_gated_scan_bwd_state(
                 code, gate.data_ptr(), x.data_ptr(), h_saved.data_ptr(), grad_out.data_ptr(),

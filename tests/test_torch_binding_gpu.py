@@ -9,6 +9,7 @@ pytestmark = pytest.mark.gpu
 
 from fast_sequential_scan_amd import scan_cu, scan_cu_single  # noqa: E402
 from fast_sequential_scan_amd import scan_cu_fp16 as scan_fp16  # noqa: E402
+from fast_sequential_scan_amd import scan_gated  # noqa: E402
 from fast_sequential_scan_amd import scan_cuda  # noqa: E402
 from fast_sequential_scan_amd import sequential_scan_cuda as ext  # noqa: E402
 from fast_sequential_scan_amd.workloads import make_inputs  # noqa: E402
@@ -119,4 +120,33 @@ def test_other_streams_get_their_own_workspace_and_node():
     side.synchronize()
     ga, _ = ext.scan_backward_half(alpha, want, dout)
     assert torch.equal(first, want) and torch.equal(out, want) and torch.equal(a.grad, ga)
+    ext.workspace_status()
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32], ids=["bf16", "f32"])
+@pytest.mark.parametrize("shape", [(2, 1000, 768), (3, 37, 64), (1, 5000, 130)])
+def test_gated_scan_same_bits_as_the_python_function(dtype, shape):
+    g = torch.Generator().manual_seed(sum(shape))
+    gate = (1.5 * torch.randn(shape, generator=g)).to(dtype).to(DEV)
+    x, dout = (torch.randn(shape, generator=g).to(dtype).to(DEV) for _ in range(2))
+    g1, x1 = gate.clone().requires_grad_(True), x.clone().requires_grad_(True)
+    want = scan_cuda.SequentialScanGated.apply(g1, x1)
+    want.backward(dout)
+    g2, x2 = gate.clone().requires_grad_(True), x.clone().requires_grad_(True)
+    got = scan_gated(g2, x2)
+    assert "ScanNode" in _node_name(got), _node_name(got)
+    got.backward(dout)
+    ext.workspace_status()
+    assert torch.equal(got, want) and torch.equal(g2.grad, g1.grad) and torch.equal(x2.grad, x1.grad)
+    with torch.no_grad():
+        assert torch.equal(scan_gated(g2, x2), want)
+    # what it does not cover: a non-contiguous gate, a gradient that arrives transposed
+    g_t = gate.transpose(1, 2).contiguous().transpose(1, 2).requires_grad_(True)
+    out = scan_gated(g_t, x)
+    assert "ScanNode" not in _node_name(out) and torch.equal(out, want)
+    g3, x3 = gate.clone().requires_grad_(True), x.clone().requires_grad_(True)
+    scan_gated(g3, x3).transpose(1, 2).backward(dout.transpose(1, 2).contiguous())
+    assert torch.equal(g3.grad, g1.grad) and torch.equal(x3.grad, x1.grad)
+    with pytest.raises(RuntimeError):
+        scan_gated(gate, x[:, :10])
     ext.workspace_status()
