@@ -57,7 +57,8 @@ def load(slow_backward: Callable[..., Any]) -> Optional[Any]:
         loader.exec_module(module)
         module.init(
             _address(lib.fss_scan_fwd_ex), _address(lib.fss_scan_bwd_ex), _address(lib.fss_gated_scan_fwd),
-            _address(lib.fss_gated_scan_bwd), _address(lib.fss_workspace_bytes), _address(lib.fss_strerror), slow_backward,
+            _address(lib.fss_gated_scan_bwd), _address(lib.fss_scan_fwd_state), _address(lib.fss_workspace_bytes),
+            _address(lib.fss_strerror), slow_backward,
         )
         _module = module
         _tried = True

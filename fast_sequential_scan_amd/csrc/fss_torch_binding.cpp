@@ -39,12 +39,15 @@ using BwdFn = int (*)(int, const void *, const void *, const void *, void *, voi
                       void *, size_t, void *, const void *);
 using GatedBwdFn = int (*)(int, const void *, const void *, const void *, const void *, void *, void *, int64_t,
                            int64_t, int64_t, void *, size_t, void *, const void *);
+using StateFwdFn = int (*)(int, const void *, const void *, void *, const void *, void *, int64_t, int64_t, int64_t,
+                           void *, size_t, void *, const void *);
 using NeedFn = size_t (*)(int64_t, int64_t, int64_t, int, int, const void *);
 using StrerrorFn = const char *(*)(int);
 
 FwdFn g_fwd = nullptr, g_gated_fwd = nullptr;
 BwdFn g_bwd = nullptr;
 GatedBwdFn g_gated_bwd = nullptr;
+StateFwdFn g_state_fwd = nullptr;
 NeedFn g_need = nullptr;
 StrerrorFn g_strerror = nullptr;
 // (kind, code, saved tensors, grad_out) -> [two gradients], the Python wrappers'; never destroyed
@@ -199,13 +202,14 @@ struct ScanNode : public torch::autograd::Function<ScanNode> {
   }
 };
 
-void init(uintptr_t fwd, uintptr_t bwd, uintptr_t gated_fwd, uintptr_t gated_bwd, uintptr_t need, uintptr_t strerror_fn,
-          py::object slow_backward) {
+void init(uintptr_t fwd, uintptr_t bwd, uintptr_t gated_fwd, uintptr_t gated_bwd, uintptr_t state_fwd, uintptr_t need,
+          uintptr_t strerror_fn, py::object slow_backward) {
   std::lock_guard<std::mutex> guard(g_lock);
   g_fwd = reinterpret_cast<FwdFn>(fwd);
   g_bwd = reinterpret_cast<BwdFn>(bwd);
   g_gated_fwd = reinterpret_cast<FwdFn>(gated_fwd);
   g_gated_bwd = reinterpret_cast<GatedBwdFn>(gated_bwd);
+  g_state_fwd = reinterpret_cast<StateFwdFn>(state_fwd);
   g_need = reinterpret_cast<NeedFn>(need);
   g_strerror = reinterpret_cast<StrerrorFn>(strerror_fn);
   g_slow_backward = new py::object(std::move(slow_backward));
@@ -262,15 +266,54 @@ std::optional<at::Tensor> scan_gated(const at::Tensor &gate, const at::Tensor &x
   return dispatch(gate, x, code, kGated);
 }
 
+// (h, h_last) of the scan that starts from the fp32 state `h_before` (bs, d) - zeros when absent -
+// for calls that need no gradient: the step of a streaming decode loop, where the sequence is a
+// few tokens and the host's time is all there is.  None for anything else.
+std::optional<std::tuple<at::Tensor, at::Tensor>> scan_state(const at::Tensor &alpha, const at::Tensor &beta,
+                                                             const std::optional<at::Tensor> &h_before) {
+  if (!g_state_fwd || !alpha.defined()) return std::nullopt;
+  const at::ScalarType t = alpha.scalar_type();
+  const int code = t == at::kBFloat16 ? 0 : t == at::kFloat ? 1 : t == at::kHalf ? 2 : -1;
+  if (code < 0 || !plain_tensor(alpha, t) || !plain_tensor(beta, t)) return std::nullopt;
+  if (alpha.sizes() != beta.sizes() || alpha.device() != beta.device() || alpha.numel() == 0) return std::nullopt;
+  const bool with_state = h_before.has_value() && h_before->defined();
+  if (with_state) {
+    const at::Tensor &h0 = *h_before;
+    if (!h0.is_cuda() || h0.scalar_type() != at::kFloat || h0.dim() != 2 || h0.size(0) != alpha.size(0) ||
+        h0.size(1) != alpha.size(2) || !h0.is_contiguous() || h0.device() != alpha.device() ||
+        at::isTensorSubclassLike(h0))
+      return std::nullopt;
+  }
+  if (at::GradMode::is_enabled() &&
+      (alpha.requires_grad() || beta.requires_grad() || (with_state && h_before->requires_grad())))
+    return std::nullopt;
+  if (at::autocast::is_autocast_enabled(at::kCUDA)) return std::nullopt;
+  const int device = alpha.device().index();
+  if (device != c10::hip::current_device()) return std::nullopt;
+  void *stream = c10::hip::getCurrentHIPStream(static_cast<c10::DeviceIndex>(device)).stream();
+  Workspace ws;
+  if (!usable_workspace(device, stream, workspace_need(kPlain, code, alpha.size(0), alpha.size(1), alpha.size(2)), ws))
+    return std::nullopt;
+  at::Tensor h = at::empty_like(alpha);
+  at::Tensor h_last = at::zeros({alpha.size(0), alpha.size(2)}, alpha.options().dtype(at::kFloat));
+  const int rc = g_state_fwd(code, alpha.data_ptr(), beta.data_ptr(), h.data_ptr(),
+                             with_state ? h_before->data_ptr() : nullptr, h_last.data_ptr(), alpha.size(0),
+                             alpha.size(1), alpha.size(2), ws.ptr, ws.size, stream, nullptr);
+  if (rc != 0) raise_status(rc);
+  return std::make_tuple(h, h_last);
+}
+
 }  // namespace
 
 PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
   m.doc() = "C++ dispatch of the plain scan over the C ABI of libfss_scan.so";
   m.def("init", &init,
-        "addresses of fss_scan_fwd_ex, fss_scan_bwd_ex, fss_gated_scan_fwd, fss_gated_scan_bwd, fss_workspace_bytes, "
-        "fss_strerror; the Python backward");
+        "addresses of fss_scan_fwd_ex, fss_scan_bwd_ex, fss_gated_scan_fwd, fss_gated_scan_bwd, fss_scan_fwd_state, "
+        "fss_workspace_bytes, fss_strerror; the Python backward");
   m.def("register_workspace", &register_workspace, "device, stream, pointer, bytes, address of the flag word, address of the launch count");
   m.def("forget_workspaces", &forget_workspaces);
   m.def("scan", &scan, "h, or None when the call is not the common case");
   m.def("scan_gated", &scan_gated, "h of the gated scan, or None when the call is not the common case");
+  m.def("scan_state", &scan_state, py::arg("alpha"), py::arg("beta"), py::arg("h_before") = py::none(),
+        "(h, h_last) without gradients, or None when the call is not the common case");
 }

@@ -83,6 +83,7 @@ class SequentialScanSingle(Function):
 _UNRESOLVED = object()
 _fast: Any = _UNRESOLVED
 _fast_gated: Any = _UNRESOLVED
+_fast_state: Any = _UNRESOLVED
 
 
 def _fast_scan(alpha: torch.Tensor, beta: torch.Tensor, code: int) -> Optional[torch.Tensor]:
@@ -162,6 +163,16 @@ def scan_with_state(
     """``h[t] = alpha[t]*h[t-1] + beta[t]`` from ``h[-1] = h_before`` (zeros when None; when given,
     ``alpha[:, 0]`` multiplies it).  Returns ``(h, h_last)`` with ``h_last`` the fp32 state after the
     last step, to be passed as ``h_before`` of the next segment."""
+    global _fast_state
+    if _fast_state is _UNRESOLVED:
+        binding = _ext.fast_dispatch()
+        _fast_state = binding.scan_state if binding is not None else None
+    # (without gradients - the step of a decode loop - the C++ dispatch takes the common call)
+    if (_fast_state is not None and isinstance(alpha, torch.Tensor) and isinstance(beta, torch.Tensor)
+            and (h_before is None or isinstance(h_before, torch.Tensor))):
+        pair = _fast_state(alpha, beta, h_before)
+        if pair is not None:
+            return pair
     return SequentialScanState.apply(alpha, beta, h_before)
 
 

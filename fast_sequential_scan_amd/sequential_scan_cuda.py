@@ -377,7 +377,7 @@ def scan_forward_state(
     code = _DTYPE_CODE[dtype]
     with _on(alpha.device):
         stream = _current_stream()
-        ws = _workspace(alpha.device, stream, _need("rm", code, _native.FSS_FWD, bs, seq, d, config))
+        ws = _workspace(alpha.device, stream, _need_plain(code, bs, seq, d, config))
         _native.check(
             lib.fss_scan_fwd_state(
                 code, alpha.data_ptr(), beta.data_ptr(), out.data_ptr(),
@@ -415,7 +415,7 @@ def scan_backward_state(
     code = _DTYPE_CODE[dtype]
     with _on(alpha_saved.device):
         stream = _current_stream()
-        ws = _workspace(alpha_saved.device, stream, _need("rm", code, _native.FSS_BWD, bs, seq, d, config))
+        ws = _workspace(alpha_saved.device, stream, _need_plain(code, bs, seq, d, config))
         _native.check(
             lib.fss_scan_bwd_state(
                 code, alpha_saved.data_ptr(), h_saved.data_ptr(), grad_out.data_ptr(),

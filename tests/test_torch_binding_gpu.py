@@ -9,7 +9,7 @@ pytestmark = pytest.mark.gpu
 
 from fast_sequential_scan_amd import scan_cu, scan_cu_single  # noqa: E402
 from fast_sequential_scan_amd import scan_cu_fp16 as scan_fp16  # noqa: E402
-from fast_sequential_scan_amd import scan_gated  # noqa: E402
+from fast_sequential_scan_amd import scan_gated, scan_with_state  # noqa: E402
 from fast_sequential_scan_amd import scan_cuda  # noqa: E402
 from fast_sequential_scan_amd import sequential_scan_cuda as ext  # noqa: E402
 from fast_sequential_scan_amd.workloads import make_inputs  # noqa: E402
@@ -150,3 +150,42 @@ def test_gated_scan_same_bits_as_the_python_function(dtype, shape):
     with pytest.raises(RuntimeError):
         scan_gated(gate, x[:, :10])
     ext.workspace_status()
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32], ids=["bf16", "f32"])
+def test_decode_loop_through_the_state_dispatch(dtype):
+    """Segments of 1, 3 and 700 steps chained through (h, h_last) without gradients - through the C++
+    dispatch from the second call on - reproduce the Python Function's outputs bit for bit and, in
+    fp32, the scan of the whole sequence."""
+    bs, seq, d = 3, 1200, 192
+    alpha, beta, _ = _tensors((bs, seq, d), dtype, seed=12)
+    binding = ext.fast_dispatch()
+    cuts = [0, 1, 4, 5, 500, 1200]
+    with torch.no_grad():
+        state = None
+        pieces, states = [], []
+        for lo, hi in zip(cuts[:-1], cuts[1:]):
+            a, b = alpha[:, lo:hi].contiguous(), beta[:, lo:hi].contiguous()
+            want_h, want_state = scan_cuda.SequentialScanState.apply(a, b, state)
+            if lo > 0:
+                assert binding.scan_state(a, b, state) is not None, "the C++ dispatch declined a plain call"
+            h, new_state = scan_with_state(a, b, state)
+            assert torch.equal(h, want_h) and torch.equal(new_state, want_state)
+            pieces.append(h)
+            states.append(new_state)
+            state = new_state
+        whole, whole_state = scan_with_state(alpha, beta)
+    ext.workspace_status()
+    if dtype == torch.float32:
+        torch.testing.assert_close(torch.cat(pieces, dim=1), whole, rtol=1e-5, atol=1e-6)
+        torch.testing.assert_close(states[-1], whole_state, rtol=1e-5, atol=1e-6)
+    # with gradients the call goes through the Python Function
+    a = alpha[:, :50].contiguous().requires_grad_(True)
+    h, last = scan_with_state(a, beta[:, :50].contiguous())
+    assert h.grad_fn is not None and "ScanNode" not in _node_name(h)
+    assert binding.scan_state(a, beta[:, :50].contiguous(), None) is None
+    # what it declines: a state of the wrong type or shape (the wrappers raise)
+    with pytest.raises(RuntimeError):
+        scan_with_state(alpha, beta, torch.zeros(bs, d, device=DEV, dtype=torch.float64))
+    with pytest.raises(RuntimeError):
+        scan_with_state(alpha, beta, torch.zeros(bs, d + 1, device=DEV))
