@@ -295,7 +295,8 @@ std::optional<std::tuple<at::Tensor, at::Tensor>> scan_state(const at::Tensor &a
   if (!usable_workspace(device, stream, workspace_need(kPlain, code, alpha.size(0), alpha.size(1), alpha.size(2)), ws))
     return std::nullopt;
   at::Tensor h = at::empty_like(alpha);
-  at::Tensor h_last = at::zeros({alpha.size(0), alpha.size(2)}, alpha.options().dtype(at::kFloat));
+  // (every channel's entry is written by the wave that holds the sequence's last step)
+  at::Tensor h_last = at::empty({alpha.size(0), alpha.size(2)}, alpha.options().dtype(at::kFloat));
   const int rc = g_state_fwd(code, alpha.data_ptr(), beta.data_ptr(), h.data_ptr(),
                              with_state ? h_before->data_ptr() : nullptr, h_last.data_ptr(), alpha.size(0),
                              alpha.size(1), alpha.size(2), ws.ptr, ws.size, stream, nullptr);

@@ -368,11 +368,13 @@ def scan_forward_state(
     h_before = _state("h_before", h_before, alpha)
     alpha, beta = alpha.contiguous(), beta.contiguous()
     out = torch.empty_like(alpha, memory_format=torch.contiguous_format)
-    h_last = torch.zeros((bs, d), dtype=torch.float32, device=alpha.device)
     if out.numel() == 0:
+        h_last = torch.zeros((bs, d), dtype=torch.float32, device=alpha.device)
         if h_before is not None and seq == 0:
             h_last.copy_(h_before)
         return out, h_last
+    # (every channel's entry is written by the wave that holds the sequence's last step)
+    h_last = torch.empty((bs, d), dtype=torch.float32, device=alpha.device)
     lib = _native.lib()
     code = _DTYPE_CODE[dtype]
     with _on(alpha.device):
