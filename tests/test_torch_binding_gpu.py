@@ -189,3 +189,37 @@ def test_decode_loop_through_the_state_dispatch(dtype):
         scan_with_state(alpha, beta, torch.zeros(bs, d, device=DEV, dtype=torch.float64))
     with pytest.raises(RuntimeError):
         scan_with_state(alpha, beta, torch.zeros(bs, d + 1, device=DEV))
+
+
+def test_captured_decode_step_replays_match_eager():
+    """A decode step through the public API - ``scan_with_state`` without gradients, which the C++
+    dispatch takes - captured as a HIP graph: every replay (with eager scans and synchronisations in
+    between) gives what the eager call gives.  The state is carried in a tensor the graph updates in place."""
+    bs, seq, d = 4, 2000, 256  # several chunks: the chaining workspace is in play
+    alpha, beta, _ = _tensors((bs, seq, d), torch.bfloat16, seed=21)
+    binding = ext.fast_dispatch()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side), torch.no_grad():
+        state = torch.zeros(bs, d, device=DEV)
+        scan_with_state(alpha, beta, state)  # warm: the stream's workspace, device check, residency query
+        assert binding.scan_state(alpha, beta, state) is not None
+        side.synchronize()
+        want = []
+        s = state.clone()
+        for _ in range(4):
+            h, s = scan_with_state(alpha, beta, s)
+            want.append((h.clone(), s.clone()))
+        side.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph, stream=side):
+            h_out, s_out = scan_with_state(alpha, beta, state)
+            state.copy_(s_out)
+        state.zero_()
+        for i in range(4):
+            graph.replay()
+            side.synchronize()
+            assert torch.equal(h_out, want[i][0]) and torch.equal(state, want[i][1]), i
+            scan_with_state(alpha, beta, torch.ones(bs, d, device=DEV))  # eager work between replays, same workspace
+            side.synchronize()
+    ext.workspace_status()
