@@ -1,4 +1,4 @@
-"""Loads ``_lib/fss_torch_binding.so`` (csrc/fss_torch_binding.cpp): the C++ dispatch of the plain and the gated scan.
+"""Loads ``_lib/fss_torch_binding.so`` (csrc/fss_torch_binding.cpp): the C++ dispatch of the plain, the gated and the channel-major scan.
 
 The module is an accelerator of host-side dispatch only: what it launches are the kernels of
 ``libfss_scan.so`` through the same C ABI the ctypes wrappers use, and whatever it does not cover
@@ -57,7 +57,8 @@ def load(slow_backward: Callable[..., Any]) -> Optional[Any]:
         loader.exec_module(module)
         module.init(
             _address(lib.fss_scan_fwd_ex), _address(lib.fss_scan_bwd_ex), _address(lib.fss_gated_scan_fwd),
-            _address(lib.fss_gated_scan_bwd), _address(lib.fss_scan_fwd_state), _address(lib.fss_workspace_bytes),
+            _address(lib.fss_gated_scan_bwd), _address(lib.fss_scan_fwd_state), _address(lib.fss_scan_fwd_cm),
+            _address(lib.fss_scan_bwd_cm), _address(lib.fss_workspace_bytes), _address(lib.fss_cm_workspace_bytes),
             _address(lib.fss_strerror), slow_backward,
         )
         _module = module

@@ -1,10 +1,10 @@
-// PyTorch-side dispatch of the plain and the gated scan in C++: what the reference's pybind11 module
+// PyTorch-side dispatch of the plain, the gated and the channel-major scan in C++: what the reference's pybind11 module
 // (csrc/sequential_scan.cpp:13-22: scan_forward, scan_backward, scan_forward_half,
 // scan_backward_half) and its two autograd Functions (sequential_scan/scan_cuda.py:13-62) do
 // between `scan_cu(alpha, beta)` and the kernel launch, here between the call and the C ABI of
 // libfss_scan.so.  Host code only: it allocates the outputs, looks up the stream and the chaining
 // workspace, calls fss_scan_fwd_ex / fss_scan_bwd_ex (fss_gated_scan_fwd / fss_gated_scan_bwd for
-// `scan_gated`) and records the autograd node.  A forward and
+// `scan_gated`, fss_scan_fwd_cm / fss_scan_bwd_cm for `scan_cm`) and records the autograd node.  A forward and
 // a backward through Python Functions and ctypes cost the host 85-120 us, as much as the kernels of
 // the headline shape take and several times those of short sequences.
 //
@@ -44,18 +44,19 @@ using StateFwdFn = int (*)(int, const void *, const void *, void *, const void *
 using NeedFn = size_t (*)(int64_t, int64_t, int64_t, int, int, const void *);
 using StrerrorFn = const char *(*)(int);
 
-FwdFn g_fwd = nullptr, g_gated_fwd = nullptr;
-BwdFn g_bwd = nullptr;
+FwdFn g_fwd = nullptr, g_gated_fwd = nullptr, g_cm_fwd = nullptr;
+BwdFn g_bwd = nullptr, g_cm_bwd = nullptr;
 GatedBwdFn g_gated_bwd = nullptr;
 StateFwdFn g_state_fwd = nullptr;
-NeedFn g_need = nullptr;
+NeedFn g_need = nullptr, g_cm_need = nullptr;
 StrerrorFn g_strerror = nullptr;
 // (kind, code, saved tensors, grad_out) -> [two gradients], the Python wrappers'; never destroyed
 // (the interpreter may be gone by the time statics are)
 py::object *g_slow_backward = nullptr;
 
-// kind of scan: the `dir` values of fss_workspace_bytes for its two directions follow from it
-constexpr int kPlain = 0, kGated = 1;
+// kind of scan.  Plain and gated: (bs, seq, d) tensors, the `dir` values of fss_workspace_bytes for the
+// two directions are 2*kind and 2*kind+1.  Channel-major: (bs, d, seq) tensors, fss_cm_workspace_bytes.
+constexpr int kPlain = 0, kGated = 1, kChannelMajor = 2;
 // the Python side reinitialises a workspace long before its 32-bit launch counter wraps
 constexpr int64_t kLaunchLimit = (static_cast<int64_t>(1) << 31) - 16;
 
@@ -82,7 +83,9 @@ size_t workspace_need(int kind, int code, int64_t bs, int64_t seq, int64_t d) {
   std::lock_guard<std::mutex> guard(g_lock);
   auto it = g_needs.find(key);
   if (it != g_needs.end()) return it->second;
-  const size_t fwd = g_need(bs, seq, d, code, 2 * kind, nullptr), bwd = g_need(bs, seq, d, code, 2 * kind + 1, nullptr);
+  // (bs, seq, d) are the tensor's three sizes in order: (bs, d, seq) for the channel-major kind
+  const size_t fwd = kind == kChannelMajor ? g_cm_need(bs, seq, d, code, 0, nullptr) : g_need(bs, seq, d, code, 2 * kind, nullptr);
+  const size_t bwd = kind == kChannelMajor ? g_cm_need(bs, seq, d, code, 1, nullptr) : g_need(bs, seq, d, code, 2 * kind + 1, nullptr);
   if (g_needs.size() > 4096) g_needs.clear();
   const size_t need = fwd > bwd ? fwd : bwd;
   g_needs[key] = need;
@@ -114,7 +117,7 @@ bool plain_tensor(const at::Tensor &t, at::ScalarType dtype) {
 at::Tensor launch_forward(int kind, const at::Tensor &alpha, const at::Tensor &beta, int code, const Workspace &ws,
                           void *stream) {
   at::Tensor h = at::empty_like(alpha);
-  const int rc = (kind == kGated ? g_gated_fwd : g_fwd)(code, alpha.data_ptr(), beta.data_ptr(), h.data_ptr(),
+  const int rc = (kind == kGated ? g_gated_fwd : kind == kChannelMajor ? g_cm_fwd : g_fwd)(code, alpha.data_ptr(), beta.data_ptr(), h.data_ptr(),
                                                         alpha.size(0), alpha.size(1), alpha.size(2), ws.ptr, ws.size,
                                                         stream, nullptr);
   if (rc != 0) raise_status(rc);
@@ -168,9 +171,9 @@ struct ScanNode : public torch::autograd::Function<ScanNode> {
                 ? g_gated_bwd(code, alpha.data_ptr(), saved[1].data_ptr(), h.data_ptr(), dout.data_ptr(),
                               grad_alpha.data_ptr(), grad_beta.data_ptr(), alpha.size(0), alpha.size(1), alpha.size(2),
                               ws.ptr, ws.size, stream, nullptr)
-                : g_bwd(code, alpha.data_ptr(), h.data_ptr(), dout.data_ptr(), grad_alpha.data_ptr(),
-                        grad_beta.data_ptr(), alpha.size(0), alpha.size(1), alpha.size(2), ws.ptr, ws.size, stream,
-                        nullptr);
+                : (kind == kChannelMajor ? g_cm_bwd : g_bwd)(code, alpha.data_ptr(), h.data_ptr(), dout.data_ptr(),
+                                                             grad_alpha.data_ptr(), grad_beta.data_ptr(), alpha.size(0),
+                                                             alpha.size(1), alpha.size(2), ws.ptr, ws.size, stream, nullptr);
         if (rc != 0) raise_status(rc);
         done = true;
       }
@@ -202,15 +205,18 @@ struct ScanNode : public torch::autograd::Function<ScanNode> {
   }
 };
 
-void init(uintptr_t fwd, uintptr_t bwd, uintptr_t gated_fwd, uintptr_t gated_bwd, uintptr_t state_fwd, uintptr_t need,
-          uintptr_t strerror_fn, py::object slow_backward) {
+void init(uintptr_t fwd, uintptr_t bwd, uintptr_t gated_fwd, uintptr_t gated_bwd, uintptr_t state_fwd, uintptr_t cm_fwd,
+          uintptr_t cm_bwd, uintptr_t need, uintptr_t cm_need, uintptr_t strerror_fn, py::object slow_backward) {
   std::lock_guard<std::mutex> guard(g_lock);
   g_fwd = reinterpret_cast<FwdFn>(fwd);
   g_bwd = reinterpret_cast<BwdFn>(bwd);
   g_gated_fwd = reinterpret_cast<FwdFn>(gated_fwd);
   g_gated_bwd = reinterpret_cast<GatedBwdFn>(gated_bwd);
   g_state_fwd = reinterpret_cast<StateFwdFn>(state_fwd);
+  g_cm_fwd = reinterpret_cast<FwdFn>(cm_fwd);
+  g_cm_bwd = reinterpret_cast<BwdFn>(cm_bwd);
   g_need = reinterpret_cast<NeedFn>(need);
+  g_cm_need = reinterpret_cast<NeedFn>(cm_need);
   g_strerror = reinterpret_cast<StrerrorFn>(strerror_fn);
   g_slow_backward = new py::object(std::move(slow_backward));
   g_needs.clear();
@@ -266,6 +272,14 @@ std::optional<at::Tensor> scan_gated(const at::Tensor &gate, const at::Tensor &x
   return dispatch(gate, x, code, kGated);
 }
 
+// (bs, d_model, seq) tensors, time contiguous; the storage type is alpha's
+std::optional<at::Tensor> scan_cm(const at::Tensor &alpha, const at::Tensor &beta) {
+  if (!alpha.defined()) return std::nullopt;
+  const at::ScalarType t = alpha.scalar_type();
+  const int64_t code = t == at::kBFloat16 ? 0 : t == at::kFloat ? 1 : t == at::kHalf ? 2 : -1;
+  return dispatch(alpha, beta, code, kChannelMajor);
+}
+
 // (h, h_last) of the scan that starts from the fp32 state `h_before` (bs, d) - zeros when absent -
 // for calls that need no gradient: the step of a streaming decode loop, where the sequence is a
 // few tokens and the host's time is all there is.  None for anything else.
@@ -310,11 +324,12 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
   m.doc() = "C++ dispatch of the plain scan over the C ABI of libfss_scan.so";
   m.def("init", &init,
         "addresses of fss_scan_fwd_ex, fss_scan_bwd_ex, fss_gated_scan_fwd, fss_gated_scan_bwd, fss_scan_fwd_state, "
-        "fss_workspace_bytes, fss_strerror; the Python backward");
+        "fss_scan_fwd_cm, fss_scan_bwd_cm, fss_workspace_bytes, fss_cm_workspace_bytes, fss_strerror; the Python backward");
   m.def("register_workspace", &register_workspace, "device, stream, pointer, bytes, address of the flag word, address of the launch count");
   m.def("forget_workspaces", &forget_workspaces);
   m.def("scan", &scan, "h, or None when the call is not the common case");
   m.def("scan_gated", &scan_gated, "h of the gated scan, or None when the call is not the common case");
+  m.def("scan_cm", &scan_cm, "h of the channel-major scan, or None when the call is not the common case");
   m.def("scan_state", &scan_state, py::arg("alpha"), py::arg("beta"), py::arg("h_before") = py::none(),
         "(h, h_last) without gradients, or None when the call is not the common case");
 }

@@ -84,6 +84,7 @@ _UNRESOLVED = object()
 _fast: Any = _UNRESOLVED
 _fast_gated: Any = _UNRESOLVED
 _fast_state: Any = _UNRESOLVED
+_fast_cm: Any = _UNRESOLVED
 
 
 def _fast_scan(alpha: torch.Tensor, beta: torch.Tensor, code: int) -> Optional[torch.Tensor]:
@@ -263,4 +264,12 @@ class SequentialScanChannelMajor(Function):
 
 def scan_cm(alpha: torch.Tensor, beta: torch.Tensor) -> torch.Tensor:
     """``h[..., t] = alpha[..., t]*h[..., t-1] + beta[..., t]`` for ``(bs, d_model, seq)`` tensors."""
+    global _fast_cm
+    if _fast_cm is _UNRESOLVED:
+        binding = _ext.fast_dispatch()
+        _fast_cm = binding.scan_cm if binding is not None else None
+    if _fast_cm is not None and isinstance(alpha, torch.Tensor) and isinstance(beta, torch.Tensor):
+        h = _fast_cm(alpha, beta)
+        if h is not None:
+            return h
     return SequentialScanChannelMajor.apply(alpha, beta)

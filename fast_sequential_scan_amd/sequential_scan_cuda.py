@@ -161,6 +161,12 @@ def _need_gated(code: int, bs: int, seq: int, d: int, config) -> int:
                _need("rm", code, _native.FSS_GATED_BWD, bs, seq, d, config))
 
 
+def _need_cm(code: int, bs: int, d: int, seq: int, config) -> int:
+    """The same for the channel-major scan."""
+    return max(_need("cm", code, _native.FSS_FWD, bs, d, seq, config),
+               _need("cm", code, _native.FSS_BWD, bs, d, seq, config))
+
+
 def _workspace(device: torch.device, stream: "_RawStream", need: int) -> "_Workspace":
     """The workspace of (device, stream), grown to `need` bytes; raises if a scan launched through
     it earlier reported a chain time-out."""
@@ -189,6 +195,8 @@ def _slow_backward(kind: int, code: int, saved: List[torch.Tensor], grad_out: to
     saved (alpha, h); kind 1: the gated scan, saved (gate, x, h))."""
     if kind == 1:
         return gated_scan_backward(saved[0], saved[1], saved[2], grad_out)
+    if kind == 2:  # channel-major, saved (alpha, h)
+        return scan_backward_cm(saved[0], saved[1], grad_out)
     return _backward(_CODE_DTYPE[code], saved[0], saved[1], grad_out)
 
 
@@ -580,7 +588,7 @@ def scan_forward_cm(alpha: torch.Tensor, beta: torch.Tensor, config=None) -> tor
     cfg = _native.make_config(config)
     with _on(alpha.device):
         stream = _current_stream()
-        ws = _workspace(alpha.device, stream, _need("cm", code, _native.FSS_FWD, bs, d, seq, config))
+        ws = _workspace(alpha.device, stream, _need_cm(code, bs, d, seq, config))
         _native.check(
             lib.fss_scan_fwd_cm(
                 code, alpha.data_ptr(), beta.data_ptr(), out.data_ptr(), bs, d, seq,
@@ -606,7 +614,7 @@ def scan_backward_cm(
     cfg = _native.make_config(config)
     with _on(alpha_saved.device):
         stream = _current_stream()
-        ws = _workspace(alpha_saved.device, stream, _need("cm", code, _native.FSS_BWD, bs, d, seq, config))
+        ws = _workspace(alpha_saved.device, stream, _need_cm(code, bs, d, seq, config))
         _native.check(
             lib.fss_scan_bwd_cm(
                 code, alpha_saved.data_ptr(), h_saved.data_ptr(), grad_out.data_ptr(),

@@ -237,11 +237,11 @@ def test_torch_binding_loads_and_declines_what_it_does_not_cover():
 
     binding = ext.fast_dispatch()
     assert binding is not None
-    for name in ("init", "scan", "scan_gated", "scan_state", "register_workspace", "forget_workspaces"):
+    for name in ("init", "scan", "scan_gated", "scan_cm", "scan_state", "register_workspace", "forget_workspaces"):
         assert callable(getattr(binding, name))
     x = torch.zeros(2, 3, 4, dtype=torch.bfloat16)
     assert binding.scan(x, x, 0) is None and binding.scan(x, x, 7) is None
-    assert binding.scan_gated(x, x) is None and binding.scan_state(x, x, None) is None
+    assert binding.scan_gated(x, x) is None and binding.scan_cm(x, x) is None and binding.scan_state(x, x, None) is None
 
 
 def test_missing_library_is_an_error(monkeypatch, tmp_path):

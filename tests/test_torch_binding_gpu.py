@@ -9,7 +9,7 @@ pytestmark = pytest.mark.gpu
 
 from fast_sequential_scan_amd import scan_cu, scan_cu_single  # noqa: E402
 from fast_sequential_scan_amd import scan_cu_fp16 as scan_fp16  # noqa: E402
-from fast_sequential_scan_amd import scan_gated, scan_with_state  # noqa: E402
+from fast_sequential_scan_amd import scan_cm, scan_gated, scan_with_state  # noqa: E402
 from fast_sequential_scan_amd import scan_cuda  # noqa: E402
 from fast_sequential_scan_amd import sequential_scan_cuda as ext  # noqa: E402
 from fast_sequential_scan_amd.workloads import make_inputs  # noqa: E402
@@ -222,4 +222,28 @@ def test_captured_decode_step_replays_match_eager():
             assert torch.equal(h_out, want[i][0]) and torch.equal(state, want[i][1]), i
             scan_with_state(alpha, beta, torch.ones(bs, d, device=DEV))  # eager work between replays, same workspace
             side.synchronize()
+    ext.workspace_status()
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32], ids=["bf16", "f32"])
+@pytest.mark.parametrize("shape", [(2, 768, 1000), (3, 64, 37), (1, 130, 5000), (2, 96, 9000)])
+def test_channel_major_scan_same_bits_as_the_python_function(dtype, shape):
+    """(bs, d_model, seq) tensors: the C++ dispatch against the Python Function, forward and backward."""
+    alpha, beta, dout = _tensors(shape, dtype, seed=sum(shape))
+    a1, b1 = alpha.clone().requires_grad_(True), beta.clone().requires_grad_(True)
+    want = scan_cuda.SequentialScanChannelMajor.apply(a1, b1)
+    want.backward(dout)
+    a2, b2 = alpha.clone().requires_grad_(True), beta.clone().requires_grad_(True)
+    got = scan_cm(a2, b2)
+    assert "ScanNode" in _node_name(got), _node_name(got)
+    got.backward(dout)
+    ext.workspace_status()
+    assert torch.equal(got, want) and torch.equal(a2.grad, a1.grad) and torch.equal(b2.grad, b1.grad)
+    with torch.no_grad():
+        assert torch.equal(scan_cm(a2, b2), want)
+    a_t = alpha.transpose(1, 2).contiguous().transpose(1, 2).requires_grad_(True)
+    out = scan_cm(a_t, beta)
+    assert "ScanNode" not in _node_name(out) and torch.equal(out, want)
+    with pytest.raises(RuntimeError):
+        scan_cm(alpha, beta[:, :, :10])
     ext.workspace_status()
