@@ -463,7 +463,7 @@ def main() -> int:
         del junk
 
     # ---- the public autograd path (allocates its outputs, goes through torch.autograd) ----
-    autograd_ms = autograd_cpu_ms = None
+    autograd_ms = autograd_cpu_ms = autograd_inline_ms = autograd_inline_cpu_ms = None
     if not args.no_autograd:
         a_req = alpha.detach().clone().requires_grad_(True)
         b_req = beta.detach().clone().requires_grad_(True)
@@ -482,6 +482,21 @@ def main() -> int:
         torch.cuda.synchronize()
         autograd_ms = (time.perf_counter() - t0) * 1e3 / n_auto
         autograd_cpu_ms = (t_enqueued - t0) * 1e3 / n_auto  # host time to issue a step; the GPU may lag behind it
+        # the same loop with torch's autograd engine running the backward on the calling thread instead of
+        # handing it to its device thread (a caller's choice; the hand-over costs up to 30 us per step on some hosts)
+        with torch.autograd.set_multithreading_enabled(False):
+            for _ in range(20):
+                scan_fn(a_req, b_req).backward(dout)
+                a_req.grad = b_req.grad = None
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            for _ in range(n_auto):
+                scan_fn(a_req, b_req).backward(dout)
+                a_req.grad = b_req.grad = None
+            t_enqueued = time.perf_counter()
+            torch.cuda.synchronize()
+            autograd_inline_ms = (time.perf_counter() - t0) * 1e3 / n_auto
+            autograd_inline_cpu_ms = (t_enqueued - t0) * 1e3 / n_auto
 
     # ---- CPU baseline + parity of this very run ----
     cpu = None
@@ -641,6 +656,9 @@ def main() -> int:
         "rotating_sets": rotating,
         "autograd_path_ms_per_step": None if autograd_ms is None else round(autograd_ms, 5),
         "autograd_path_host_ms_per_step": None if autograd_cpu_ms is None else round(autograd_cpu_ms, 5),
+        "autograd_path_backward_on_calling_thread": None if autograd_inline_ms is None else {
+            "ms_per_step": round(autograd_inline_ms, 5), "host_ms_per_step": round(autograd_inline_cpu_ms, 5),
+            "how": "torch.autograd.set_multithreading_enabled(False)"},
         "parity": parity,
         "cpu_baseline": cpu,
     }
