@@ -440,26 +440,36 @@ def main() -> int:
         junk = torch.zeros(args.flush_mb << 18, dtype=torch.int32, device=dev)
         torch.cuda.synchronize()
         e = [torch.cuda.Event(enable_timing=True) for _ in range(4)]
-        cf, cb = [], []
-        for _ in range(10):
-            junk.sum()
-            e[0].record(stream)
-            fwd()
-            e[1].record(stream)
-            junk.sum()
-            e[2].record(stream)
-            bwd()
-            e[3].record(stream)
-            torch.cuda.synchronize()
-            cf.append(e[0].elapsed_time(e[1]))
-            cb.append(e[2].elapsed_time(e[3]))
-        cold = {
-            "fwd_ms": round(statistics.median(cf), 5),
-            "bwd_ms": round(statistics.median(cb), 5),
-            "fwd_GBps": round(fwd_bytes_per_elem * n_elem / (statistics.median(cf) * 1e-3) / 1e9, 1),
-            "bwd_GBps": round(bwd_bytes_per_elem * n_elem / (statistics.median(cb) * 1e-3) / 1e9, 1),
-            "flush_MB": args.flush_mb,
-        }
+
+        def cold_leg():
+            cf, cb = [], []
+            for _ in range(10):
+                junk.sum()
+                e[0].record(stream)
+                fwd()
+                e[1].record(stream)
+                junk.sum()
+                e[2].record(stream)
+                bwd()
+                e[3].record(stream)
+                torch.cuda.synchronize()
+                cf.append(e[0].elapsed_time(e[1]))
+                cb.append(e[2].elapsed_time(e[3]))
+            return {
+                "fwd_ms": round(statistics.median(cf), 5),
+                "bwd_ms": round(statistics.median(cb), 5),
+                "fwd_GBps": round(fwd_bytes_per_elem * n_elem / (statistics.median(cf) * 1e-3) / 1e9, 1),
+                "bwd_GBps": round(bwd_bytes_per_elem * n_elem / (statistics.median(cb) * 1e-3) / 1e9, 1),
+            }
+
+        cold = cold_leg()
+        cold["flush_MB"] = args.flush_mb
+        if args.cache_policy == "auto" and not cm:
+            ext.set_cache_policy("streaming")
+            try:
+                cold["streaming_policy"] = cold_leg()
+            finally:
+                ext.set_cache_policy("auto")
         del junk
 
     # ---- the public autograd path (allocates its outputs, goes through torch.autograd) ----
