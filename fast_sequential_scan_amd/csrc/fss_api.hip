@@ -126,6 +126,8 @@ int run_scan(int dtype, int dir, const void *alpha, const void *in_b, const void
   args.n_groups = static_cast<int32_t>(pl.n_groups);
   args.wg_cols = pl.cfg.cols;
   args.look_waves = look_waves(pl.cfg.waves, pl.cfg.vec, pl.cfg.cols);
+  args.period = chain_period(pl.n_groups, pl.cfg.waves);
+  args.span = look_span(args.n_chunks, args.period, args.look_waves);
   args.spin_limit = __atomic_load_n(&g_spin_limit, __ATOMIC_RELAXED);
   const int64_t tensor_bytes = bs * seq * d * static_cast<int64_t>(esize);
   if (streaming)
@@ -264,6 +266,31 @@ int fss_debug_tile_groups(int32_t n_groups, int32_t grid, int32_t n_tiles, int32
     groups[tile] = static_cast<int32_t>(
         fss::tile_group(order, static_cast<uint32_t>(tile % n_groups), static_cast<uint32_t>(tile / n_groups)));
   return FSS_OK;
+}
+
+int fss_debug_chain_plan(int64_t bs, int64_t seq, int64_t d, int dtype, int dir, size_t align_bytes,
+                         const fss_config *cfg, int32_t *out) {
+  if (!out) return FSS_ERR_NULL_POINTER;
+  fss::Plan pl;
+  const bool streaming = __atomic_load_n(&fss::g_cache_policy, __ATOMIC_RELAXED) == FSS_CACHE_STREAMING;
+  const int rc = fss::make_plan(pl, bs, seq, d, dtype, dir, align_bytes ? align_bytes : 16, cfg, streaming);
+  if (rc != FSS_OK) return rc;
+  const int look = fss::look_waves(pl.cfg.waves, pl.cfg.vec, pl.cfg.cols);
+  const int period = fss::chain_period(pl.n_groups, pl.cfg.waves);
+  out[0] = static_cast<int32_t>(pl.n_chunks);
+  out[1] = pl.cfg.waves / pl.cfg.cols;
+  out[2] = pl.cfg.steps;
+  out[3] = period;
+  out[4] = look;
+  out[5] = fss::look_span(static_cast<int>(pl.n_chunks), period, look);
+  out[6] = pl.cfg.vec;
+  out[7] = pl.cfg.cols;
+  return FSS_OK;
+}
+
+int32_t fss_debug_chain_anchor(int32_t chunk, int32_t period) {
+  if (chunk < 0 || period < 1) return -1;
+  return fss::chain_anchor(chunk, period);
 }
 
 uint32_t fss_debug_set_spin_limit(uint32_t polls) {

@@ -258,7 +258,6 @@ constexpr int kMaxLookWaves = 16;
 // chunks one look-back wave covers at most (measured: 2 -> 4 gains up to 12 % on chains of
 // hundreds of chunks, 8 nothing more)
 constexpr int kMaxSpan = 4;
-enum : uint32_t { kPredNone = 0, kPredMap = 1, kPredState = 2 };
 
 __device__ __forceinline__ uint32_t ld_u32(const uint32_t *p) {
   return __hip_atomic_load((const FSS_GLOBAL uint32_t *)p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -313,6 +312,8 @@ struct ScanArgs {
   int32_t n_groups;       // column groups per chunk: n_ctiles / wg_cols
   int32_t wg_cols;        // adjacent column tiles a workgroup covers side by side (1 or 2)
   int32_t look_waves;     // waves per column tile that look back in parallel (1..kMaxLookWaves)
+  int32_t period;         // chunks of a sequence between two anchors of the chain (chain_anchor), >= 1
+  int32_t span;           // chunks one look-back wave covers, one after the other (1..kMaxSpan)
   uint32_t spin_limit;    // polls before a look-back gives up (kSpinLimit unless a test lowered it)
   uint32_t *hdr;          // workspace header
   uint64_t *words;        // tagged words
@@ -445,82 +446,106 @@ struct TileCtx {
   uint32_t lane_off;     // byte offset of the lane's channels inside the tile's row segment
   bool col_ok;           // the lane's channels exist (d % VEC == 0, so all or none)
   float2 *lds_map;       // [wave][v][lane] = (A, B) of this tile
-  float2 *lds_pred;      // [look wave][v][lane] = what an earlier chunk offers
-  uint32_t *s_kind;      // [look wave] kind of that offer
-  uint32_t *s_kind_other;  // the same of the workgroup's other column tile (two column tiles per workgroup only)
+  float2 *lds_pred;      // [look wave][v][lane] = what that wave's earlier chunks do to a state
   int span;              // chunks one look-back wave covers: more than 1 when the sequence has more chunks than such waves
+  int anchor;            // the earlier chunk whose outgoing state this chunk's chain starts from (chain_anchor)
 #ifdef FSS_TRACE
   int trace_wave;
 #endif
 };
 
-// Chunks one look-back wave covers, one after the other.  Only the chunks of a column group
-// that the grid works on at once (gridDim / n_groups of them, tiles being numbered chunk-major)
-// can still lack an outgoing state; whatever lies before them was finished in an earlier round
-// of the grid, so the first look there ends the walk.  One round of the look-back should reach
-// across those chunks; a chain it does not reach simply takes another round.
-__device__ __forceinline__ int look_span(int n_chunks, int n_groups, int look) {
-  const int in_flight = (static_cast<int>(gridDim.x) + n_groups - 1) / n_groups;
-  const int need = n_chunks - 1 < in_flight ? n_chunks - 1 : in_flight;
+// ---- the order in which a chunk's incoming state is composed -----------------------------
+//
+// The state entering chunk k is  map[k-1] o map[k-2] o ... o map[a+1] (state[a])  for one earlier
+// chunk a = chain_anchor(k), the "anchor" of k.  Which chunk that is, and how the maps between are
+// grouped when they are composed, is fixed by k and by the plan (period, look-back waves, span)
+// - never by which of the earlier chunks happen to have finished when k looks back.  The
+// composition of affine maps is associative only up to fp32 rounding, so this is what makes
+// the result of a chained scan a function of its inputs and its launch configuration alone:
+// the same bits from run to run, on any stream, whatever else the device is doing.
+//
+// `period` is the number of chunks of one sequence that a full grid works on at once (tiles are
+// numbered chunk-major, so the chunks of a sequence in flight together are consecutive).  Chunk
+// k of round R = k / period takes the maps of its own round's earlier chunks - published as soon
+// as their rows are loaded - and the outgoing state of the last chunk of round R-1, which a
+// grid of the planned size finished a round ago (in round 0: of chunk 0, which needs no
+// look-back).  The period is planned from the nominal device, not from the grid actually
+// launched: a smaller grid or device meets the same anchors (and merely finds the maps
+// already there), so the results do not depend on it either.
+__host__ __device__ inline int chain_anchor(int chunk, int period) {
+  const int round_first = chunk - chunk % period;
+  return round_first > 0 ? round_first - 1 : 0;
+}
+
+// Chunks one look-back wave covers, one after the other: one round of the look-back (`look`
+// waves in parallel) should reach across a period; a chain it does not reach takes another round.
+__host__ __device__ inline int look_span(int n_chunks, int period, int look) {
+  const int need = n_chunks - 1 < period ? n_chunks - 1 : period;
   const int span = (need + look - 1) / look;
   return span < 1 ? 1 : (span > kMaxSpan ? kMaxSpan : span);
 }
 
-// One look at what chunk `j` of this column tile offers: its outgoing state if it
-// has published one, else (j > 0) its map.  Split in two so that other work can be
-// placed between the loads and the use of what they return.
+// One look at chunk `j` of this column tile: at its outgoing state (`want_state`: j is the
+// anchor) or at its map.  Split in two so that other work can be placed between the loads and
+// the use of what they return.
 template <int VEC>
 struct ChunkWords {
-  uint64_t a[VEC], b[VEC], s[VEC];
+  uint64_t a[VEC], b[VEC];
 };
 
 template <int VEC>
-__device__ __forceinline__ void poll_issue(const ScanArgs &p, const TileCtx &c, int j, ChunkWords<VEC> &w) {
+__device__ __forceinline__ void poll_issue(const ScanArgs &p, const TileCtx &c, int j, bool want_state,
+                                           ChunkWords<VEC> &w) {
   const uint64_t *theirs = p.words + (static_cast<size_t>(j) * p.n_ctiles + c.ctile) * 3 * (64 * VEC) + c.lane;
+  // (a state is asked for as both halves of a "map": the same straight-line code either way)
+  const uint64_t *word_a = theirs + (want_state ? 2 * VEC * 64 : 0);
+  const uint64_t *word_b = theirs + (want_state ? 2 * VEC * 64 : VEC * 64);
 #pragma unroll
   for (int v = 0; v < VEC; ++v) {
-    w.s[v] = ld_word(theirs + (2 * VEC + v) * 64);
-    w.a[v] = ld_word(theirs + (0 * VEC + v) * 64);
-    w.b[v] = ld_word(theirs + (1 * VEC + v) * 64);
+    w.a[v] = ld_word(word_a + v * 64);
+    w.b[v] = ld_word(word_b + v * 64);
   }
 }
 
-// The answer is taken for the whole wave, so that one word per wave can describe
-// it.  Returns kPredNone when neither a state nor a map is there yet.
+// True once every lane of the wave has what it asked for (the answer is taken for the whole
+// wave); then (qA, qB) is the map, a state s being the map x -> 0*x + s.
 template <int VEC>
-__device__ __forceinline__ uint32_t poll_eval(const TileCtx &c, int j, const ChunkWords<VEC> &w, float *qA,
-                                              float *qB) {
-  bool have_state = true, have_map = true;
+__device__ __forceinline__ bool poll_eval(const TileCtx &c, bool want_state, const ChunkWords<VEC> &w, float *qA,
+                                          float *qB) {
+  bool have = true;
+#pragma unroll
+  for (int v = 0; v < VEC; ++v) have = have && word_tag(w.a[v]) == c.tag && word_tag(w.b[v]) == c.tag;
+  if (__builtin_amdgcn_ballot_w64(have) != ~0ull) return false;
 #pragma unroll
   for (int v = 0; v < VEC; ++v) {
-    have_state = have_state && word_tag(w.s[v]) == c.tag;
-    have_map = have_map && word_tag(w.a[v]) == c.tag && word_tag(w.b[v]) == c.tag;
+    qA[v] = want_state ? 0.0f : word_val(w.a[v]);
+    qB[v] = word_val(w.b[v]);
   }
-  if (__builtin_amdgcn_ballot_w64(have_state) == ~0ull) {
-#pragma unroll
-    for (int v = 0; v < VEC; ++v) {
-      qA[v] = 0.0f;
-      qB[v] = word_val(w.s[v]);
-    }
-    return kPredState;
-  }
-  if (j > 0 && __builtin_amdgcn_ballot_w64(have_map) == ~0ull) {
-#pragma unroll
-    for (int v = 0; v < VEC; ++v) {
-      qA[v] = word_val(w.a[v]);
-      qB[v] = word_val(w.b[v]);
-    }
-    return kPredMap;
-  }
-  return kPredNone;
+  return true;
 }
 
+// Waits (bounded) for chunk j's state or map.  A wave that gives up reports it and carries on
+// with a NaN state, so that the grid still drains and everything downstream is visibly poisoned.
 template <int VEC>
-__device__ __forceinline__ uint32_t poll_chunk(const ScanArgs &p, const TileCtx &c, int j, float *qA,
-                                               float *qB) {
-  ChunkWords<VEC> w;
-  poll_issue<VEC>(p, c, j, w);
-  return poll_eval<VEC>(c, j, w, qA, qB);
+__device__ __forceinline__ void await_chunk(const ScanArgs &p, const TileCtx &c, int j, bool want_state, float *qA,
+                                            float *qB) {
+  uint32_t polls = 0;
+  for (;;) {
+    if (polls >= p.spin_limit) {
+      if (c.lane == 0) report_timeout(p.hdr);
+#pragma unroll
+      for (int v = 0; v < VEC; ++v) {
+        qA[v] = 0.0f;
+        qB[v] = local_const(__builtin_nanf(""));
+      }
+      return;
+    }
+    ChunkWords<VEC> w;
+    poll_issue<VEC>(p, c, j, want_state, w);
+    if (poll_eval<VEC>(c, want_state, w, qA, qB)) return;
+    ++polls;
+    __builtin_amdgcn_s_sleep(2);
+  }
 }
 
 // (A, B) <- map[count-1] o ... o map[0] for this lane's channels: the maps of the
@@ -596,14 +621,18 @@ __device__ __forceinline__ void fold_and_leave_prefixes(float2 *lds_map, int lan
 // entering the slice.  Every wave of the workgroup must call it (barriers).
 //
 // After one barrier wave 0 composes all the waves' maps into the chunk's map and
-// publishes it, leaving in every wave's slot the composition of the waves before it.  Meanwhile wave w (w < look) fetches what chunk-1-w offers - its
-// outgoing state if it has one, else its map - so a look-back over `look` chunks
-// costs one memory round trip instead of one per chunk.  After a second barrier
-// every wave folds what the look-back waves found into the chunk's incoming state
-// itself (a few multiply-adds: cheaper than a third barrier and a broadcast), wave 0
-// also publishes the chunk's outgoing state, and every wave applies the composition
-// of the waves before it (one LDS read; the first chunk of a sequence, which has no second
-// barrier to wait at, composes it itself).  Chains longer than `look` repeat the fetch.
+// publishes it, leaving in every wave's slot the composition of the waves before it.
+// Meanwhile the look-back: the chunks from chunk-1 down to the anchor (chain_anchor) are
+// dealt out to the first `look` waves, `span` consecutive chunks each, nearest first; each
+// such wave waits for its chunks' maps (the anchor's outgoing state) and composes them, so a
+// look-back over look*span chunks costs `span` memory round trips instead of one per chunk.
+// After a second barrier every wave folds what the look-back waves left in LDS into the
+// chunk's incoming state itself (a few multiply-adds: cheaper than a third barrier and a
+// broadcast), wave 0 also publishes the chunk's outgoing state, and every wave applies the
+// composition of the waves before it (one LDS read; the first chunk of a sequence, which has
+// no second barrier to wait at, composes it itself).  A chain of more than look*span chunks
+// repeats the look-back.  Who looks at which chunk, and the order of every composition, depend
+// on the chunk's index and the plan alone.
 //
 // `mid` (only with HAS_MID) is called once by every wave, by the look-back waves right after their
 // first fetch has been issued: loads it issues travel while the chain is resolved and
@@ -646,9 +675,6 @@ __device__ __forceinline__ void chain_chunks(const ScanArgs &p, const TileCtx &c
   if (!look_back) {
     if constexpr (HAS_MID) mid();
     fold_wave_maps<VEC>(c.lds_map, lane, wave, pA, pB);
-  }
-
-  if (!look_back) {
     // first chunk of the sequence (or the only one): the incoming state is the
     // sequence's own (0 in the plain scan)
     if (wave == 0 && c.chained && !c.last) {
@@ -669,83 +695,43 @@ __device__ __forceinline__ void chain_chunks(const ScanArgs &p, const TileCtx &c
     accB[v] = local_const(0.0f);
     hin[v] = local_const(0.0f);
   }
-  int nearest = c.chunk - 1;  // nearest earlier chunk not folded yet
-  int other_nearest = nearest;
+  const int anchor = c.anchor;
+  const int reach = c.look * c.span;  // chunks one round of the look-back covers
+  int nearest = c.chunk - 1;          // nearest earlier chunk not folded yet (>= anchor)
   // The first look goes out ahead of the loop, with `mid` in a straight line between the
   // issue of its loads and their use: only so does the compiler wait for exactly those
   // loads and not for the ones `mid` has issued behind them.
-  uint32_t kind0 = kPredNone;
+  bool have0 = false;
   float q0A[VEC], q0B[VEC];
 #pragma unroll
   for (int v = 0; v < VEC; ++v) q0A[v] = q0B[v] = local_const(0.0f);
   if constexpr (HAS_MID) {
-    if (wave < c.look && nearest - wave * c.span >= 0) {
+    const int j0 = nearest - wave * c.span;
+    if (wave < c.look && j0 >= anchor && p.spin_limit != 0) {
       ChunkWords<VEC> w;
-      poll_issue<VEC>(p, c, nearest - wave * c.span, w);
+      poll_issue<VEC>(p, c, j0, j0 == anchor, w);
       mid();
-      kind0 = poll_eval<VEC>(c, nearest - wave * c.span, w, q0A, q0B);
+      have0 = poll_eval<VEC>(c, j0 == anchor, w, q0A, q0B);
     } else {
       mid();
     }
   }
-  // A workgroup that covers two column tiles runs two look-backs side by side, which must
-  // leave this loop together (they share the barriers).  Every wave therefore follows the
-  // other column's look-back as well: what its look-back waves found is in LDS behind the
-  // same barrier, so all waves of the workgroup see the same two answers and agree.
-  bool done = false;
-  bool other_done = p.wg_cols <= 1;  // (wg_cols is 1 wherever the kernel was compiled for one column)
   for (;;) {
     const int j = nearest - wave * c.span;
-    if (!done && wave < c.look && j >= 0) {
+    if (wave < c.look && j >= anchor) {
       float qA[VEC], qB[VEC];
-      uint32_t polls = 0;
-      uint32_t kind = kind0;  // what the first look found (nothing, in later rounds)
 #pragma unroll
       for (int v = 0; v < VEC; ++v) {
         qA[v] = q0A[v];
         qB[v] = q0B[v];
       }
-      kind0 = kPredNone;
-      if (p.spin_limit == 0) kind = kPredNone;
-      while (kind == kPredNone) {
-        if (polls >= p.spin_limit) {
-          // give up, so that the grid still drains: a NaN state poisons what follows
-          if (lane == 0) report_timeout(p.hdr);
-          kind = kPredState;
-#pragma unroll
-          for (int v = 0; v < VEC; ++v) {
-            qA[v] = 0.0f;
-            qB[v] = local_const(__builtin_nanf(""));
-          }
-          break;
-        }
-        kind = poll_chunk<VEC>(p, c, j, qA, qB);
-        if (kind != kPredNone) break;
-        ++polls;
-        __builtin_amdgcn_s_sleep(2);
-      }
+      if (!have0) await_chunk<VEC>(p, c, j, j == anchor, qA, qB);
+      have0 = false;
       // long chains: the wave also takes the chunks before that one (by now they have nearly
       // always published), so that one round of the look-back reaches `span` times as far
-      for (int k = 1; k < c.span && kind == kPredMap && j - k >= 0; ++k) {
+      for (int k = 1; k < c.span && j - k >= anchor; ++k) {
         float rA[VEC], rB[VEC];
-        polls = 0;
-        for (;;) {
-          if (polls >= p.spin_limit) {
-            if (lane == 0) report_timeout(p.hdr);
-            kind = kPredState;
-#pragma unroll
-            for (int v = 0; v < VEC; ++v) {
-              rA[v] = 0.0f;
-              rB[v] = local_const(__builtin_nanf(""));
-            }
-            break;
-          }
-          kind = poll_chunk<VEC>(p, c, j - k, rA, rB);
-          if (kind != kPredNone) break;
-          ++polls;
-          __builtin_amdgcn_s_sleep(2);
-        }
-        // (a state is the map x -> 0*x + value)
+        await_chunk<VEC>(p, c, j - k, j - k == anchor, rA, rB);
 #pragma unroll
         for (int v = 0; v < VEC; ++v) {
           qB[v] = fma0(qA[v], rB[v], qB[v]);
@@ -754,53 +740,28 @@ __device__ __forceinline__ void chain_chunks(const ScanArgs &p, const TileCtx &c
       }
 #pragma unroll
       for (int v = 0; v < VEC; ++v) c.lds_pred[(wave * VEC + v) * 64 + lane] = make_float2(qA[v], qB[v]);
-      if (lane == 0) c.s_kind[wave] = kind;
     }
     __syncthreads();
     // every wave folds what the look-back waves found (the same few LDS reads in each wave
     // cost less than a second barrier and a broadcast by wave 0)
-    if (!done) {
-      bool resolved = false;
-      for (int w = 0; w < c.look && nearest - w * c.span >= 0 && !resolved; ++w) {
-        const bool is_state = c.s_kind[w] == kPredState;
+    for (int w = 0; w < c.look && nearest - w * c.span >= anchor; ++w) {
 #pragma unroll
-        for (int v = 0; v < VEC; ++v) {
-          const float2 m = c.lds_pred[(w * VEC + v) * 64 + lane];
-          if (is_state) {
-            hin[v] = fma0(accA[v], m.y, accB[v]);
-          } else {
-            accB[v] = fma0(accA[v], m.y, accB[v]);
-            accA[v] *= m.x;
-          }
-        }
-        resolved = is_state;
-      }
-      if (resolved) {  // chunk 0 always offers a state, so this is reached
-        done = true;
-        if (wave == 0 && !c.last) {
-#pragma unroll
-          for (int v = 0; v < VEC; ++v)
-            st_word(mine + (2 * VEC + v) * 64, c.tag, fma0(cA[v], hin[v], cB[v]));
-        }
-      } else {
-        nearest -= c.look * c.span;
-        if (nearest < 0) {  // cannot happen; never spin on a logic error
-          if (lane == 0 && wave == 0) report_timeout(p.hdr);
-          done = true;
-        }
+      for (int v = 0; v < VEC; ++v) {
+        const float2 m = c.lds_pred[(w * VEC + v) * 64 + lane];
+        accB[v] = fma0(accA[v], m.y, accB[v]);
+        accA[v] *= m.x;
       }
     }
-    if (!other_done) {
-      // (the other column is at the same chunk and in the same round, so the same slots count)
-      for (int w = 0; w < c.look && other_nearest - w * c.span >= 0 && !other_done; ++w)
-        other_done = c.s_kind_other[w] == kPredState;
-      if (!other_done) {
-        other_nearest -= c.look * c.span;
-        if (other_nearest < 0) other_done = true;  // as above: cannot happen
-      }
-    }
-    if (done && other_done) break;
+    nearest -= reach;
+    if (nearest < anchor) break;
     __syncthreads();  // the slots are about to be overwritten: wait until every wave has read them
+  }
+  // (the last group folded ended with the anchor's state, the map x -> 0*x + s: accB is the state)
+#pragma unroll
+  for (int v = 0; v < VEC; ++v) hin[v] = accB[v];
+  if (wave == 0 && !c.last) {
+#pragma unroll
+    for (int v = 0; v < VEC; ++v) st_word(mine + (2 * VEC + v) * 64, c.tag, fma0(cA[v], hin[v], cB[v]));
   }
   FSS_STAMP(c, p, 4);
   // (the prefix wave 0 left in this wave's slot, behind the loop's barrier)

@@ -74,6 +74,19 @@ inline bool config_valid(const fss_config &c, int dtype, bool gated = false, int
 // (planning must work without a device; the grid itself is sized from the runtime's count).
 constexpr int64_t kCus = 256;
 
+// Chunks of one sequence that a full grid works on at once: the spacing of the chain's anchors
+// (chain_anchor in fss_device.h).  Planned from the nominal device - kCus compute units holding
+// 16 waves of a scan each - and from nothing that can differ between two launches of one
+// configuration (not the grid actually launched, not the device's own CU count), so that the
+// order in which carries are composed, and with it every bit of the result, is fixed by the
+// shape and the configuration.
+inline int chain_period(int64_t n_groups, int waves) {
+  const int64_t per_cu = waves >= 16 ? 1 : 16 / (waves > 0 ? waves : 1);
+  const int64_t nominal_grid = kCus * per_cu;
+  const int64_t period = ceil_div(nominal_grid, n_groups > 0 ? n_groups : 1);
+  return static_cast<int>(period < 1 ? 1 : (period > (1 << 20) ? (1 << 20) : period));
+}
+
 // One candidate launch configuration: taken when it yields at least `need` tiles.
 struct Rung {
   int vec, steps, waves;

@@ -195,19 +195,16 @@ __device__ __forceinline__ void cm_tile(const ScanArgs &p, const TileCtx &c, int
 template <typename E, int VEC, int ROWS, bool BWD>
 __global__ __launch_bounds__(1024) void cm_scan_kernel(const ScanArgs p) {
   extern __shared__ float lds[];
-  __shared__ uint32_t s_kind[kMaxLookWaves];
 
   TileCtx c;
   c.wcol = 0;
-  c.s_kind_other = s_kind;
   c.lane = threadIdx.x & 63;
   c.wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   c.n_waves = blockDim.x >> 6;
   c.look = p.look_waves;
-  c.span = look_span(p.n_chunks, p.n_groups, p.look_waves);
+  c.span = p.span;
   float2 *const lds_maps = reinterpret_cast<float2 *>(lds);  // laid out as in scan_kernel with one slot per lane
   c.lds_pred = lds_maps + 2 * c.n_waves * 64;
-  c.s_kind = s_kind;
   c.seq = p.seq;
   c.row_bytes = 0;
   c.lane_off = 0;
@@ -227,6 +224,7 @@ __global__ __launch_bounds__(1024) void cm_scan_kernel(const ScanArgs p) {
     c.chunk = static_cast<int>(chunk);
     c.ctile = static_cast<int>(ctile);
     c.last = c.chunk == p.n_chunks - 1;
+    c.anchor = __builtin_amdgcn_readfirstlane(chain_anchor(c.chunk, p.period));
     cm_tile<E, VEC, ROWS, BWD>(p, c, static_cast<int64_t>(ctile) * ROWS, p.d);
   }
   count_out(p, c);
@@ -303,6 +301,8 @@ int run_cm_scan(int dtype, int dir, const void *alpha, const void *in_b, const v
   args.n_groups = static_cast<int32_t>(pl.n_rowtiles);
   args.wg_cols = 1;
   args.look_waves = look_waves(pl.waves, 1);
+  args.period = chain_period(pl.n_rowtiles, pl.waves);
+  args.span = look_span(args.n_chunks, args.period, args.look_waves);
   args.spin_limit = __atomic_load_n(&g_spin_limit, __ATOMIC_RELAXED);
   args.hdr = static_cast<uint32_t *>(workspace);
   args.words = workspace ? reinterpret_cast<uint64_t *>(static_cast<char *>(workspace) + kHeaderBytes) : nullptr;

@@ -459,7 +459,6 @@ __global__ __launch_bounds__(MAXW * 64) void scan_kernel(const ScanArgs p, const
   constexpr int kLaneSlots = 64 * VEC;  // channels per tile
 
   extern __shared__ float lds[];
-  __shared__ uint32_t s_kind[2 * kMaxLookWaves];
 
   // The waves of a workgroup: wg_cols column tiles side by side, each with n_waves waves
   // that take consecutive time slices.  Everything the chain phase touches is per column tile.
@@ -473,14 +472,12 @@ __global__ __launch_bounds__(MAXW * 64) void scan_kernel(const ScanArgs p, const
   c.wcol = COLS > 1 ? (wave_in_group & 1) : 0;
   c.wave = COLS > 1 ? (wave_in_group >> 1) : wave_in_group;
   c.look = p.look_waves;
-  c.span = look_span(p.n_chunks, p.n_groups, p.look_waves);
+  c.span = p.span;
   // LDS: two sets of per-wave maps (tiles alternate between them, so a wave that runs
   // ahead into the next tile cannot overwrite a map a slower wave still reads), then
   // the slots the look-back waves fill
   float2 *const lds_maps = reinterpret_cast<float2 *>(lds);
   c.lds_pred = lds_maps + (2 * waves_total + c.wcol * c.look) * kLaneSlots;
-  c.s_kind = s_kind + c.wcol * kMaxLookWaves;
-  c.s_kind_other = s_kind + (1 - c.wcol) * kMaxLookWaves;
   c.seq = p.seq;
   c.row_bytes = p.d * E::kBytes;
 #ifdef FSS_TRACE
@@ -520,6 +517,7 @@ __global__ __launch_bounds__(MAXW * 64) void scan_kernel(const ScanArgs p, const
     c.chunk = static_cast<int>(chunk);
     c.ctile = static_cast<int>(ctile);
     c.last = c.chunk == p.n_chunks - 1;
+    c.anchor = __builtin_amdgcn_readfirstlane(chain_anchor(c.chunk, p.period));
 
     const int64_t col0 = static_cast<int64_t>(coltile) * kLaneSlots;  // first channel of the tile
     c.col_ok = col0 + c.lane * VEC < p.d;

@@ -18,7 +18,7 @@ ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 
 def test_library_exports_every_declared_symbol():
     header = open(os.path.join(ROOT, "include", "fss_scan.h")).read()
-    declared = set(re.findall(r"^(?:int|size_t|uint32_t|const char \*)\s*(fss_[a-z0-9_]+)\(", header, flags=re.M))
+    declared = set(re.findall(r"^(?:int|size_t|uint32_t|int32_t|const char \*)\s*(fss_[a-z0-9_]+)\(", header, flags=re.M))
     assert declared == set(_native.EXPORTED_SYMBOLS)
     lib = ctypes.CDLL(_native.LIB_PATH)
     for name in declared:
