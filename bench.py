@@ -10,15 +10,28 @@ tensors already resident in HBM.  Prints ONE JSON line:
                    alpha, beta and writes h = 6 B; backward reads alpha, h, dout and
                    writes grad_alpha, grad_beta = 10 B) divided by the wall time per step
   roofline         the dominant kernel (the backward scan, 10 of the 16 B): its
-                   algorithmic bytes per launch over its mean duration, measured with
-                   HIP events recorded around the launches of sampled steps of the timed
-                   region and of a sampling loop that follows it (at least 32 samples
-                   whatever --steps is), less what a pair of events adds to a kernel
-                   between them (calibrated in the same run with the library's copy
-                   kernel: one launch between two events against four); `traffic` is
-                   the counter-measured HBM bytes per launch from profiles/, when that
-                   summary covers the configuration; `frac_no_reuse` is the same
-                   fraction with eight sets of tensors in rotation
+                   algorithmic bytes per launch over its launch duration.  The duration is
+                   the kernel's share of the wall time per step of the timed region - the
+                   step split in the ratio of the two launches as HIP events around sampled
+                   steps see them - so forward and backward add up to `ms_per_step` and the
+                   few microseconds between two launches are charged to the kernels, not
+                   dropped (`avg_launch_ms`; a rocprofv3 kernel trace, which leaves those
+                   gaps out, reads 0-3 % shorter).  Beside it: `avg_launch_ms_events_raw`
+                   (events as read, at least 32 samples) and `avg_launch_ms_events_corrected`
+                   (less what a pair of events adds to a kernel between them, calibrated in the
+                   same run with the library's copy kernel: one launch between two events
+                   against four).  `traffic` is the counter-measured HBM bytes per launch from
+                   profiles/, when that summary covers the configuration; `frac_no_reuse` is
+                   the same fraction with eight sets of tensors in rotation;
+                   `frac_of_machine` the kernel's rate in that rotation over what the
+                   library's plain streaming kernel reaches on the same buffers with the
+                   same mix of reads and writes (`machine_stream`)
+  machine_stream   fss_stream_mix over the same eight tensor sets in rotation: 3 reads, 2 reads +
+                   1 non-temporal write (the forward's mix), 3 reads + 2 non-temporal writes
+                   (the backward's): this machine's own streaming rates, GB/s
+  workloads        all ten measured workloads, forward+backward on one set of tensors and over
+                   sets in rotation (more than 1.5 GB, nothing reused): ms per step, the two
+                   kernels' shares, fraction of 8 TB/s
   rotating_sets    the same step over eight sets of tensors in rotation, so that no step finds its
                    inputs in the memory-side cache (`value` reuses one set, as the reference's
                    benchmark does); `--rotate 8` makes that the timed region itself
@@ -79,6 +92,9 @@ def parse_args():
                          "one cache-clearing write before every timed call as triton's do_bench does; one JSON line")
     ap.add_argument("--sweep-bs", type=int, default=8)
     ap.add_argument("--sweep-d", type=int, default=1024)
+    ap.add_argument("--no-workloads", action="store_true",
+                    help="skip the table of all ten workloads (profiler runs: its launches would be averaged "
+                         "into the kernels' statistics)")
     ap.add_argument("--copy-mb", type=int, default=0,
                     help="run only the library's plain copy kernel on this many MiB, --steps times "
                          "(hardware counters of the scan kernels are scaled by what they read for it)")
@@ -140,6 +156,142 @@ def sweep(args, torch, scan_cu, dev) -> int:
         "sweep": rows,
     }))
     return 0
+
+
+def frac_of_machine(machine, key, nbytes, kernel_ms):
+    """The kernel's rate over tensor sets in rotation as a fraction of the plain streaming kernel's
+    on the same buffers with the same mix of reads and writes."""
+    if not machine or not kernel_ms:
+        return None
+    return round(nbytes / (kernel_ms * 1e-3) / 1e9 / machine[key], 4)
+
+
+def machine_stream_leg(lib, _native, torch, pointer_sets, tensor_bytes, sp):
+    """What this machine streams: the library's plain streaming kernel (fss_stream_mix) over the
+    tensor sets of the rotation - every launch meets buffers that were last touched seven launches
+    (several GB) ago - with the forward's mix of streams (reads alpha, beta; writes h), the
+    backward's (reads alpha, h, dout; writes grad_alpha, grad_beta) and reads only."""
+    sink = torch.zeros(16, dtype=torch.uint8, device="cuda")
+    mixes = {
+        "read_only_GBps": (lambda p: ([p[0], p[1], p[2]], [])),
+        "fwd_mix_GBps": (lambda p: ([p[0], p[1]], [p[3]])),
+        "bwd_mix_GBps": (lambda p: ([p[0], p[3], p[2]], [p[4], p[5]])),
+    }
+    out = {"tensor_sets": len(pointer_sets), "bytes_per_stream": tensor_bytes,
+           "kernel": "fss::stream_mix_kernel<reads, writes, non-temporal writes>, 16 B per lane, linear"}
+    n_launches = 4 * len(pointer_sets)
+    for name, pick in mixes.items():
+        def run(n):
+            for i in range(n):
+                reads, writes = pick(pointer_sets[i % len(pointer_sets)])
+                _native.stream_mix(reads, writes, tensor_bytes, True, sp, sink.data_ptr())
+        run(len(pointer_sets))
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        run(n_launches)
+        torch.cuda.synchronize()
+        ms = (time.perf_counter() - t0) * 1e3 / n_launches
+        reads, writes = pick(pointer_sets[0])
+        out[name] = round((len(reads) + len(writes)) * tensor_bytes / (ms * 1e-3) / 1e9, 1)
+        out[name.replace("_GBps", "_ms_per_launch")] = round(ms, 5)
+    return out
+
+
+def measure_workload(lib, _native, torch, dev, case):
+    """One measured workload, briefly: forward+backward through the C ABI with the library's own
+    choices, on one set of tensors (as the reference's benchmark loops) and over enough sets in
+    rotation that nothing is found in a cache again (more than 1.5 GB).  Inputs are drawn on the
+    device with the workload's recipe; their values only matter to the timing through the recipe.
+    Kernel times are the kernels' shares of the wall time per step (split as HIP events around
+    16 sampled steps see the two launches)."""
+    from fast_sequential_scan_amd.workloads import BASELINE_CASES
+
+    recipe, bs, seq, d = BASELINE_CASES[case]
+    n = bs * seq * d
+    gen = torch.Generator(device=dev).manual_seed(sum(case.encode()))
+    x = torch.randn(bs, seq, d, device=dev, generator=gen)
+    beta = torch.randn(bs, seq, d, device=dev, generator=gen)
+    if recipe == "normal":
+        alpha = x
+    elif recipe == "sigmoid_plus2":
+        alpha = torch.sigmoid(x + 2.0)
+    else:
+        alpha = torch.sigmoid(x)
+    if recipe == "hawk":
+        beta = beta * torch.sqrt(1.0 - alpha * alpha)
+    alpha, beta = alpha.to(torch.bfloat16), beta.to(torch.bfloat16)
+    dout = torch.randn(bs, seq, d, device=dev, generator=gen).to(torch.bfloat16)
+    del x
+    per_set = 6 * n * 2
+    n_sets = min(64, max(3, -(-(3 << 29) // per_set)))
+    sets = [(alpha, beta, dout, torch.empty_like(alpha), torch.empty_like(alpha), torch.empty_like(alpha))]
+    for _ in range(n_sets - 1):
+        sets.append((alpha.clone(), beta.clone(), dout.clone(), torch.empty_like(alpha), torch.empty_like(alpha),
+                     torch.empty_like(alpha)))
+    ptrs = [tuple(t.data_ptr() for t in ts) for ts in sets]
+    stream = torch.cuda.current_stream()
+    sp = stream.cuda_stream
+    code = _native.FSS_BF16
+    ws_bytes = max(lib.fss_workspace_bytes(bs, seq, d, code, _native.FSS_FWD, None),
+                   lib.fss_workspace_bytes(bs, seq, d, code, _native.FSS_BWD, None))
+    ws = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
+    _native.check(lib.fss_workspace_init(ws.data_ptr(), ws.numel(), sp))
+    pws = ws.data_ptr()
+
+    def step(p):
+        pa, pb, pd, ph, pga, pgb = p
+        rc = lib.fss_scan_fwd_ex(code, pa, pb, ph, bs, seq, d, pws, ws_bytes, sp, None)
+        if rc == 0:
+            rc = lib.fss_scan_bwd_ex(code, pa, ph, pd, pga, pgb, bs, seq, d, pws, ws_bytes, sp, None)
+        if rc:
+            _native.check(rc)
+
+    def timed(rotate, n_steps):
+        k = len(ptrs) if rotate else 1
+        for i in range(max(5, k)):
+            step(ptrs[i % k])
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for i in range(n_steps):
+            step(ptrs[i % k])
+        torch.cuda.synchronize()
+        ms = (time.perf_counter() - t0) * 1e3 / n_steps
+        evs = [[torch.cuda.Event(enable_timing=True) for _ in range(3)] for _ in range(16)]
+        for i, e in enumerate(evs):
+            pa, pb, pd, ph, pga, pgb = ptrs[i % k]
+            e[0].record(stream)
+            _native.check(lib.fss_scan_fwd_ex(code, pa, pb, ph, bs, seq, d, pws, ws_bytes, sp, None))
+            e[1].record(stream)
+            _native.check(lib.fss_scan_bwd_ex(code, pa, ph, pd, pga, pgb, bs, seq, d, pws, ws_bytes, sp, None))
+            e[2].record(stream)
+        torch.cuda.synchronize()
+        f = statistics.fmean(e[0].elapsed_time(e[1]) for e in evs)
+        b = statistics.fmean(e[1].elapsed_time(e[2]) for e in evs)
+        return ms, ms * f / (f + b), ms * b / (f + b)
+
+    step_bytes = 16 * n
+    n_steps = int(max(30, min(300, 0.012 / (step_bytes / 5.5e12 + 15e-6))))  # about 12 ms of GPU time per leg
+    ms, f_ms, b_ms = timed(False, n_steps)
+    rms, rf_ms, rb_ms = timed(True, max(n_steps // 2, 2 * n_sets))
+    _native.check(lib.fss_workspace_status(pws, sp))
+    cf, cb = _native.FssConfig(), _native.FssConfig()
+    lib.fss_choose_config(bs, seq, d, code, _native.FSS_FWD, 16, ctypes.byref(cf))
+    lib.fss_choose_config(bs, seq, d, code, _native.FSS_BWD, 16, ctypes.byref(cb))
+
+    def frac(nbytes, t_ms):
+        return round(nbytes / (t_ms * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4)
+
+    return {
+        "case": case, "bs": bs, "seq": seq, "d_model": d, "recipe": recipe,
+        "launch_config_fwd": [cf.vec, cf.steps, cf.waves], "launch_config_bwd": [cb.vec, cb.steps, cb.waves],
+        "ms_per_step": round(ms, 5), "fwd_ms": round(f_ms, 5), "bwd_ms": round(b_ms, 5),
+        "GBps": round(step_bytes / (ms * 1e-3) / 1e9, 1), "frac": frac(step_bytes, ms),
+        "fwd_frac": frac(6 * n, f_ms), "bwd_frac": frac(10 * n, b_ms),
+        "no_reuse": {"tensor_sets": n_sets, "ms_per_step": round(rms, 5), "fwd_ms": round(rf_ms, 5),
+                     "bwd_ms": round(rb_ms, 5), "frac": frac(step_bytes, rms),
+                     "fwd_frac": frac(6 * n, rf_ms), "bwd_frac": frac(10 * n, rb_ms)},
+        "frac_no_reuse": frac(step_bytes, rms),
+    }
 
 
 def main() -> int:
@@ -376,7 +528,12 @@ def main() -> int:
         bwd_raw += [b for _, b in more]
     fwd_ms = [max(t - event_overhead, 1e-6) for t in fwd_raw]
     bwd_ms = [max(t - event_overhead, 1e-6) for t in bwd_raw]
-    fwd_mean, bwd_mean = statistics.fmean(fwd_ms), statistics.fmean(bwd_ms)
+    fwd_corr, bwd_corr = statistics.fmean(fwd_ms), statistics.fmean(bwd_ms)
+    # the kernels' shares of the wall time per step, split as the events see the two launches:
+    # they add up to ms_per_step, launch gaps included
+    raw_f, raw_b = statistics.fmean(fwd_raw), statistics.fmean(bwd_raw)
+    fwd_mean = ms_per_step * raw_f / (raw_f + raw_b)
+    bwd_mean = ms_per_step * raw_b / (raw_f + raw_b)
     step_bytes = (fwd_bytes_per_elem + bwd_bytes_per_elem) * n_elem
     value = step_bytes / (ms_per_step * 1e-3) / 1e9
     bwd_gbps = bwd_bytes_per_elem * n_elem / (bwd_mean * 1e-3) / 1e9
@@ -385,6 +542,7 @@ def main() -> int:
     # ---- the same step over eight tensor sets in rotation (nothing reused between steps), unless
     # the timed region above already rotated; reported next to `value`, never as `value` ----
     rotating = {}
+    machine = None
     if len(pointer_sets) == 1 and args.flush_mb > 0:
         extra = [(alpha.clone(), beta.clone(), dout.clone(), torch.empty_like(h), torch.empty_like(h),
                   torch.empty_like(h)) for _ in range(7)]
@@ -405,19 +563,23 @@ def main() -> int:
             torch.cuda.synchronize()
             rot_ms = (time.perf_counter() - t0) * 1e3 / n_rot
             rot = launch_pair_samples(32)
-            rot_fwd = statistics.fmean(max(f - event_overhead, 1e-6) for f, _ in rot)
-            rot_bwd = statistics.fmean(max(b - event_overhead, 1e-6) for _, b in rot)
+            rf, rb = statistics.fmean(f for f, _ in rot), statistics.fmean(b for _, b in rot)
+            rot_fwd, rot_bwd = rot_ms * rf / (rf + rb), rot_ms * rb / (rf + rb)  # shares of the wall time, as above
             return {"tensor_sets": len(pointer_sets), "steps": n_rot, "ms_per_step": round(rot_ms, 5),
                     "GBps": round(step_bytes / (rot_ms * 1e-3) / 1e9, 1),
                     "pct_of_hbm_peak": round(100.0 * step_bytes / (rot_ms * 1e-3) / 1e9 / HBM_PEAK_GBPS, 2),
                     "fwd_ms": round(rot_fwd, 5), "bwd_ms": round(rot_bwd, 5),
+                    "fwd_ms_events_corrected": round(max(rf - event_overhead, 1e-6), 5),
+                    "bwd_ms_events_corrected": round(max(rb - event_overhead, 1e-6), 5),
                     "fwd_frac": round(fwd_bytes_per_elem * n_elem / (rot_fwd * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4),
                     "bwd_frac": round(bwd_bytes_per_elem * n_elem / (rot_bwd * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4)}
 
         rotating = rotating_leg()
+        if not gated and not cm:
+            machine = machine_stream_leg(lib, _native, torch, pointer_sets, alpha.numel() * alpha.element_size(), sp)
         if args.cache_policy == "auto" and not cm:
             # the same rotation as a caller would run it who knows that nothing is reused
-            # (fss_set_cache_policy(FSS_CACHE_STREAMING)); bit-identical results
+            # (fss_set_cache_policy(FSS_CACHE_STREAMING): other cache hints, same tiling, same bits)
             ext.set_cache_policy("streaming")
             try:
                 rotating["streaming_policy"] = rotating_leg()
@@ -507,6 +669,13 @@ def main() -> int:
             torch.cuda.synchronize()
             autograd_inline_ms = (time.perf_counter() - t0) * 1e3 / n_auto
             autograd_inline_cpu_ms = (t_enqueued - t0) * 1e3 / n_auto
+
+    # ---- every measured workload, briefly (the headline run only) ----
+    workloads = None
+    if args.case == "C3_4096" and args.dtype == "bf16" and args.op == "scan" and not args.no_workloads \
+            and args.rotate == 1 and fwd_cfg is None and bwd_cfg is None:
+        del tensor_sets[1:]
+        workloads = [measure_workload(lib, _native, torch, dev, case) for case in BASELINE_CASES]
 
     # ---- CPU baseline + parity of this very run ----
     cpu = None
@@ -636,8 +805,10 @@ def main() -> int:
         "event_samples_in_timed_region": in_region,
         "event_pair_overhead_ms": round(event_overhead, 5),
         "event_pair_empty_ms": round(empty_pair, 5),
-        "fwd_ms_event_raw": round(statistics.fmean(fwd_raw), 5),
-        "bwd_ms_event_raw": round(statistics.fmean(bwd_raw), 5),
+        "fwd_ms_event_raw": round(raw_f, 5),
+        "bwd_ms_event_raw": round(raw_b, 5),
+        "fwd_ms_events_corrected": round(fwd_corr, 5),
+        "bwd_ms_events_corrected": round(bwd_corr, 5),
         "roofline": {
             "bound": "hbm",
             "kernel": f"{'cm_' if cm else ''}scan_kernel<{kname},...,BWD=true{',GATED' if gated else ''}> (backward scan)",
@@ -646,9 +817,12 @@ def main() -> int:
             "unit": "GB/s",
             "frac": round(bwd_gbps / HBM_PEAK_GBPS, 4),
             "frac_no_reuse": rotating.get("bwd_frac"),
+            "frac_of_machine": frac_of_machine(machine, "bwd_mix_GBps", bwd_bytes_per_elem * n_elem, rotating.get("bwd_ms")),
             "traffic": traffic["bwd"],
             "bytes_per_launch": bwd_bytes_per_elem * n_elem,
             "avg_launch_ms": round(bwd_mean, 5),
+            "avg_launch_ms_events_raw": round(raw_b, 5),
+            "avg_launch_ms_events_corrected": round(bwd_corr, 5),
         },
         "roofline_fwd": {
             "bound": "hbm",
@@ -658,10 +832,15 @@ def main() -> int:
             "unit": "GB/s",
             "frac": round(fwd_gbps / HBM_PEAK_GBPS, 4),
             "frac_no_reuse": rotating.get("fwd_frac"),
+            "frac_of_machine": frac_of_machine(machine, "fwd_mix_GBps", fwd_bytes_per_elem * n_elem, rotating.get("fwd_ms")),
             "traffic": traffic["fwd"],
             "bytes_per_launch": fwd_bytes_per_elem * n_elem,
             "avg_launch_ms": round(fwd_mean, 5),
+            "avg_launch_ms_events_raw": round(raw_f, 5),
+            "avg_launch_ms_events_corrected": round(fwd_corr, 5),
         },
+        "machine_stream": machine,
+        "workloads": workloads,
         "cold_cache": cold,
         "rotating_sets": rotating,
         "autograd_path_ms_per_step": None if autograd_ms is None else round(autograd_ms, 5),

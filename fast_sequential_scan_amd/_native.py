@@ -34,6 +34,7 @@ EXPORTED_SYMBOLS = (
     "fss_workspace_attach_flag",
     "fss_debug_set_spin_limit",
     "fss_debug_tile_groups",
+    "fss_debug_noalloc_reinit_after",
     "fss_debug_chain_plan",
     "fss_debug_chain_anchor",
     "fss_scan_fwd_noalloc",
@@ -55,6 +56,7 @@ EXPORTED_SYMBOLS = (
     "fss_scan_fwd_cm",
     "fss_scan_bwd_cm",
     "fss_copy_bytes",
+    "fss_stream_mix",
 )
 
 
@@ -105,6 +107,8 @@ def _declare(lib: ctypes.CDLL) -> None:
     lib.fss_debug_set_spin_limit.restype = ctypes.c_uint32
     lib.fss_debug_set_spin_limit.argtypes = [ctypes.c_uint32]
     lib.fss_debug_tile_groups.argtypes = [ctypes.c_int32, ctypes.c_int32, ctypes.c_int32, ctypes.POINTER(ctypes.c_int32)]
+    lib.fss_debug_noalloc_reinit_after.restype = ctypes.c_uint64
+    lib.fss_debug_noalloc_reinit_after.argtypes = [ctypes.c_uint64]
     lib.fss_debug_chain_plan.restype = _int
     lib.fss_debug_chain_plan.argtypes = [_i64, _i64, _i64, _int, _int, _sz, _cfgp, ctypes.POINTER(ctypes.c_int32)]
     lib.fss_debug_chain_anchor.restype = ctypes.c_int32
@@ -147,6 +151,8 @@ def _declare(lib: ctypes.CDLL) -> None:
     lib.fss_scan_bwd_cm.restype = _int
     lib.fss_scan_bwd_cm.argtypes = [_int, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _vp, _sz, _vp, _cfgp]
     lib.fss_copy_bytes.argtypes = [_vp, _vp, _sz, _vp]
+    lib.fss_stream_mix.restype = _int
+    lib.fss_stream_mix.argtypes = [ctypes.POINTER(_vp), _int, ctypes.POINTER(_vp), _int, _sz, _int, _vp]
 
 
 def lib() -> ctypes.CDLL:
@@ -177,6 +183,14 @@ def check(status: int) -> None:
         if hip:
             msg += f" (hipError_t {hip})"
         raise FssError(status, msg)
+
+
+def stream_mix(reads, writes, nbytes: int, nontemporal_writes: bool, stream_handle: int, sink: int = 0) -> None:
+    """fss_stream_mix over lists of device addresses; `sink`: 16 writable bytes for a read-only run."""
+    rd = (_vp * len(reads))(*reads)
+    wr_list = list(writes) if writes else [sink]
+    wr = (_vp * len(wr_list))(*wr_list)
+    check(lib().fss_stream_mix(rd, len(reads), wr, len(writes), nbytes, int(nontemporal_writes), stream_handle))
 
 
 def make_config(cfg: Optional[Tuple[int, int, int]]):

@@ -28,6 +28,46 @@ __global__ void copy_kernel(const u32x4 *__restrict__ src, u32x4 *__restrict__ d
     dst[i] = src[i];
 }
 
+// Calibration: the plainest kernel that moves a scan's mix of streams - R buffers read, W written,
+// each lane 16 bytes at a time, linearly, no dependence between elements.  What it reaches is
+// what this machine's memory system gives a kernel with that read/write mix; the scan kernels
+// are judged against it as well as against the nominal peak.  out0 = XOR of the reads,
+// out1 = ~out0 (so that every load is used and the result can be checked).
+struct StreamMixArgs {
+  const u32x4 *rd[3];
+  u32x4 *wr[2];
+  size_t n_vec;
+};
+template <int R, int W, bool NT>
+__global__ __launch_bounds__(256) void stream_mix_kernel(const StreamMixArgs a) {
+  const size_t stride = static_cast<size_t>(gridDim.x) * blockDim.x;
+  for (size_t i = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x; i < a.n_vec; i += stride) {
+    u32x4 v = a.rd[0][i];
+    if (R > 1) v ^= a.rd[1][i];
+    if (R > 2) v ^= a.rd[2][i];
+    if (W > 0) {
+      if (NT) __builtin_nontemporal_store(v, a.wr[0] + i); else a.wr[0][i] = v;
+    }
+    if (W > 1) {
+      if (NT) __builtin_nontemporal_store(~v, a.wr[1] + i); else a.wr[1][i] = ~v;
+    }
+    if (W == 0) {
+      // read-only: the loads must not be optimised away; the store never happens in practice
+      // (the caller passes a 16-byte sink for the one value that would trigger it)
+      if (v.x == 0x9e3779b9u && v.y == 0x7f4a7c15u && v.z == 0xf39cc060u && v.w == 0x5cedc834u) a.wr[0][0] = v;
+    }
+  }
+}
+
+template <int R, int W>
+static void launch_stream_mix(const StreamMixArgs &a, bool nt, hipStream_t stream) {
+  const dim3 grid(2048), block(256);
+  if (nt)
+    hipLaunchKernelGGL((stream_mix_kernel<R, W, true>), grid, block, 0, stream, a);
+  else
+    hipLaunchKernelGGL((stream_mix_kernel<R, W, false>), grid, block, 0, stream, a);
+}
+
 int g_cache_policy = FSS_CACHE_AUTO;  // fss_set_cache_policy
 uint32_t g_spin_limit = kSpinLimit;    // fss_debug_set_spin_limit
 
@@ -42,8 +82,18 @@ static __device__ __align__(256) unsigned char scratch[FSS_NOALLOC_SCRATCH_BYTES
 struct ScratchSlot {
   std::mutex lock;
   void *ptr = nullptr;
+  uint64_t launches = 0;  // chained or not: an upper bound on how far the array's launch tag has advanced
+  uint32_t *flag = nullptr;  // host-visible word attached through fss_workspace_attach_flag(NULL, ...)
 };
 static ScratchSlot g_scratch[64];
+
+// The validity tags of the chaining words are a 32-bit launch counter kept in the array itself.
+// A caller's workspace is re-initialised by its owner before the counter can wrap; nobody but
+// the library can reach this array, so the library counts the launches through it and zeroes it
+// again (a fill kernel on the call's stream: nothing is allocated) long before that.  Without
+// this, words left behind by an earlier, larger shape could carry a live tag again after the wrap.
+constexpr uint64_t kScratchReinitAfter = 1ull << 31;
+static uint64_t g_scratch_reinit_after = kScratchReinitAfter;  // fss_debug_noalloc_reinit_after
 
 // Address of the current device's copy of `scratch`; looked up at the first call on that
 // device.  The same set-up creates the event that orders scans across streams, so that no
@@ -78,6 +128,51 @@ static int scratch_of_current_device(void **out) {
   return FSS_OK;
 }
 
+static int launch_workspace_init(void *workspace, size_t bytes, hipStream_t stream) {
+  const size_t n_words = bytes / 4;
+  size_t blocks = (n_words + 255) / 256;
+  if (blocks > 4096) blocks = 4096;
+  hipLaunchKernelGGL(workspace_init_kernel, dim3(static_cast<uint32_t>(blocks)), dim3(256), 0, stream,
+                     static_cast<uint32_t *>(workspace), n_words);
+  const hipError_t e = hipGetLastError();
+  if (e != hipSuccess) {
+    tls_hip_error = static_cast<int>(e);
+    return FSS_ERR_LAUNCH;
+  }
+  return FSS_OK;
+}
+
+static int launch_workspace_attach(void *workspace, uint32_t *flag, hipStream_t stream) {
+  hipLaunchKernelGGL(workspace_attach_kernel, dim3(1), dim3(1), 0, stream, static_cast<uint32_t *>(workspace),
+                     static_cast<uint64_t>(reinterpret_cast<uintptr_t>(flag)));
+  const hipError_t e = hipGetLastError();
+  if (e != hipSuccess) {
+    tls_hip_error = static_cast<int>(e);
+    return FSS_ERR_LAUNCH;
+  }
+  return FSS_OK;
+}
+
+// Counts one launch through the current device's scratch array and, when the count says that
+// its launch tag could come near wrapping, zeroes the array on `stream` first (and attaches the
+// host-visible word again).  The fill is ordered against scans on other streams like a scan.
+static int count_scratch_launch(void *ptr, hipStream_t stream) {
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return FSS_ERR_LAUNCH;
+  ScratchSlot &slot = g_scratch[dev];
+  uint32_t *flag = nullptr;
+  {
+    std::lock_guard<std::mutex> guard(slot.lock);
+    if (++slot.launches <= __atomic_load_n(&g_scratch_reinit_after, __ATOMIC_RELAXED)) return FSS_OK;
+    slot.launches = 1;
+    flag = slot.flag;
+  }
+  const ScanOrderGuard ordered(stream);
+  int rc = launch_workspace_init(ptr, FSS_NOALLOC_SCRATCH_BYTES, stream);
+  if (rc == FSS_OK && flag) rc = launch_workspace_attach(ptr, flag, stream);
+  return rc;
+}
+
 int run_scan(int dtype, int dir, const void *alpha, const void *in_b, const void *in_h, void *out0,
              void *out1, int64_t bs, int64_t seq, int64_t d, void *workspace, size_t workspace_bytes,
              void *stream, const fss_config *cfg, const float *state_in = nullptr,
@@ -101,7 +196,7 @@ int run_scan(int dtype, int dir, const void *alpha, const void *in_b, const void
   const bool streaming = __atomic_load_n(&g_cache_policy, __ATOMIC_RELAXED) == FSS_CACHE_STREAMING;
   const bool with_state = state_in || state_out || h_before;
   Plan pl;
-  int rc = make_plan(pl, bs, seq, d, dtype, plan_dir, align, cfg, streaming && !with_state);
+  int rc = make_plan(pl, bs, seq, d, dtype, plan_dir, align, cfg);
   if (rc != FSS_OK) return rc;
   if (pl.n_chunks > 1) {
     if (!workspace || workspace_bytes < pl.ws_bytes) return FSS_ERR_WORKSPACE_SMALL;
@@ -192,15 +287,11 @@ size_t fss_workspace_bytes(int64_t bs, int64_t seq, int64_t d, int dtype, int di
   // The tensors' alignment is unknown here and changes the plan (less aligned tensors take
   // fewer channels per lane, which can mean more, smaller tiles and more chaining words):
   // the answer covers every alignment.
-  // ... and either cache policy (the streaming one may take two column tiles per workgroup, whose
-  // chunks are half as long)
   size_t best = fss::kHeaderBytes;
-  for (size_t align = 2; align <= 16; align <<= 1)
-    for (int two = 0; two < 2; ++two) {
-      fss::Plan pl;
-      if (fss::make_plan(pl, bs, seq, d, dtype, dir, align, cfg, two != 0) == FSS_OK && pl.ws_bytes > best)
-        best = pl.ws_bytes;
-    }
+  for (size_t align = 2; align <= 16; align <<= 1) {
+    fss::Plan pl;
+    if (fss::make_plan(pl, bs, seq, d, dtype, dir, align, cfg) == FSS_OK && pl.ws_bytes > best) best = pl.ws_bytes;
+  }
   return best;
 }
 
@@ -208,12 +299,11 @@ size_t fss_workspace_bytes_max(int64_t bs, int64_t seq, int64_t d) {
   size_t best = fss::kHeaderBytes;
   for (int dtype = FSS_BF16; dtype <= FSS_F16; ++dtype)
     for (int dir = FSS_FWD; dir <= FSS_GATED_BWD; ++dir)
-      for (size_t align = 2; align <= 16; align <<= 1)
-        for (int two = 0; two < 2; ++two) {
-          fss::Plan pl;
-          if (fss::make_plan(pl, bs, seq, d, dtype, dir, align, nullptr, two != 0) == FSS_OK && pl.ws_bytes > best)
-            best = pl.ws_bytes;
-        }
+      for (size_t align = 2; align <= 16; align <<= 1) {
+        fss::Plan pl;
+        if (fss::make_plan(pl, bs, seq, d, dtype, dir, align, nullptr) == FSS_OK && pl.ws_bytes > best)
+          best = pl.ws_bytes;
+      }
   return best;
 }
 
@@ -221,8 +311,7 @@ int fss_choose_config(int64_t bs, int64_t seq, int64_t d, int dtype, int dir, si
                       fss_config *out) {
   if (!out) return FSS_ERR_NULL_POINTER;
   fss::Plan pl;
-  const bool streaming = __atomic_load_n(&fss::g_cache_policy, __ATOMIC_RELAXED) == FSS_CACHE_STREAMING;
-  const int rc = fss::make_plan(pl, bs, seq, d, dtype, dir, align_bytes ? align_bytes : 16, nullptr, streaming);
+  const int rc = fss::make_plan(pl, bs, seq, d, dtype, dir, align_bytes ? align_bytes : 16, nullptr);
   if (rc == FSS_OK) *out = pl.cfg;
   return rc;
 }
@@ -231,31 +320,28 @@ int fss_workspace_init(void *workspace, size_t bytes, void *stream) {
   if (!workspace) return FSS_ERR_NULL_POINTER;
   if (bytes < fss::kHeaderBytes) return FSS_ERR_WORKSPACE_SMALL;
   if (reinterpret_cast<uintptr_t>(workspace) % 256 != 0 || bytes % 4 != 0) return FSS_ERR_MISALIGNED;
-  const size_t n_words = bytes / 4;
-  size_t blocks = (n_words + 255) / 256;
-  if (blocks > 4096) blocks = 4096;
-  hipLaunchKernelGGL(fss::workspace_init_kernel, dim3(static_cast<uint32_t>(blocks)), dim3(256), 0,
-                     static_cast<hipStream_t>(stream), static_cast<uint32_t *>(workspace), n_words);
-  const hipError_t e = hipGetLastError();
-  if (e != hipSuccess) {
-    fss::tls_hip_error = static_cast<int>(e);
-    return FSS_ERR_LAUNCH;
-  }
-  return FSS_OK;
+  return fss::launch_workspace_init(workspace, bytes, static_cast<hipStream_t>(stream));
 }
 
 int fss_workspace_attach_flag(void *workspace, uint32_t *flag, void *stream) {
-  if (!workspace) return FSS_ERR_NULL_POINTER;
   if (reinterpret_cast<uintptr_t>(workspace) % 256 != 0 || reinterpret_cast<uintptr_t>(flag) % 4 != 0)
     return FSS_ERR_MISALIGNED;
-  hipLaunchKernelGGL(fss::workspace_attach_kernel, dim3(1), dim3(1), 0, static_cast<hipStream_t>(stream),
-                     static_cast<uint32_t *>(workspace), static_cast<uint64_t>(reinterpret_cast<uintptr_t>(flag)));
-  const hipError_t e = hipGetLastError();
-  if (e != hipSuccess) {
-    fss::tls_hip_error = static_cast<int>(e);
-    return FSS_ERR_LAUNCH;
+  if (!workspace) {
+    // the static array of fss_scan_fwd_noalloc on the current device; remembered, so that the
+    // word stays attached when the library zeroes that array again
+    const int rc = fss::scratch_of_current_device(&workspace);
+    if (rc != FSS_OK) return rc;
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return FSS_ERR_LAUNCH;
+    std::lock_guard<std::mutex> guard(fss::g_scratch[dev].lock);
+    fss::g_scratch[dev].flag = flag;
   }
-  return FSS_OK;
+  return fss::launch_workspace_attach(workspace, flag, static_cast<hipStream_t>(stream));
+}
+
+uint64_t fss_debug_noalloc_reinit_after(uint64_t launches) {
+  if (launches == 0) launches = fss::kScratchReinitAfter;
+  return __atomic_exchange_n(&fss::g_scratch_reinit_after, launches, __ATOMIC_RELAXED);
 }
 
 int fss_debug_tile_groups(int32_t n_groups, int32_t grid, int32_t n_tiles, int32_t *groups) {
@@ -272,8 +358,7 @@ int fss_debug_chain_plan(int64_t bs, int64_t seq, int64_t d, int dtype, int dir,
                          const fss_config *cfg, int32_t *out) {
   if (!out) return FSS_ERR_NULL_POINTER;
   fss::Plan pl;
-  const bool streaming = __atomic_load_n(&fss::g_cache_policy, __ATOMIC_RELAXED) == FSS_CACHE_STREAMING;
-  const int rc = fss::make_plan(pl, bs, seq, d, dtype, dir, align_bytes ? align_bytes : 16, cfg, streaming);
+  const int rc = fss::make_plan(pl, bs, seq, d, dtype, dir, align_bytes ? align_bytes : 16, cfg);
   if (rc != FSS_OK) return rc;
   const int look = fss::look_waves(pl.cfg.waves, pl.cfg.vec, pl.cfg.cols);
   const int period = fss::chain_period(pl.n_groups, pl.cfg.waves);
@@ -298,7 +383,10 @@ uint32_t fss_debug_set_spin_limit(uint32_t polls) {
 }
 
 int fss_workspace_status(void *workspace, void *stream) {
-  if (!workspace) return FSS_ERR_NULL_POINTER;
+  if (!workspace) {  // the static array of fss_scan_fwd_noalloc on the current device
+    const int rc = fss::scratch_of_current_device(&workspace);
+    if (rc != FSS_OK) return rc;
+  }
   hipStream_t s = static_cast<hipStream_t>(stream);
   uint32_t hdr[4] = {0, 0, 0, 0};
   hipError_t e = hipMemcpyAsync(hdr, workspace, sizeof(hdr), hipMemcpyDeviceToHost, s);
@@ -329,7 +417,9 @@ int fss_scan_fwd_noalloc(int dtype, const void *alpha, const void *beta, void *h
   if (bs == 0 || seq == 0 || d == 0) return FSS_OK;
   if (fss_workspace_bytes(bs, seq, d, dtype, FSS_FWD, nullptr) > FSS_NOALLOC_SCRATCH_BYTES) return FSS_ERR_TOO_LARGE;
   void *ptr = nullptr;
-  const int rc = fss::scratch_of_current_device(&ptr);
+  int rc = fss::scratch_of_current_device(&ptr);
+  if (rc != FSS_OK) return rc;
+  rc = fss::count_scratch_launch(ptr, static_cast<hipStream_t>(stream));
   if (rc != FSS_OK) return rc;
   return fss::run_scan(dtype, FSS_FWD, alpha, beta, nullptr, h, nullptr, bs, seq, d, ptr, FSS_NOALLOC_SCRATCH_BYTES,
                        stream, nullptr);
@@ -446,6 +536,44 @@ int fss_copy_bytes(const void *src, void *dst, size_t bytes, void *stream) {
   hipLaunchKernelGGL(fss::copy_kernel, dim3(static_cast<uint32_t>(blocks)), dim3(256), 0,
                      static_cast<hipStream_t>(stream), static_cast<const fss::u32x4 *>(src),
                      static_cast<fss::u32x4 *>(dst), n_vec);
+  const hipError_t e = hipGetLastError();
+  if (e != hipSuccess) {
+    fss::tls_hip_error = static_cast<int>(e);
+    return FSS_ERR_LAUNCH;
+  }
+  return FSS_OK;
+}
+
+int fss_stream_mix(const void *const *reads, int n_reads, void *const *writes, int n_writes, size_t bytes,
+                   int nontemporal_writes, void *stream) {
+  if (!reads || n_reads < 1 || n_reads > 3 || n_writes < 0 || n_writes > 2) return FSS_ERR_BAD_CONFIG;
+  if (!writes) return FSS_ERR_NULL_POINTER;  // (read-only runs still name one 16-byte sink)
+  if (bytes % 16 != 0) return FSS_ERR_MISALIGNED;
+  fss::StreamMixArgs a = {{nullptr, nullptr, nullptr}, {nullptr, nullptr}, bytes / 16};
+  for (int i = 0; i < n_reads; ++i) {
+    if (!reads[i]) return FSS_ERR_NULL_POINTER;
+    if (reinterpret_cast<uintptr_t>(reads[i]) % 16 != 0) return FSS_ERR_MISALIGNED;
+    a.rd[i] = static_cast<const fss::u32x4 *>(reads[i]);
+  }
+  for (int i = 0; i < (n_writes > 0 ? n_writes : 1); ++i) {
+    if (!writes[i]) return FSS_ERR_NULL_POINTER;
+    if (reinterpret_cast<uintptr_t>(writes[i]) % 16 != 0) return FSS_ERR_MISALIGNED;
+    a.wr[i] = static_cast<fss::u32x4 *>(writes[i]);
+  }
+  if (bytes == 0) return FSS_OK;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  const bool nt = nontemporal_writes != 0;
+  switch (n_reads * 10 + n_writes) {
+    case 10: fss::launch_stream_mix<1, 0>(a, nt, s); break;
+    case 11: fss::launch_stream_mix<1, 1>(a, nt, s); break;
+    case 12: fss::launch_stream_mix<1, 2>(a, nt, s); break;
+    case 20: fss::launch_stream_mix<2, 0>(a, nt, s); break;
+    case 21: fss::launch_stream_mix<2, 1>(a, nt, s); break;
+    case 22: fss::launch_stream_mix<2, 2>(a, nt, s); break;
+    case 30: fss::launch_stream_mix<3, 0>(a, nt, s); break;
+    case 31: fss::launch_stream_mix<3, 1>(a, nt, s); break;
+    default: fss::launch_stream_mix<3, 2>(a, nt, s); break;
+  }
   const hipError_t e = hipGetLastError();
   if (e != hipSuccess) {
     fss::tls_hip_error = static_cast<int>(e);

@@ -93,27 +93,6 @@ struct Rung {
   int64_t need;
 };
 
-// Column tiles a workgroup covers side by side (fss_config.cols) when the caller leaves the
-// choice open; vec, steps and waves of `c` are already fixed.  `two_ok`: the caller of the
-// planner has a kernel for two (plain scan without state) and expects nothing to be found in
-// the caches again (FSS_CACHE_STREAMING).  Two column tiles make every row a workgroup touches
-// 512 contiguous bytes.  Measured in the forward with 4 bytes per lane, 32 steps and 16 waves
-// over tensor sets in rotation (49 shapes, bs 2..16, seq 2048..16384, d 512..4096): where the
-// launch has at most two tiles per CU, 5-13 % faster on 8 shapes of 9 (bs 8 seq 4096 d 1024:
-// 51.2 -> 44.5 us); with four tiles per CU +-0, with eight 1 % slower; when the tensors are
-// found in the memory-side cache again (forward and backward alternating on one set of tensors)
-// 7 % slower; in the backward, whose chunks then halve to 128 steps, slower throughout.
-inline int choose_cols(const fss_config &c, int64_t bs, int64_t seq, int64_t d, int dtype, int dir, bool gated,
-                       bool two_ok) {
-  if (!two_ok || gated || dir != FSS_FWD) return 1;
-  const int esize = dtype != FSS_F32 ? 2 : 4;
-  if (c.vec * esize != 4 || c.steps != 32 || c.waves != 16) return 1;
-  const int64_t tiles_per_row = ceil_div(d, 64 * static_cast<int64_t>(c.vec));
-  if (tiles_per_row % 2 != 0) return 1;
-  const int64_t tiles = bs * tiles_per_row * ceil_div(seq, static_cast<int64_t>(c.steps) * c.waves);
-  return tiles > kCus && tiles <= 2 * kCus ? 2 : 1;
-}
-
 // Fills the zero fields of `c`.  `align` is the common alignment in bytes of all
 // tensors of the call.
 //
@@ -127,7 +106,7 @@ inline int choose_cols(const fss_config &c, int64_t bs, int64_t seq, int64_t d, 
 // is halved at each rung is what the sweeps decided.  Below the last rung the problem
 // is latency-bound and the smallest tile is as good as any.
 inline void complete_config(fss_config &c, int64_t bs, int64_t seq, int64_t d, int dtype, int dir,
-                     size_t align, bool gated = false, bool two_ok = false) {
+                     size_t align, bool gated = false) {
   const bool narrow = dtype != FSS_F32;  // 16-bit storage
   const int esize = narrow ? 2 : 4;
   // two channels per lane: even d, 2-element alignment, and never pad a row to twice its width
@@ -221,7 +200,15 @@ inline void complete_config(fss_config &c, int64_t bs, int64_t seq, int64_t d, i
   c.vec = pick.vec;
   c.steps = pick.steps;
   c.waves = pick.waves;
-  if (!c.cols) c.cols = choose_cols(c, bs, seq, d, dtype, dir, gated, two_ok);
+  // Two column tiles per workgroup (rows of 512 contiguous bytes, chunks half as long) are never
+  // the library's own choice: measured in the forward with 4 bytes per lane, 32 steps and 16 waves
+  // they are 4-13 % faster where a launch has at most two tiles per CU and nothing is found in a
+  // cache (bs 8 seq 4096 d 1024: 42.9 -> 41.2 us over tensor sets in rotation), 5-7 % slower when
+  // the tensors are found in the memory-side cache again (30.8 -> 32.4 us), and slower throughout
+  // in the backward, whose chunks would shrink to 128 steps.  The library cannot know which of
+  // the two it is in, and a different tiling rounds the carries differently, so it stays an
+  // explicit configuration.
+  if (!c.cols) c.cols = 1;
 }
 
 struct Plan {
@@ -233,9 +220,8 @@ struct Plan {
   size_t ws_bytes;
 };
 
-// `two_columns_ok`: the library may choose two column tiles per workgroup (see choose_cols).
 inline int make_plan(Plan &pl, int64_t bs, int64_t seq, int64_t d, int dtype, int dir, size_t align,
-              const fss_config *user, bool two_columns_ok = false) {
+              const fss_config *user) {
   if (bs < 0 || seq < 0 || d < 0) return FSS_ERR_BAD_SHAPE;
   if (dtype != FSS_BF16 && dtype != FSS_F32 && dtype != FSS_F16) return FSS_ERR_BAD_CONFIG;
   if (dir < FSS_FWD || dir > FSS_GATED_BWD) return FSS_ERR_BAD_CONFIG;
@@ -251,7 +237,7 @@ inline int make_plan(Plan &pl, int64_t bs, int64_t seq, int64_t d, int dtype, in
   if (user) c = *user;
   if (c.max_groups < 0 || c.cols < 0) return FSS_ERR_BAD_CONFIG;
   const int64_t dd = d > 0 ? d : 1, ss = seq > 0 ? seq : 1, bb = bs > 0 ? bs : 1;
-  complete_config(c, bb, ss, dd, dtype, dir, align, gated, two_columns_ok);
+  complete_config(c, bb, ss, dd, dtype, dir, align, gated);
   if (!config_valid(c, dtype, gated, dir)) return FSS_ERR_BAD_CONFIG;
   if (dd % c.vec != 0) return FSS_ERR_BAD_CONFIG;
   if (align % (static_cast<size_t>(c.vec) * esize) != 0) return FSS_ERR_MISALIGNED;

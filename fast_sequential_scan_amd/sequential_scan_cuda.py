@@ -37,6 +37,11 @@ _CODE_DTYPE = {code: dtype for dtype, code in _DTYPE_CODE.items()}
 # one workspace per (device, stream): calls on one stream are ordered, calls on
 # different streams must not share the chaining words
 _workspaces: Dict[Tuple[int, int], "_Workspace"] = {}
+# workspaces replaced by larger ones: their host-side words (the pinned time-out flag, the launch
+# count) stay alive for the rest of the process, because scans already enqueued may still set the
+# flag and a backward on an autograd thread may have looked the old entry up just before it was
+# replaced; only the device buffer goes back to the allocator (its reuse is ordered by the stream)
+_retired: List["_Workspace"] = []
 
 # the validity tags in a workspace are a 32-bit launch counter: reset long before it wraps
 _REINIT_AFTER_LAUNCHES = 1 << 31
@@ -175,12 +180,17 @@ def _workspace(device: torch.device, stream: "_RawStream", need: int) -> "_Works
     if ws is None or ws.size < need:
         if ws is not None:
             ws.raise_if_flagged()
+        old = ws
         ws = _Workspace(torch.empty(max(need, 1 << 20), dtype=torch.uint8, device=device), stream.cuda_stream)
-        _workspaces[key] = ws
+        # the C++ dispatch learns of the new workspace before the old one lets go of anything
         binding = _torch_binding.loaded()
         if binding is not None:
             binding.register_workspace(
                 key[0], key[1], ws.ptr, ws.size, ws.flag.data_ptr(), ctypes.addressof(ws.launches))
+        _workspaces[key] = ws
+        if old is not None:
+            old.buf = None
+            _retired.append(old)
     else:
         if ws.flag_word.value:
             ws.raise_if_flagged()

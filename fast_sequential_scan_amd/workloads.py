@@ -6,6 +6,11 @@ The five recipes are the workload configurations this build is measured on:
   C3  bs 8, d 1024, seq in {512,1000,2048,3000,4096,8192}; alpha = sigmoid(N(0,1)), beta ~ N(0,1)
   C4  bs 4, seq 8192, d 2048; alpha = sigmoid(N(0,1)+2), beta ~ N(0,1)
   C5  bs 1, seq 65521 (prime), d 256; alpha = sigmoid(N(0,1)), beta ~ N(0,1)
+A sixth recipe, "near_one", is the long-memory regime of a trained Hawk / Griffin block:
+alpha = sigmoid(N(0,1)+6) (median 0.9975), beta = N(0,1)*sqrt(1-alpha^2).  In the five above
+the product of a chunk's few hundred alphas underflows or all but vanishes, so the state handed
+from chunk to chunk is just the previous chunk's own contribution; here that product is
+0.1-0.6 and the composed carries matter to every output.
 The upstream gradient is N(0,1) everywhere.  Values are drawn in fp32 on the CPU
 from a fixed seed and then rounded to the storage dtype, so the device kernel
 and the CPU oracle see bit-identical inputs.
@@ -16,7 +21,14 @@ from typing import Tuple
 
 import torch
 
-RECIPES = ("normal", "hawk", "sigmoid", "sigmoid_plus2")
+RECIPES = ("normal", "hawk", "sigmoid", "sigmoid_plus2", "near_one")
+
+# the long-memory recipe at the shapes of the three workloads with the longest chains
+LONG_MEMORY_CASES = {
+    "near_one_C3_4096": ("near_one", 8, 4096, 1024),
+    "near_one_C4": ("near_one", 4, 8192, 2048),
+    "near_one_C5": ("near_one", 1, 65521, 256),
+}
 
 BASELINE_CASES = {
     "C1": ("normal", 2, 1024, 768),
@@ -50,6 +62,9 @@ def make_inputs(
         alpha = torch.sigmoid(x)
     elif recipe == "sigmoid_plus2":
         alpha = torch.sigmoid(x + 2.0)
+    elif recipe == "near_one":
+        alpha = torch.sigmoid(x + 6.0)
+        beta = beta * torch.sqrt(1.0 - alpha * alpha)
     else:
         raise ValueError(recipe)
     return alpha.to(dtype), beta.to(dtype), dout.to(dtype)

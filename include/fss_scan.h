@@ -14,7 +14,22 @@
  * with |alpha| <= 1, the recurrence's regime, this matches the sequential order to fp32
  * rounding.  With |alpha| > 1 over long stretches A can overflow to inf; a state of exactly
  * 0 still stays 0 (as sequentially), but a tiny non-zero state times such an A is inf where
- * the sequential order might have stayed finite.
+ * the sequential order might have stayed finite.  A non-finite alpha is outside the contract:
+ * where it meets a state of exactly 0 the result is NaN inside a lane's slice of timesteps
+ * (as sequentially) and the zero state is kept at a slice or chunk boundary, so what comes
+ * out depends on the launch configuration.
+ *
+ * What is guaranteed about the bits.  The order in which the chunks' maps are composed is
+ * fixed by the shape and the launch configuration (fss_config: vec, steps, waves, cols) and
+ * by nothing else: not the timing of the workgroups, the stream, the cache policy, the number
+ * of workgroups launched (max_groups), the device's CU count, the workspace (the caller's or
+ * the static one of fss_scan_fwd_noalloc) or earlier calls.  So one call returns the same
+ * bits on every run, as the reference does by walking each channel with one thread
+ * (csrc/include/sequential_scan_kernel_bf16.cuh:121-151).  Two DIFFERENT configurations agree
+ * only to fp32 rounding of the carries (they cut the sequence at different places); where no
+ * chunk is needed (one wave covers the sequence) the result is the sequential one bit for bit
+ * given fused multiply-adds.  The configuration the library chooses by itself is a function
+ * of shape, dtype, direction and the tensors' common alignment (fss_choose_config).
  *
  * This header replaces, for a host written in any language, the pybind11 module
  * `sequential_scan_cuda` of the reference (csrc/sequential_scan.cpp:13-22) and
@@ -102,8 +117,9 @@ typedef enum fss_dir { FSS_FWD = 0, FSS_BWD = 1, FSS_GATED_FWD = 2, FSS_GATED_BW
  *          (waves/cols)*steps consecutive timesteps of 64*vec*cols channels at a time;
  *          two column tiles side by side make every row a workgroup touches 512
  *          contiguous bytes instead of 256, which the memory system serves faster
- * Results do not depend on the configuration beyond fp32 rounding of the
- * carries handed between chunks.
+ * Results depend on vec, steps, waves and cols only through fp32 rounding of the carries
+ * handed between chunks (a different tiling cuts the sequence at different places), and not at
+ * all on max_groups: see "What is guaranteed about the bits" above.
  */
 typedef struct fss_config {
   int32_t vec;
@@ -123,13 +139,14 @@ int fss_last_hip_error(void);
  * cfg may be NULL. */
 size_t fss_workspace_bytes(int64_t bs, int64_t seq, int64_t d, int dtype, int dir,
                            const fss_config *cfg);
-/* Upper bound over all directions (gated included), both dtypes and every
+/* Upper bound over all directions (gated included), all three dtypes and every
  * configuration the library may choose by itself. */
 size_t fss_workspace_bytes_max(int64_t bs, int64_t seq, int64_t d);
 /* Resets the workspace with a fill kernel on `stream` (graph-capturable). */
 int fss_workspace_init(void *workspace, size_t bytes, void *stream);
 /* Synchronises `stream`, then reports FSS_OK or FSS_ERR_CHAIN_TIMEOUT and clears
- * the sticky error word.  For tests and debugging. */
+ * the sticky error word.  For tests and debugging.  workspace = NULL stands for the static
+ * array of fss_scan_fwd_noalloc on the current device. */
 int fss_workspace_status(void *workspace, void *stream);
 /*
  * A chunk that gives up waiting (see FSS_ERR_CHAIN_TIMEOUT above) hands on a NaN state, so
@@ -138,8 +155,10 @@ int fss_workspace_status(void *workspace, void *stream);
  * 32-bit word that the device can write and the host can read (hipHostMalloc memory): a
  * kernel that gives up stores 1 there as well.  The host polls the word whenever it likes
  * (it is set by the time the kernel has finished) and clears it itself.  Asynchronous on
- * `stream` (a small kernel, graph-capturable); fss_workspace_init detaches the word; NULL
- * detaches it too.  No counterpart in the reference, whose kernels never wait.
+ * `stream` (a small kernel, graph-capturable); fss_workspace_init detaches the word; flag =
+ * NULL detaches it too.  workspace = NULL stands for the static array of fss_scan_fwd_noalloc
+ * on the current device (the word then stays attached when the library zeroes that array
+ * again).  No counterpart in the reference, whose kernels never wait.
  */
 int fss_workspace_attach_flag(void *workspace, uint32_t *flag, void *stream);
 /*
@@ -149,6 +168,11 @@ int fss_workspace_attach_flag(void *workspace, uint32_t *flag, void *stream);
  * Process-wide; returns the previous value.
  */
 uint32_t fss_debug_set_spin_limit(uint32_t polls);
+/*
+ * Test hook: after how many calls per device fss_scan_fwd_noalloc zeroes its static array again
+ * (default 2^31; 0 restores the default).  Process-wide; returns the previous value.
+ */
+uint64_t fss_debug_noalloc_reinit_after(uint64_t launches);
 /*
  * Test hook (host only, no device call): the order in which the row-major kernels take
  * their tiles.  Tiles are numbered chunk-major (tile = chunk * n_groups + slot) and workgroup b
@@ -230,7 +254,8 @@ int fss_scan_bwd_f32(const void *alpha, const void *h, const void *dout,
  *                        large model): the forward output always carries the streaming hint and
  *                        the backward always reads dout with it (measured 2-3 % faster then, 3 % slower in a loop
  *                        over one set of tensors).
- * Results are bit-identical under both.  Returns the previous policy, or -1 for an unknown one.
+ * The policy selects cache hints on loads and stores and nothing else - never the tiling - so
+ * results are bit-identical under both.  Returns the previous policy, or -1 for an unknown one.
  */
 enum fss_cache_policy { FSS_CACHE_AUTO = 0, FSS_CACHE_STREAMING = 1 };
 int fss_set_cache_policy(int policy);
@@ -244,10 +269,16 @@ int fss_set_cache_policy(int policy);
  * library or in the HIP runtime (the first call on a device looks up the array's address
  * and creates the event that orders scans across streams).  A shape whose
  * fss_workspace_bytes(.., FSS_FWD, NULL) exceeds the array is refused with
- * FSS_ERR_TOO_LARGE.  All calls on one GPU share that GPU's array: calls that can overlap
- * on one GPU race (within one process the library already orders scans across streams;
- * replays of different captured graphs and different processes are the caller's to keep
- * apart).  Results are bit-identical to fss_scan_fwd_ex.
+ * FSS_ERR_TOO_LARGE.  All calls of one process on one GPU share that GPU's array (another
+ * process has its own copy): calls that can overlap on one GPU race - the library already
+ * orders scans across streams; replays of different captured graphs are the caller's to keep
+ * apart.  Results are bit-identical to fss_scan_fwd_ex with cfg = NULL (same kernel, same
+ * plan; only where the chaining words live differs).  The validity tags of the array are a
+ * 32-bit launch counter like a workspace's; the library counts the calls through this entry
+ * point per device and zeroes the array again (a fill kernel on the call's stream) every 2^31
+ * calls, so a long-lived process never meets a wrapped tag.  A chain time-out is reported as
+ * for any workspace: fss_workspace_status(NULL, stream), or a word attached with
+ * fss_workspace_attach_flag(NULL, flag, stream).
  */
 #define FSS_NOALLOC_SCRATCH_BYTES (16u << 20)
 int fss_scan_fwd_noalloc(int dtype, const void *alpha, const void *beta, void *h, int64_t bs,
@@ -364,6 +395,21 @@ int fss_scan_bwd_cm(int dtype, const void *alpha, const void *h, const void *dou
  * scan kernels can be scaled by what the same counters read for a transfer of
  * known size. */
 int fss_copy_bytes(const void *src, void *dst, size_t bytes, void *stream);
+
+/*
+ * Calibration kernel: the plainest kernel that moves a scan's mix of streams.  Reads `n_reads`
+ * (1..3) buffers and writes `n_writes` (0..2) buffers of `bytes` bytes each (a multiple of 16;
+ * all pointers 16-byte aligned), linearly, 16 bytes per lane, with no dependence between
+ * elements; `nontemporal_writes` marks the stores as the scans mark theirs.  writes[0]
+ * receives the XOR of the reads, writes[1] its complement.  With n_writes = 0, writes[0] must
+ * still name 16 writable bytes (a sink that is not written in practice).  The forward scan's
+ * mix is 2 reads + 1 write, the backward's 3 reads + 2 writes: what this kernel reaches over
+ * buffers that fit no cache is what the machine's memory system gives that mix, and
+ * bench.py reports the scans against it next to the nominal 8 TB/s.  No counterpart in the
+ * reference.
+ */
+int fss_stream_mix(const void *const *reads, int n_reads, void *const *writes, int n_writes,
+                   size_t bytes, int nontemporal_writes, void *stream);
 
 #ifdef __cplusplus
 }

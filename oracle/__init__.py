@@ -172,6 +172,40 @@ def bf16_bits_to_f32(bits) -> np.ndarray:
     return out
 
 
+# ---- the HIP kernels' own composition order, restated sequentially (oracle/chained_model.c) ----
+
+
+def chained_scan_fwd(alpha, beta, steps: int, waves: int, period: int, look: int, span: int) -> np.ndarray:
+    """Forward scan composed exactly as the row-major HIP kernels compose it for a tiling of
+    `waves` slices of `steps` timesteps per chunk and the given chain plan.  uint16 arrays are
+    bf16 bit patterns (bf16 bits out), anything else is taken as float32 (float32 out)."""
+    bits = np.asarray(alpha).dtype == np.uint16
+    dt = np.uint16 if bits else np.float32
+    a, b = _c(alpha, dt), _c(beta, dt)
+    _same_shape(a, b)
+    h = np.empty_like(a)
+    fn = _load().chained_scan_fwd_bf16 if bits else _load().chained_scan_fwd_f32
+    rc = fn(_p(a), _p(b), _p(h), *_dims(a), *(ctypes.c_int(int(v)) for v in (steps, waves, period, look, span)))
+    if rc != 0:
+        raise ValueError("bad chain configuration")
+    return h
+
+
+def chained_scan_bwd(alpha, h, dout, steps: int, waves: int, period: int, look: int, span: int):
+    """(grad_alpha, grad_beta) composed as the row-major HIP backward composes them."""
+    bits = np.asarray(alpha).dtype == np.uint16
+    dt = np.uint16 if bits else np.float32
+    a, hh, do = _c(alpha, dt), _c(h, dt), _c(dout, dt)
+    _same_shape(a, hh, do)
+    ga, gb = np.empty_like(a), np.empty_like(a)
+    fn = _load().chained_scan_bwd_bf16 if bits else _load().chained_scan_bwd_f32
+    rc = fn(_p(a), _p(hh), _p(do), _p(ga), _p(gb), *_dims(a),
+            *(ctypes.c_int(int(v)) for v in (steps, waves, period, look, span)))
+    if rc != 0:
+        raise ValueError("bad chain configuration")
+    return ga, gb
+
+
 # torch <-> bit-pattern helpers (torch imported lazily: the oracle itself is NumPy)
 
 

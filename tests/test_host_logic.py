@@ -18,7 +18,7 @@ ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 
 def test_library_exports_every_declared_symbol():
     header = open(os.path.join(ROOT, "include", "fss_scan.h")).read()
-    declared = set(re.findall(r"^(?:int|size_t|uint32_t|int32_t|const char \*)\s*(fss_[a-z0-9_]+)\(", header, flags=re.M))
+    declared = set(re.findall(r"^(?:int|size_t|uint32_t|int32_t|uint64_t|const char \*)\s*(fss_[a-z0-9_]+)\(", header, flags=re.M))
     assert declared == set(_native.EXPORTED_SYMBOLS)
     lib = ctypes.CDLL(_native.LIB_PATH)
     for name in declared:
@@ -51,24 +51,23 @@ def test_workspace_sizing_and_config_choice():
                 need = lib.fss_workspace_bytes(bs, seq, d, dtype, direction, None)
                 assert need >= 4096 and need % 256 == 0
                 assert need <= lib.fss_workspace_bytes_max(bs, seq, d)
-                # the answer covers every alignment the tensors may have and either cache policy (under
-                # the streaming one a forward of at most two tiles per CU takes two column tiles per
-                # workgroup, whose chunks are half as long)
-                per_plan = []
+                # the answer covers every alignment the tensors may have; the cache policy selects
+                # hints on loads and stores, never the tiling, so it cannot change the plan
+                per_policy = []
                 for policy in (_native.FSS_CACHE_AUTO, _native.FSS_CACHE_STREAMING):
                     previous = lib.fss_set_cache_policy(policy)
                     try:
-                        per_plan += [plan_bytes(lib, bs, seq, d, dtype, direction, a)[0] for a in (2, 4, 8, 16) if a >= esize]
+                        per_policy.append([plan_bytes(lib, bs, seq, d, dtype, direction, a)[0] for a in (2, 4, 8, 16) if a >= esize])
                     finally:
                         lib.fss_set_cache_policy(previous)
-                assert need == max(per_plan)
-    # the forward at the headline shape (512 tiles: two per CU): two column tiles per workgroup under the
-    # streaming policy, one otherwise; never in the backward
-    for policy, cols in ((_native.FSS_CACHE_STREAMING, 2), (_native.FSS_CACHE_AUTO, 1)):
+                assert per_policy[0] == per_policy[1]
+                assert need == max(per_policy[0])
+    # two column tiles per workgroup are never the library's own choice, under either policy
+    for policy in (_native.FSS_CACHE_STREAMING, _native.FSS_CACHE_AUTO):
         previous = lib.fss_set_cache_policy(policy)
         try:
             assert lib.fss_choose_config(8, 4096, 1024, 0, 0, 16, ctypes.byref(cfg)) == 0
-            assert (cfg.vec, cfg.steps, cfg.waves, cfg.cols) == (2, 32, 16, cols)
+            assert (cfg.vec, cfg.steps, cfg.waves, cfg.cols) == (2, 32, 16, 1)
             assert lib.fss_choose_config(8, 4096, 1024, 0, 1, 16, ctypes.byref(cfg)) == 0 and cfg.cols == 1
             assert lib.fss_choose_config(8, 8192, 1024, 0, 0, 16, ctypes.byref(cfg)) == 0 and cfg.cols == 1
         finally:
@@ -447,3 +446,30 @@ def test_tile_order_covers_every_group_of_every_chunk_once():
     assert all(len(set(g[:, b].tolist())) == 4 for b in range(256))
     assert lib.fss_debug_tile_groups(0, 256, 0, (ctypes.c_int32 * 1)()) != 0
     assert lib.fss_debug_tile_groups(8, 8, 8, None) != 0
+
+
+def test_missing_cpp_dispatch_falls_back_to_the_python_wrappers(monkeypatch, tmp_path):
+    """The C++ dispatch only shortens the host's way to the launch: when its module is missing or
+    does not load, one warning is given and every call goes through the ctypes wrappers over the
+    same HIP library (which itself has no stand-in: test_missing_library_raises...).  With
+    FSS_TORCH_BINDING=1 the missing module is an error."""
+    from fast_sequential_scan_amd import _torch_binding as tb
+
+    monkeypatch.setattr(tb, "_module", None)
+    monkeypatch.setattr(tb, "_tried", False)
+    monkeypatch.setattr(tb, "PATH", str(tmp_path / "nowhere.so"))
+    monkeypatch.delenv("FSS_TORCH_BINDING", raising=False)
+    with pytest.warns(RuntimeWarning, match="C\\+\\+ dispatch is not available"):
+        assert tb.load(lambda *a: None) is None
+    assert tb.load(lambda *a: None) is None  # decided once: no second attempt, no second warning
+    # a file that is no extension module: same fallback
+    bad = tmp_path / "fss_torch_binding.so"
+    bad.write_bytes(b"not an ELF file")
+    monkeypatch.setattr(tb, "_tried", False)
+    monkeypatch.setattr(tb, "PATH", str(bad))
+    with pytest.warns(RuntimeWarning):
+        assert tb.load(lambda *a: None) is None
+    monkeypatch.setattr(tb, "_tried", False)
+    monkeypatch.setenv("FSS_TORCH_BINDING", "1")
+    with pytest.raises((tb.TorchBindingMissing, ImportError, OSError)):
+        tb.load(lambda *a: None)

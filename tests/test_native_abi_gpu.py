@@ -18,3 +18,34 @@ def test_plain_c_host_runs_the_scans():
     done = subprocess.run([BINARY], capture_output=True, text=True, timeout=100)
     assert done.returncode == 0, done.stdout + done.stderr
     assert done.stdout.startswith("abi_check ok"), done.stdout
+
+
+def test_stream_mix_calibration_kernel_moves_what_it_says():
+    """fss_stream_mix: writes[0] = XOR of the reads, writes[1] = its complement; read-only runs write nothing."""
+    import torch
+
+    from fast_sequential_scan_amd import _native
+
+    dev = "cuda:0"
+    n = 1 << 20
+    g = torch.Generator(device=dev).manual_seed(1)
+    reads = [torch.randint(-2**31, 2**31 - 1, (n,), dtype=torch.int32, device=dev, generator=g) for _ in range(3)]
+    sp = torch.cuda.current_stream().cuda_stream
+    for r in (1, 2, 3):
+        for w in (1, 2):
+            for nt in (False, True):
+                outs = [torch.zeros(n, dtype=torch.int32, device=dev) for _ in range(w)]
+                _native.stream_mix([t.data_ptr() for t in reads[:r]], [t.data_ptr() for t in outs], 4 * n, nt, sp)
+                want = reads[0].clone()
+                for t in reads[1:r]:
+                    want ^= t
+                torch.cuda.synchronize()
+                assert torch.equal(outs[0], want)
+                if w == 2:
+                    assert torch.equal(outs[1], ~want)
+    sink = torch.zeros(4, dtype=torch.int32, device=dev)
+    _native.stream_mix([t.data_ptr() for t in reads], [], 4 * n, True, sp, sink.data_ptr())
+    torch.cuda.synchronize()
+    assert int(sink.abs().sum()) == 0
+    lib = _native.lib()
+    assert lib.fss_stream_mix(None, 1, None, 0, 16, 0, None) != 0

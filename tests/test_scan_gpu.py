@@ -320,8 +320,9 @@ def test_fp32_at_headline_shape(oracle):
 
 
 def test_cache_policies_give_identical_results():
-    """The streaming policy only changes cache hints: every output bit stays.  Shapes on both sides
-    of the sizes at which the automatic policy switches."""
+    """The cache policy selects hints on loads and stores, never the tiling: every output bit stays.
+    Shapes on both sides of the sizes at which the automatic policy switches its hints (the same
+    with alphas near 1, where the composed carries matter: tests/test_determinism_gpu.py)."""
     import fast_sequential_scan_amd as pkg
 
     for shape in ((4, 1000, 512), (8, 4096, 1024)):

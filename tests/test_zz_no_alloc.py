@@ -73,3 +73,58 @@ def test_noalloc_forward_rejects_what_it_cannot_hold():
     assert lib.fss_scan_fwd_noalloc(7, p, p, p, 1, 4, 2, sp) == 5
     assert lib.fss_scan_fwd_noalloc(_native.FSS_BF16, p, p, p, 0, 4, 2, sp) == 0
     torch.cuda.synchronize()
+
+
+def test_noalloc_array_is_zeroed_again_before_its_launch_tag_can_wrap():
+    """The validity tags of the chaining words are a 32-bit launch counter kept in the array, and
+    nobody but the library can reset that array: it counts the calls per device and zeroes the
+    array again on the call's stream (nothing allocated) long before the counter wraps.  Here the
+    limit is lowered to 3 calls, so a row of calls on a large and a small shape crosses it several
+    times; alphas near 1, so that a stale or missing carry would show in every output."""
+    lib = _native.lib()
+    sp = torch.cuda.current_stream().cuda_stream
+    cases = []
+    for shape in ((8, 4096, 1024), (2, 1000, 328)):
+        alpha, beta, _ = make_inputs("near_one", *shape, seed=3 + sum(shape))
+        a, b = alpha.to(DEV), beta.to(DEV)
+        cases.append((a, b, _reference(lib, _native.FSS_BF16, a, b, sp)))
+    flag = torch.zeros(1, dtype=torch.int32).pin_memory()
+    _native.check(lib.fss_workspace_attach_flag(None, flag.data_ptr(), sp))
+    previous = lib.fss_debug_noalloc_reinit_after(3)
+    try:
+        outs = [(torch.full_like(cases[i % 2][0], float("nan")), cases[i % 2][2]) for i in range(11)]
+        torch.cuda.synchronize()
+        allocated = torch.cuda.memory_allocated()
+        for i, (out, _want) in enumerate(outs):
+            a, b, _ = cases[i % 2]
+            _native.check(lib.fss_scan_fwd_noalloc(_native.FSS_BF16, a.data_ptr(), b.data_ptr(), out.data_ptr(), *a.shape, sp))
+        torch.cuda.synchronize()
+        assert torch.cuda.memory_allocated() == allocated  # the zeroing in between allocates nothing either
+        for out, want in outs:
+            assert torch.equal(out, want)
+        assert lib.fss_workspace_status(None, sp) == 0 and int(flag[0]) == 0
+        # a chain time-out in that array is reported like one in a caller's workspace - through the
+        # status call and through the attached word, which survived the zeroing above
+        limit = lib.fss_debug_set_spin_limit(0)
+        try:
+            a, b, _want = cases[0]
+            out = torch.empty_like(a)
+            _native.check(lib.fss_scan_fwd_noalloc(_native.FSS_BF16, a.data_ptr(), b.data_ptr(), out.data_ptr(), *a.shape, sp))
+            torch.cuda.synchronize()
+        finally:
+            lib.fss_debug_set_spin_limit(limit)
+        assert int(flag[0]) == 1
+        assert lib.fss_workspace_status(None, sp) == _native.FSS_ERR_CHAIN_TIMEOUT
+        assert lib.fss_workspace_status(None, sp) == 0
+        assert bool(torch.isnan(out.float()).any())
+        flag[0] = 0
+        # and the array is good again at the next call
+        a, b, want = cases[1]
+        out = torch.empty_like(a)
+        _native.check(lib.fss_scan_fwd_noalloc(_native.FSS_BF16, a.data_ptr(), b.data_ptr(), out.data_ptr(), *a.shape, sp))
+        torch.cuda.synchronize()
+        assert torch.equal(out, want) and int(flag[0]) == 0
+    finally:
+        lib.fss_debug_noalloc_reinit_after(previous)
+        _native.check(lib.fss_workspace_attach_flag(None, None, sp))
+        torch.cuda.synchronize()
