@@ -14,10 +14,11 @@
  * with |alpha| <= 1, the recurrence's regime, this matches the sequential order to fp32
  * rounding.  With |alpha| > 1 over long stretches A can overflow to inf; a state of exactly
  * 0 still stays 0 (as sequentially), but a tiny non-zero state times such an A is inf where
- * the sequential order might have stayed finite.  A non-finite alpha is outside the contract:
- * where it meets a state of exactly 0 the result is NaN inside a lane's slice of timesteps
- * (as sequentially) and the zero state is kept at a slice or chunk boundary, so what comes
- * out depends on the launch configuration.
+ * the sequential order might have stayed finite.  An alpha that is itself +-inf or NaN makes
+ * exactly the outputs non-finite that the sequential order makes non-finite (that step and
+ * every later one of its channel); which of NaN and +-inf an output then holds can depend on
+ * the launch configuration (a composed map with an infinite coefficient can turn the
+ * sequential order's -inf into inf - inf = NaN).
  *
  * What is guaranteed about the bits.  The order in which the chunks' maps are composed is
  * fixed by the shape and the launch configuration (fss_config: vec, steps, waves, cols) and

@@ -187,3 +187,39 @@ def _with_policy(policy, fn):
         return fn()
     finally:
         pkg.set_cache_policy(previous)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32], ids=["bf16", "f32"])
+@pytest.mark.parametrize("cfg", [(1, 8, 2), (2, 16, 4), None], ids=str)
+def test_infinite_alpha_poisons_exactly_what_it_poisons_sequentially(oracle, dtype, cfg):
+    """alpha = +inf meeting a state of exactly 0 gives NaN, meeting anything else +-inf, and every
+    later state of that channel is NaN or +-inf - in the sequential loop
+    (sequential_scan/common.py:46-59) and here alike: the same elements are non-finite, nothing else
+    is touched, whether the inf sits inside a lane's slice of timesteps, on its first step or on the
+    first step of a chunk.  WHICH non-finite value comes out can differ: where the sequential order
+    keeps -inf, a composed map with an infinite coefficient can give inf - inf = NaN, so with a
+    non-finite alpha only the finiteness of an output is independent of the tiling.  (The
+    composition keeps a zero state at 0 when a PRODUCT of finite alphas overflowed, which the
+    sequential order also does: tests/test_scan_gpu.py's growing-recurrence case.)"""
+    bs, seq, d = 2, 600, 128
+    alpha, beta, dout = make_inputs("sigmoid", bs, seq, d, dtype=dtype, seed=31)
+    beta[:, :300, :64] = 0  # channels 0-63: the state is exactly 0 until step 300
+    steps = 8 if cfg is None else cfg[1]
+    for t in (16, 16 + 3, 128, 256 + steps, 299):  # chunk starts, slice starts and steps inside a slice, whatever the tiling
+        alpha[0, t, 0:2] = float("inf")      # meets 0 -> NaN
+        alpha[0, t, 64:66] = float("inf")    # meets a non-zero state -> +-inf
+    a, b = alpha.to(DEV), beta.to(DEV)
+    h = ext._forward(dtype, a, b, cfg)
+    ext.workspace_status()
+    if dtype == torch.bfloat16:
+        want = oracle.bf16_bits_to_f32(oracle.scan_fwd_bf16(as_model_array(alpha), as_model_array(beta), fused=True))
+    else:
+        want = oracle.scan_fwd_f32(alpha.numpy(), beta.numpy(), fused=True)
+    got = h.float().cpu().numpy()
+    assert np.array_equal(np.isfinite(got), np.isfinite(want))
+    assert np.isnan(got[0, 16:, 0]).all() and np.isfinite(got[0, :16, 0]).all()   # inf * 0: NaN in both
+    assert np.isinf(got[0, 16, 64]) and not np.isfinite(got[0, 16:, 64]).any()
+    finite = np.isfinite(want)
+    assert finite[1].all() and finite[0, :, 2:64].all() and finite[0, :, 66:].all()
+    tol = 1e-2 if dtype == torch.bfloat16 else 1e-4
+    assert np.allclose(got[finite], want[finite], rtol=tol, atol=tol)
