@@ -697,6 +697,13 @@ __device__ __forceinline__ void chain_chunks(const ScanArgs &p, const TileCtx &c
   }
   const int anchor = c.anchor;
   const int reach = c.look * c.span;  // chunks one round of the look-back covers
+  // Which wave asks which chunk: look index 0 asks the nearest chunk.  Where the waves issue loads
+  // of their own inside this phase (`mid`), the look-back is the work of the LAST waves (look
+  // index 0 = the last wave): wave 0 is busy composing and publishing the chunk's own map and
+  // would ask behind that and behind its own loads (bs 8 seq 4096 d 1024 bf16 backward 54.8 ->
+  // 54.0 us, 60.3 -> 58.4 us over tensor sets in rotation; the forward, which issues nothing
+  // here, measured 0.3-0.6 us slower that way and keeps the first waves).
+  const int li = HAS_MID ? c.n_waves - 1 - wave : wave;
   int nearest = c.chunk - 1;          // nearest earlier chunk not folded yet (>= anchor)
   // The first look goes out ahead of the loop, with `mid` in a straight line between the
   // issue of its loads and their use: only so does the compiler wait for exactly those
@@ -706,8 +713,8 @@ __device__ __forceinline__ void chain_chunks(const ScanArgs &p, const TileCtx &c
 #pragma unroll
   for (int v = 0; v < VEC; ++v) q0A[v] = q0B[v] = local_const(0.0f);
   if constexpr (HAS_MID) {
-    const int j0 = nearest - wave * c.span;
-    if (wave < c.look && j0 >= anchor && p.spin_limit != 0) {
+    const int j0 = nearest - li * c.span;
+    if (li < c.look && j0 >= anchor && p.spin_limit != 0) {
       ChunkWords<VEC> w;
       poll_issue<VEC>(p, c, j0, j0 == anchor, w);
       mid();
@@ -717,8 +724,8 @@ __device__ __forceinline__ void chain_chunks(const ScanArgs &p, const TileCtx &c
     }
   }
   for (;;) {
-    const int j = nearest - wave * c.span;
-    if (wave < c.look && j >= anchor) {
+    const int j = nearest - li * c.span;
+    if (li < c.look && j >= anchor) {
       float qA[VEC], qB[VEC];
 #pragma unroll
       for (int v = 0; v < VEC; ++v) {
@@ -739,7 +746,7 @@ __device__ __forceinline__ void chain_chunks(const ScanArgs &p, const TileCtx &c
         }
       }
 #pragma unroll
-      for (int v = 0; v < VEC; ++v) c.lds_pred[(wave * VEC + v) * 64 + lane] = make_float2(qA[v], qB[v]);
+      for (int v = 0; v < VEC; ++v) c.lds_pred[(li * VEC + v) * 64 + lane] = make_float2(qA[v], qB[v]);
     }
     __syncthreads();
     // every wave folds what the look-back waves found (the same few LDS reads in each wave
