@@ -449,6 +449,8 @@ struct TileCtx {
   float2 *lds_pred;      // [look wave][v][lane] = what that wave's earlier chunks do to a state
   int span;              // chunks one look-back wave covers: more than 1 when the sequence has more chunks than such waves
   int anchor;            // the earlier chunk whose outgoing state this chunk's chain starts from (chain_anchor)
+  uint32_t *s_ready;     // [wave] of this column tile: the number of the last tile whose map the wave has left in LDS
+  uint32_t tile_no;      // number of this tile among the workgroup's tiles, from 1
 #ifdef FSS_TRACE
   int trace_wave;
 #endif
@@ -548,71 +550,56 @@ __device__ __forceinline__ void await_chunk(const ScanArgs &p, const TileCtx &c,
   }
 }
 
-// (A, B) <- map[count-1] o ... o map[0] for this lane's channels: the maps of the
-// first `count` waves of the workgroup composed in scan order.  Reads go out in
-// small batches so that their LDS latencies overlap.
-template <int VEC>
-__device__ __forceinline__ void fold_wave_maps(const float2 *lds_map, int lane, int count, float *A,
-                                               float *B) {
-  constexpr int kBatch = 4;
-#pragma unroll
-  for (int v = 0; v < VEC; ++v) {
-    A[v] = 1.0f;
-    B[v] = 0.0f;
-  }
-  for (int w0 = 0; w0 < count; w0 += kBatch) {
-    float2 m[kBatch][VEC];
-#pragma unroll
-    for (int i = 0; i < kBatch; ++i) {
-      const int w = w0 + i < count ? w0 + i : count - 1;  // clamped: the read stays in bounds
-#pragma unroll
-      for (int v = 0; v < VEC; ++v) m[i][v] = lds_map[(w * VEC + v) * 64 + lane];
-    }
-#pragma unroll
-    for (int i = 0; i < kBatch; ++i) {
-      if (w0 + i < count) {
-#pragma unroll
-        for (int v = 0; v < VEC; ++v) {
-          B[v] = fma0(m[i][v].x, B[v], m[i][v].y);
-          A[v] *= m[i][v].x;
-        }
-      }
-    }
+// ---- hand-over of the waves' maps inside a workgroup ------------------------------------------
+//
+// A wave that has left its map in LDS says so in its word of `ready` (release; the number of the
+// tile, which only grows, so nothing is ever reset).  Wave 0 composes the maps in wave order as
+// they arrive, instead of behind a barrier that waits for the slowest wave before the first
+// map is touched: a wave's rows arrive microseconds apart, and when the last map lands the
+// others are already composed, so the chunk's map goes out a microsecond earlier - to every later
+// chunk that is waiting for it.
+__device__ __forceinline__ void announce_map(uint32_t *ready, int wave, uint32_t seq) {
+  __hip_atomic_store(ready + wave, seq, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_WORKGROUP);
+}
+__device__ __forceinline__ void await_map(const uint32_t *ready, int wave, uint32_t seq) {
+  // (wave-uniform address: one LDS word, broadcast)
+  while (__hip_atomic_load(ready + wave, __ATOMIC_ACQUIRE, __HIP_MEMORY_SCOPE_WORKGROUP) < seq)
+    __builtin_amdgcn_s_sleep(1);
+}
+// every wave of the column tile has left its map (lane l looks at wave l's word)
+__device__ __forceinline__ void await_all_maps(const uint32_t *ready, int lane, int n_waves, uint32_t seq) {
+  for (;;) {
+    const uint32_t r = lane < n_waves
+                           ? __hip_atomic_load(ready + lane, __ATOMIC_ACQUIRE, __HIP_MEMORY_SCOPE_WORKGROUP)
+                           : seq;
+    if (__builtin_amdgcn_ballot_w64(r < seq) == 0ull) return;
+    __builtin_amdgcn_s_sleep(1);
   }
 }
 
-// The same composition over all `count` waves, by one wave for the whole workgroup: slot w
-// receives what the waves before w do to the chunk's incoming state (the composition of maps
-// 0 .. w-1, in place of map w, which nobody else reads), and (A, B) the chunk's map.  Every
-// other wave then finds its prefix with one LDS read after the next barrier, instead of
-// composing up to 15 maps itself on the way to its last phase.  Same operations in the same
-// order as fold_wave_maps, so the results are bit for bit the same.
+// (A, B) <- map[count-1] o ... o map[0], composed by one wave for the whole workgroup as the maps
+// arrive: slot w receives what the waves before w do to the chunk's incoming state (the
+// composition of maps 0 .. w-1, in place of map w, which nobody else reads), and (A, B) the
+// chunk's map.  Every other wave then finds its prefix with one LDS read behind the next barrier.
+// The order of the composition is the waves' order, whatever the order of their arrival.
 template <int VEC>
-__device__ __forceinline__ void fold_and_leave_prefixes(float2 *lds_map, int lane, int count, float *A, float *B) {
-  constexpr int kBatch = 4;
+__device__ __forceinline__ void fold_arriving_maps(float2 *lds_map, const uint32_t *ready, uint32_t seq, int lane,
+                                                   int count, float *A, float *B) {
 #pragma unroll
   for (int v = 0; v < VEC; ++v) {
     A[v] = 1.0f;
     B[v] = 0.0f;
   }
-  for (int w0 = 0; w0 < count; w0 += kBatch) {
-    float2 m[kBatch][VEC];
+  for (int w = 0; w < count; ++w) {
+    if (w > 0) await_map(ready, w, seq);  // (slot 0 is this wave's own)
+    float2 m[VEC];
 #pragma unroll
-    for (int i = 0; i < kBatch; ++i) {
-      const int w = w0 + i < count ? w0 + i : count - 1;  // clamped: the read stays in bounds
+    for (int v = 0; v < VEC; ++v) m[v] = lds_map[(w * VEC + v) * 64 + lane];
 #pragma unroll
-      for (int v = 0; v < VEC; ++v) m[i][v] = lds_map[(w * VEC + v) * 64 + lane];
-    }
-#pragma unroll
-    for (int i = 0; i < kBatch; ++i) {
-      if (w0 + i < count) {
-#pragma unroll
-        for (int v = 0; v < VEC; ++v) {
-          lds_map[((w0 + i) * VEC + v) * 64 + lane] = make_float2(A[v], B[v]);
-          B[v] = fma0(m[i][v].x, B[v], m[i][v].y);
-          A[v] *= m[i][v].x;
-        }
-      }
+    for (int v = 0; v < VEC; ++v) {
+      lds_map[(w * VEC + v) * 64 + lane] = make_float2(A[v], B[v]);
+      B[v] = fma0(m[v].x, B[v], m[v].y);
+      A[v] *= m[v].x;
     }
   }
 }
@@ -620,17 +607,16 @@ __device__ __forceinline__ void fold_and_leave_prefixes(float2 *lds_map, int lan
 // Phase 2.  In: this wave's slice as the map x -> mA*x + mB.  Out: the state
 // entering the slice.  Every wave of the workgroup must call it (barriers).
 //
-// After one barrier wave 0 composes all the waves' maps into the chunk's map and
-// publishes it, leaving in every wave's slot the composition of the waves before it.
-// Meanwhile the look-back: the chunks from chunk-1 down to the anchor (chain_anchor) are
-// dealt out to the first `look` waves, `span` consecutive chunks each, nearest first; each
-// such wave waits for its chunks' maps (the anchor's outgoing state) and composes them, so a
+// Every wave leaves its map in LDS and says so (announce_map); wave 0 composes the maps into the
+// chunk's map as they arrive and publishes it, leaving in every wave's slot the composition of
+// the waves before it.  Meanwhile the look-back: the chunks from chunk-1 down to the anchor
+// (chain_anchor) are dealt out to `look` waves, `span` consecutive chunks each, nearest first;
+// each such wave waits for its chunks' maps (the anchor's outgoing state) and composes them, so a
 // look-back over look*span chunks costs `span` memory round trips instead of one per chunk.
-// After a second barrier every wave folds what the look-back waves left in LDS into the
-// chunk's incoming state itself (a few multiply-adds: cheaper than a third barrier and a
+// After the one barrier of the phase every wave folds what the look-back waves left in LDS into
+// the chunk's incoming state itself (a few multiply-adds: cheaper than another barrier and a
 // broadcast), wave 0 also publishes the chunk's outgoing state, and every wave applies the
-// composition of the waves before it (one LDS read; the first chunk of a sequence, which has
-// no second barrier to wait at, composes it itself).  A chain of more than look*span chunks
+// composition of the waves before it (one LDS read).  A chain of more than look*span chunks
 // repeats the look-back.  Who looks at which chunk, and the order of every composition, depend
 // on the chunk's index and the plan alone.
 //
@@ -644,43 +630,49 @@ __device__ __forceinline__ void chain_chunks(const ScanArgs &p, const TileCtx &c
   const int lane = c.lane, wave = c.wave;
 #pragma unroll
   for (int v = 0; v < VEC; ++v) c.lds_map[(wave * VEC + v) * 64 + lane] = make_float2(mA[v], mB[v]);
-  __syncthreads();
+  announce_map(c.s_ready, wave, c.tile_no);
   FSS_STAMP(c, p, 2);
 
   const bool look_back = c.chained && c.chunk > 0;
   uint64_t *mine = nullptr;
   float cA[VEC], cB[VEC];
-  if (wave == 0 && look_back) {
+  if (wave == 0) {
     // the chunk's own map, needed by later chunks: out as early as possible - and on the way
-    // every wave's prefix, left where its map was (the waves read it behind the look-back's barrier)
-    fold_and_leave_prefixes<VEC>(c.lds_map, lane, c.n_waves, cA, cB);
-    mine = p.words + (static_cast<size_t>(c.chunk) * p.n_ctiles + c.ctile) * 3 * kLaneSlots + lane;
-    if (!c.last) {
+    // every wave's prefix, left where its map was (the waves read it behind the next barrier)
+    fold_arriving_maps<VEC>(c.lds_map, c.s_ready, c.tile_no, lane, c.n_waves, cA, cB);
+    if (c.chained && !c.last) {
+      mine = p.words + (static_cast<size_t>(c.chunk) * p.n_ctiles + c.ctile) * 3 * kLaneSlots + lane;
+      if (look_back) {
 #pragma unroll
-      for (int v = 0; v < VEC; ++v) {
-        st_word(mine + (0 * VEC + v) * 64, c.tag, cA[v]);
-        st_word(mine + (1 * VEC + v) * 64, c.tag, cB[v]);
+        for (int v = 0; v < VEC; ++v) {
+          st_word(mine + (0 * VEC + v) * 64, c.tag, cA[v]);
+          st_word(mine + (1 * VEC + v) * 64, c.tag, cB[v]);
+        }
+      } else {
+        // first chunk of a chained sequence: nobody asks for its map, only for its outgoing state
+#pragma unroll
+        for (int v = 0; v < VEC; ++v)
+          st_word(mine + (2 * VEC + v) * 64, c.tag, seq_in ? fma0(cA[v], seq_in[v], cB[v]) : cB[v]);
       }
     }
-  } else if (wave == 0 && c.chained && !c.last) {
-    // first chunk of a chained sequence: its map is needed for its outgoing state only (the
-    // other waves compose their prefixes themselves: no barrier follows that they could wait at)
-    fold_wave_maps<VEC>(c.lds_map, lane, c.n_waves, cA, cB);
-    mine = p.words + (static_cast<size_t>(c.chunk) * p.n_ctiles + c.ctile) * 3 * kLaneSlots + lane;
   }
   FSS_STAMP(c, p, 3);
 
   // (pA, pB): what the waves before this one do to the chunk's incoming state
   float pA[VEC], pB[VEC];
   if (!look_back) {
-    if constexpr (HAS_MID) mid();
-    fold_wave_maps<VEC>(c.lds_map, lane, wave, pA, pB);
     // first chunk of the sequence (or the only one): the incoming state is the
     // sequence's own (0 in the plain scan)
-    if (wave == 0 && c.chained && !c.last) {
+    if constexpr (HAS_MID) {
+      if (wave != 0) await_all_maps(c.s_ready, lane, c.n_waves, c.tile_no);  // (as below: not before the others' rows are in)
+      mid();
+    }
+    __syncthreads();  // wave 0 has left every wave's prefix
 #pragma unroll
-      for (int v = 0; v < VEC; ++v)
-        st_word(mine + (2 * VEC + v) * 64, c.tag, seq_in ? fma0(cA[v], seq_in[v], cB[v]) : cB[v]);
+    for (int v = 0; v < VEC; ++v) {
+      const float2 e = c.lds_map[(wave * VEC + v) * 64 + lane];
+      pA[v] = e.x;
+      pB[v] = e.y;
     }
 #pragma unroll
     for (int v = 0; v < VEC; ++v) state[v] = seq_in ? fma0(pA[v], seq_in[v], pB[v]) : pB[v];
@@ -712,9 +704,16 @@ __device__ __forceinline__ void chain_chunks(const ScanArgs &p, const TileCtx &c
   float q0A[VEC], q0B[VEC];
 #pragma unroll
   for (int v = 0; v < VEC; ++v) q0A[v] = q0B[v] = local_const(0.0f);
+  // The look-back starts once every wave of the column tile has its rows (the chunks it asks run
+  // in step with this one: asking earlier only polls for longer).  Waves with loads of their own
+  // to issue here wait for that moment too (issued while the other waves' rows are still on
+  // their way, those loads only delay them: bs 8 seq 4096 d 1024 backward 53.5 -> 56.4 us); the
+  // rest go straight on to the barrier.
+  const bool looks = li < c.look && nearest - li * c.span >= anchor;
+  if (looks || (HAS_MID && wave != 0)) await_all_maps(c.s_ready, lane, c.n_waves, c.tile_no);
   if constexpr (HAS_MID) {
     const int j0 = nearest - li * c.span;
-    if (li < c.look && j0 >= anchor && p.spin_limit != 0) {
+    if (looks && p.spin_limit != 0) {
       ChunkWords<VEC> w;
       poll_issue<VEC>(p, c, j0, j0 == anchor, w);
       mid();

@@ -195,6 +195,7 @@ __device__ __forceinline__ void cm_tile(const ScanArgs &p, const TileCtx &c, int
 template <typename E, int VEC, int ROWS, bool BWD>
 __global__ __launch_bounds__(1024) void cm_scan_kernel(const ScanArgs p) {
   extern __shared__ float lds[];
+  __shared__ uint32_t s_ready[16];  // per wave: see announce_map
 
   TileCtx c;
   c.wcol = 0;
@@ -206,6 +207,9 @@ __global__ __launch_bounds__(1024) void cm_scan_kernel(const ScanArgs p) {
   float2 *const lds_maps = reinterpret_cast<float2 *>(lds);  // laid out as in scan_kernel with one slot per lane
   c.lds_pred = lds_maps + 2 * c.n_waves * 64;
   c.seq = p.seq;
+  c.s_ready = s_ready;
+  if (threadIdx.x < 16) s_ready[threadIdx.x] = 0u;
+  __syncthreads();
   c.row_bytes = 0;
   c.lane_off = 0;
   c.col_ok = true;
@@ -217,7 +221,9 @@ __global__ __launch_bounds__(1024) void cm_scan_kernel(const ScanArgs p) {
   c.tag = c.chained ? __builtin_amdgcn_readfirstlane(ld_u32(p.hdr + HDR_EPOCH)) + 1u : 0u;
 
   uint32_t parity = 0;
+  uint32_t tile_no = 0;
   for (uint32_t tile = blockIdx.x; tile < static_cast<uint32_t>(p.n_tiles); tile += gridDim.x, parity ^= 1u) {
+    c.tile_no = ++tile_no;
     c.lds_map = lds_maps + parity * c.n_waves * 64;
     const uint32_t chunk = __builtin_amdgcn_readfirstlane(tile / static_cast<uint32_t>(p.n_ctiles));
     const uint32_t ctile = tile - chunk * static_cast<uint32_t>(p.n_ctiles);

@@ -459,6 +459,7 @@ __global__ __launch_bounds__(MAXW * 64) void scan_kernel(const ScanArgs p, const
   constexpr int kLaneSlots = 64 * VEC;  // channels per tile
 
   extern __shared__ float lds[];
+  __shared__ uint32_t s_ready[2 * 16];  // per column tile and wave: see announce_map
 
   // The waves of a workgroup: wg_cols column tiles side by side, each with n_waves waves
   // that take consecutive time slices.  Everything the chain phase touches is per column tile.
@@ -480,6 +481,9 @@ __global__ __launch_bounds__(MAXW * 64) void scan_kernel(const ScanArgs p, const
   c.lds_pred = lds_maps + (2 * waves_total + c.wcol * c.look) * kLaneSlots;
   c.seq = p.seq;
   c.row_bytes = p.d * E::kBytes;
+  c.s_ready = s_ready + c.wcol * 16;
+  if (threadIdx.x < 2 * 16) s_ready[threadIdx.x] = 0u;
+  __syncthreads();
 #ifdef FSS_TRACE
   c.trace_wave = FSS_TRACE_WAVE < 0 ? c.n_waves - 1 : FSS_TRACE_WAVE;
 #endif
@@ -505,7 +509,9 @@ __global__ __launch_bounds__(MAXW * 64) void scan_kernel(const ScanArgs p, const
   const TileOrder order = tile_order(static_cast<uint32_t>(p.n_groups), gridDim.x);
   const uint32_t n_groups = order.n_groups;
   uint32_t parity = 0;
+  uint32_t tile_no = 0;
   for (uint32_t tile = blockIdx.x; tile < static_cast<uint32_t>(p.n_tiles); tile += gridDim.x, parity ^= 1u) {
+    c.tile_no = ++tile_no;
     c.lds_map = lds_maps + (parity * waves_total + c.wcol * c.n_waves) * kLaneSlots;
     // unsigned, wave-uniform arithmetic: stays on the scalar unit
     // (the compiler divides through a vector-unit reciprocal: pin the quotients back)
