@@ -283,7 +283,7 @@ def measure_workload(lib, _native, torch, dev, case):
 
     return {
         "case": case, "bs": bs, "seq": seq, "d_model": d, "recipe": recipe,
-        "launch_config_fwd": [cf.vec, cf.steps, cf.waves], "launch_config_bwd": [cb.vec, cb.steps, cb.waves],
+        "launch_config_fwd": [cf.vec, cf.steps, cf.waves, cf.cols], "launch_config_bwd": [cb.vec, cb.steps, cb.waves, cb.cols],
         "ms_per_step": round(ms, 5), "fwd_ms": round(f_ms, 5), "bwd_ms": round(b_ms, 5),
         "GBps": round(step_bytes / (ms * 1e-3) / 1e9, 1), "frac": frac(step_bytes, ms),
         "fwd_frac": frac(6 * n, f_ms), "bwd_frac": frac(10 * n, b_ms),
@@ -439,7 +439,8 @@ def main() -> int:
             c.waves = min(8, -(-seq // (64 * c.vec)))
         else:
             lib.fss_choose_config(bs, seq, d, fss_dtype, direction, 16, ctypes.byref(c))
-        chosen[name] = list(user) if user else [c.vec, c.steps, c.waves]
+        chosen[name] = list(user[:3]) if user else [c.vec, c.steps, c.waves]
+        chosen[name + "_cols"] = (user[4] if user and len(user) > 4 and user[4] else 1) if (user or cm) else c.cols
 
     # ---- warm-up, then the timed region: exactly K steps between two synchronisations ----
     for _ in range(args.warmup):
@@ -767,7 +768,7 @@ def main() -> int:
             scale_r = part["copy"]["bytes_read"] / (part["copy"]["fetch_kib"] * 1024.0)
             scale_w = part["copy"]["bytes_written"] / (part["copy"]["write_kib"] * 1024.0)
             for name in ("fwd", "bwd"):
-                if part[name]["config"] == chosen[name]:
+                if part[name]["config"] == chosen[name] and part[name].get("cols", 1) == chosen[name + "_cols"]:
                     traffic[name] = int(part[name]["fetch_kib"] * 1024 * scale_r + part[name]["write_kib"] * 1024 * scale_w)
     except (OSError, KeyError, ValueError):
         pass
@@ -794,6 +795,7 @@ def main() -> int:
             "bs": bs, "seq": seq, "d_model": d,
             "launch_config_fwd_vec_steps_waves": chosen["fwd"],
             "launch_config_bwd_vec_steps_waves": chosen["bwd"],
+            "column_tiles_per_workgroup_fwd_bwd": [chosen["fwd_cols"], chosen["bwd_cols"]],
         },
         "pct_of_hbm_peak": round(100.0 * value / HBM_PEAK_GBPS, 2),
         "pct_of_hbm_peak_no_reuse": rotating.get("pct_of_hbm_peak"),

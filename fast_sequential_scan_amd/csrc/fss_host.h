@@ -93,6 +93,30 @@ struct Rung {
   int64_t need;
 };
 
+// Column tiles a workgroup covers side by side (fss_config.cols) when the caller leaves the
+// choice open; vec, steps and waves of `c` are already fixed.  Two column tiles make every row a
+// workgroup touches 512 contiguous bytes instead of 256 and its chunks half as long.  Measured in
+// the forward with 4 bytes per lane, 32 steps and 16 waves (bf16, 49 shapes, bs 2..16, seq
+// 2048..16384, d 512..4096, tensor sets in rotation so that nothing is found in a cache): where
+// the launch has more than one and at most two tiles per CU, 5-13 % faster on 8 shapes of 9;
+// with four tiles per CU +-0, with eight 1 % slower; in the backward, whose chunks would shrink
+// to 128 steps, slower throughout.  At bs 8 seq 4096 d 1024: forward 42.8 -> 40.9 us and the
+// forward+backward step 105.4 -> 103.3 us over tensor sets in rotation, a forward behind flushed
+// caches 48.2 -> 45.6 us; when the tensors are found in the memory-side cache again (forward and
+// backward alternating on one set of tensors) forward 31.0 -> 32.2 us, step 88.6 -> 90.5 us.  The
+// library cannot know which of the two it is in and takes what serves the caller whose tensors
+// come from memory.  The choice depends on the shape alone - never on a policy or on earlier
+// calls - because a different tiling rounds the carries differently.
+inline int choose_cols(const fss_config &c, int64_t bs, int64_t seq, int64_t d, int dtype, int dir, bool gated) {
+  if (gated || dir != FSS_FWD) return 1;
+  const int esize = dtype != FSS_F32 ? 2 : 4;
+  if (c.vec * esize != 4 || c.steps != 32 || c.waves != 16) return 1;
+  const int64_t tiles_per_row = ceil_div(d, 64 * static_cast<int64_t>(c.vec));
+  if (tiles_per_row % 2 != 0) return 1;
+  const int64_t tiles = bs * tiles_per_row * ceil_div(seq, static_cast<int64_t>(c.steps) * c.waves);
+  return tiles > kCus && tiles <= 2 * kCus ? 2 : 1;
+}
+
 // Fills the zero fields of `c`.  `align` is the common alignment in bytes of all
 // tensors of the call.
 //
@@ -200,15 +224,7 @@ inline void complete_config(fss_config &c, int64_t bs, int64_t seq, int64_t d, i
   c.vec = pick.vec;
   c.steps = pick.steps;
   c.waves = pick.waves;
-  // Two column tiles per workgroup (rows of 512 contiguous bytes, chunks half as long) are never
-  // the library's own choice: measured in the forward with 4 bytes per lane, 32 steps and 16 waves
-  // they are 4-13 % faster where a launch has at most two tiles per CU and nothing is found in a
-  // cache (bs 8 seq 4096 d 1024: 42.9 -> 41.2 us over tensor sets in rotation), 5-7 % slower when
-  // the tensors are found in the memory-side cache again (30.8 -> 32.4 us), and slower throughout
-  // in the backward, whose chunks would shrink to 128 steps.  The library cannot know which of
-  // the two it is in, and a different tiling rounds the carries differently, so it stays an
-  // explicit configuration.
-  if (!c.cols) c.cols = 1;
+  if (!c.cols) c.cols = choose_cols(c, bs, seq, d, dtype, dir, gated);
 }
 
 struct Plan {

@@ -586,11 +586,19 @@ int launch_one(const ScanArgs &args, const StateArgs<true> &state, const Plan &p
 }
 
 // Two column tiles per workgroup exist for the plain scan's 4-byte-per-lane kernels (the ones
-// large shapes run); config_supported_cols says the same to the planner.
-template <typename E, bool BWD>
+// large shapes run), with 16 steps per lane in both directions and with 32 in the forward; the
+// forward also with states (the library takes two columns by itself there, and the scan with
+// states must cut the sequence where the plain scan does).
+template <typename E, bool BWD, bool STATE>
 int launch_two_columns(const ScanArgs &args, const StateArgs<true> &state, const Plan &pl, hipStream_t stream) {
   constexpr int V = E::kBytes == 2 ? 2 : 1;
   if (pl.cfg.vec != V) return FSS_ERR_BAD_CONFIG;
+  if constexpr (STATE) {
+    if constexpr (!BWD) {
+      if (pl.cfg.steps == 32) return launch_one<E, V, 32, BWD, true, false, false, 2>(args, state, pl, stream);
+    }
+    return FSS_ERR_BAD_CONFIG;
+  } else {
   switch (pl.cfg.steps) {
 #define FSS_CASE2(S)                                                                                   \
   case S:                                                                                              \
@@ -609,15 +617,13 @@ int launch_two_columns(const ScanArgs &args, const StateArgs<true> &state, const
   }
 #undef FSS_CASE2
   return FSS_ERR_BAD_CONFIG;
+  }
 }
 
 template <typename E, bool BWD, bool STATE>
 int launch_typed(const ScanArgs &args, const StateArgs<true> &state, const Plan &pl, hipStream_t stream) {
   constexpr bool is_16bit = E::kBytes == 2;
-  if (pl.cfg.cols == 2) {
-    if constexpr (STATE) return FSS_ERR_BAD_CONFIG;
-    else return launch_two_columns<E, BWD>(args, state, pl, stream);
-  }
+  if (pl.cfg.cols == 2) return launch_two_columns<E, BWD, STATE>(args, state, pl, stream);
   const int key = pl.cfg.vec * 100 + pl.cfg.steps;
   switch (key) {
 #define FSS_CASE(V, S)                                                                            \

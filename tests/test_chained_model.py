@@ -88,9 +88,14 @@ def test_fold_covers_every_chunk_between_once_nearest_first(period, look, span):
 
 def test_chain_plan_of_the_measured_workloads():
     # (shape, dtype, dir) -> chunk length and period: the planned grid holds 256 workgroups of 16 waves
+    # (the forward at this shape is a two-round launch: two column tiles per workgroup, so 8 of its
+    # 16 waves lie along time and a chunk is 256 steps)
     p = chain_plan(8, 4096, 1024, _native.FSS_BF16, _native.FSS_FWD)
+    assert (p["steps"], p["waves"], p["vec"], p["cols"]) == (32, 8, 2, 2)
+    assert p["n_chunks"] == 16 and p["period"] == 8 and p["span"] == 1
+    p = chain_plan(8, 8192, 1024, _native.FSS_BF16, _native.FSS_FWD)
     assert (p["steps"], p["waves"], p["vec"], p["cols"]) == (32, 16, 2, 1)
-    assert p["n_chunks"] == 8 and p["period"] == 4 and p["span"] == 1
+    assert p["n_chunks"] == 16 and p["period"] == 4 and p["span"] == 1
     p = chain_plan(8, 4096, 1024, _native.FSS_BF16, _native.FSS_BWD)
     assert (p["steps"], p["waves"]) == (16, 16) and p["n_chunks"] == 16 and p["period"] == 4
     p = chain_plan(1, 65521, 256, _native.FSS_BF16, _native.FSS_FWD)

@@ -60,8 +60,12 @@ def test_state_scan_matches_extended_oracle(oracle, dtype, rtol, atol, shape, co
         _close(got, ref, rtol, atol, name)
 
 
-def test_without_state_equals_plain_scan():
-    alpha, beta, dout = make_inputs("hawk", 3, 900, 192, seed=93)
+@pytest.mark.parametrize("shape,recipe", [((3, 900, 192), "hawk"), ((8, 4096, 1024), "near_one")], ids=["small", "two_round_forward"])
+def test_without_state_equals_plain_scan(shape, recipe):
+    """Bit for bit: the scan with states cuts the sequence where the plain scan does - also where the
+    library gives the forward two column tiles per workgroup (the second shape; alphas near 1 there,
+    so that a different tiling would show)."""
+    alpha, beta, dout = make_inputs(recipe, *shape, seed=93)
     a, b, do = alpha.to(DEV), beta.to(DEV), dout.to(DEV)
     h, h_last = ext.scan_forward_state(a, b, None)
     h_plain = ext.scan_forward_half(a, b)
