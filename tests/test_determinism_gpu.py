@@ -223,3 +223,73 @@ def test_infinite_alpha_poisons_exactly_what_it_poisons_sequentially(oracle, dty
     assert finite[1].all() and finite[0, :, 2:64].all() and finite[0, :, 66:].all()
     tol = 1e-2 if dtype == torch.bfloat16 else 1e-4
     assert np.allclose(got[finite], want[finite], rtol=tol, atol=tol)
+
+
+def _random_tilings(n, seed):
+    """(dtype, shape, forward configuration, backward configuration) drawn at random from what the
+    row-major kernels are compiled for, with short chunks so that sequences chain many of them."""
+    rng = np.random.default_rng(seed)
+    out = []
+    while len(out) < n:
+        dtype = torch.bfloat16 if rng.random() < 0.6 else torch.float32
+        vec = int(rng.choice([1, 2, 4, 8] if dtype == torch.bfloat16 else [1, 2, 4]))
+        steps = int(rng.choice([8, 16, 32]))
+        budget = 64 if dtype == torch.bfloat16 else 32
+        if vec * steps > budget:
+            continue
+        max_waves = 4 if vec >= 8 else 8 if vec >= 4 else 16
+        waves = int(rng.integers(1, max_waves + 1))
+        cols = 1
+        if vec * (2 if dtype == torch.bfloat16 else 4) == 4 and steps in (16, 32) and waves % 2 == 0 and rng.random() < 0.4:
+            cols = 2
+        bs = int(rng.integers(1, 4))
+        d = 64 * vec * cols * int(rng.integers(1, 4))
+        seq = int(rng.integers(steps * max(waves // cols, 1) + 1, 40 * steps * max(waves // cols, 1)))
+        seq = min(seq, 6000)
+        groups = int(rng.choice([0, 0, 1, 2, 5, 16]))
+        fwd = (vec, steps, waves, groups, cols)
+        # the backward has no 32-step kernels beyond 8 waves at two channels per lane, none with two
+        # column tiles at 32 steps, and holds three tensors: stay within what it is compiled for
+        b_steps = steps if vec * steps * 3 <= budget * 2 or vec < 2 else 16 if vec * 16 <= budget else 8
+        if dtype == torch.float32 and vec * b_steps > 32:
+            b_steps = 8
+        b_cols = cols if b_steps == 16 else 1
+        b_waves = waves if not (vec >= 2 and b_steps == 32 and waves > 8) else 8
+        if b_cols == 2 and b_waves % 2:
+            b_cols = 1
+        bwd = (vec, b_steps, b_waves, groups, b_cols)
+        out.append((dtype, (bs, seq, d), fwd, bwd))
+    return out
+
+
+TWO_COLUMN_TILINGS = [
+    (torch.bfloat16, (2, 3000, 512), (2, 32, 8, 0, 2), (2, 16, 8, 0, 2)),
+    (torch.bfloat16, (1, 5000, 256), (2, 16, 6, 3, 2), (2, 16, 6, 3, 2)),
+    (torch.bfloat16, (3, 2222, 1024), (2, 32, 16, 0, 2), (2, 16, 16, 7, 2)),
+    (torch.float32, (2, 2000, 256), (1, 32, 4, 0, 2), (1, 16, 4, 0, 2)),
+]
+
+
+@pytest.mark.parametrize("dtype,shape,fwd_cfg,bwd_cfg", _random_tilings(36, seed=20) + TWO_COLUMN_TILINGS,
+                         ids=lambda v: str(v).replace("torch.", "").replace(" ", ""))
+def test_random_tilings_return_the_models_bits(oracle, dtype, shape, fwd_cfg, bwd_cfg):
+    """Any tiling the kernels are compiled for, capped grids and two column tiles included: the device
+    returns the bits of the sequential model of that tiling (alphas near 1)."""
+    lib = _native.lib()
+    plan = (ctypes.c_int32 * 8)()
+    for direction, cfg in ((_native.FSS_FWD, fwd_cfg), (_native.FSS_BWD, bwd_cfg)):
+        if lib.fss_debug_chain_plan(*shape, CODE[dtype], direction, 16, _native.make_config(cfg), plan) != 0:
+            pytest.skip(f"configuration {cfg} is not one the library has a kernel for")
+    alpha, beta, dout = long_memory_inputs("near_one", shape, dtype, seed=sum(shape) + fwd_cfg[1])
+    a, b, do = alpha.to(DEV), beta.to(DEV), dout.to(DEV)
+    h = ext._forward(dtype, a, b, fwd_cfg)
+    ga, gb = ext._backward(dtype, a, h, do, bwd_cfg)
+    ext.workspace_status()
+    order = ("steps", "waves", "period", "look", "span")
+    fwd = chain_plan(shape, dtype, _native.FSS_FWD, fwd_cfg)
+    bwd = chain_plan(shape, dtype, _native.FSS_BWD, bwd_cfg)
+    a_m, b_m, do_m = as_model_array(alpha), as_model_array(beta), as_model_array(dout)
+    np.testing.assert_array_equal(as_model_array(h), oracle.chained_scan_fwd(a_m, b_m, *(fwd[k] for k in order)))
+    ga_model, gb_model = oracle.chained_scan_bwd(a_m, as_model_array(h), do_m, *(bwd[k] for k in order))
+    np.testing.assert_array_equal(as_model_array(gb), gb_model)
+    np.testing.assert_array_equal(as_model_array(ga), ga_model)
