@@ -293,3 +293,45 @@ def test_random_tilings_return_the_models_bits(oracle, dtype, shape, fwd_cfg, bw
     ga_model, gb_model = oracle.chained_scan_bwd(a_m, as_model_array(h), do_m, *(bwd[k] for k in order))
     np.testing.assert_array_equal(as_model_array(gb), gb_model)
     np.testing.assert_array_equal(as_model_array(ga), ga_model)
+
+
+def test_the_other_kernel_families_return_the_same_bits_from_run_to_run():
+    """The gated scan, the scans with states and the channel-major scan chain their chunks through the
+    same phase: eight launches of each, long-memory inputs, one set of bits (outputs finite)."""
+    shape = (4, 6000, 256)
+    alpha, beta, dout = make_inputs("near_one", *shape, seed=77)
+    g = torch.Generator().manual_seed(78)
+    gate = (torch.randn(shape, generator=g) + 6.0).to(torch.bfloat16).to(DEV)
+    h0 = torch.randn(shape[0], shape[2], generator=g).to(DEV)
+    g_last = torch.randn(shape[0], shape[2], generator=g).to(DEV)
+    a, b, do = alpha.to(DEV), beta.to(DEV), dout.to(DEV)
+    # channel-major: (bs, d, seq) with a sequence long enough to be chained through memory
+    a_cm, b_cm, do_cm = (t[:2, :, :64].transpose(1, 2).contiguous().repeat(1, 1, 3) for t in (a, b, do))
+
+    def gated():
+        h = ext.gated_scan_forward(gate, b)
+        return (h, *ext.gated_scan_backward(gate, b, h, do))
+
+    def with_states():
+        h, h_last = ext.scan_forward_state(a, b, h0)
+        return (h, h_last, *ext.scan_backward_state(a, h, do, h0, g_last))
+
+    def gated_with_states():
+        h, h_last = ext.gated_scan_forward_state(gate, b, h0)
+        return (h, h_last, *ext.gated_scan_backward_state(gate, b, h, do, h0, g_last))
+
+    def channel_major():
+        h = ext.scan_forward_cm(a_cm, b_cm)
+        return (h, *ext.scan_backward_cm(a_cm, h, do_cm))
+
+    assert a_cm.shape == (2, 64, 18000)
+    for run in (gated, with_states, gated_with_states, channel_major):
+        first = run()
+        torch.cuda.synchronize()
+        same = []
+        for _ in range(8):
+            same.append(torch.stack([(x == y).all() for x, y in zip(first, run())]))
+        assert bool(torch.stack(same).all()), run.__name__
+        for x in first:
+            assert bool(torch.isfinite(x.float()).all()), run.__name__
+    ext.workspace_status()
