@@ -112,7 +112,7 @@ def _declare(lib: ctypes.CDLL) -> None:
     lib.fss_debug_chain_plan.restype = _int
     lib.fss_debug_chain_plan.argtypes = [_i64, _i64, _i64, _int, _int, _sz, _cfgp, ctypes.POINTER(ctypes.c_int32)]
     lib.fss_debug_chain_anchor.restype = ctypes.c_int32
-    lib.fss_debug_chain_anchor.argtypes = [ctypes.c_int32, ctypes.c_int32]
+    lib.fss_debug_chain_anchor.argtypes = [ctypes.c_int32, ctypes.c_int32, ctypes.c_int32]
     lib.fss_scan_fwd_noalloc.restype = _int
     lib.fss_scan_fwd_noalloc.argtypes = [_int, _vp, _vp, _vp, _i64, _i64, _i64, _vp]
     lib.fss_choose_config.restype = _int

@@ -222,7 +222,6 @@ int run_scan(int dtype, int dir, const void *alpha, const void *in_b, const void
   args.wg_cols = pl.cfg.cols;
   args.look_waves = look_waves(pl.cfg.waves, pl.cfg.vec, pl.cfg.cols);
   args.period = chain_period(pl.n_groups, pl.cfg.waves);
-  args.span = look_span(args.n_chunks, args.period, args.look_waves);
   args.spin_limit = __atomic_load_n(&g_spin_limit, __ATOMIC_RELAXED);
   const int64_t tensor_bytes = bs * seq * d * static_cast<int64_t>(esize);
   if (streaming)
@@ -367,15 +366,15 @@ int fss_debug_chain_plan(int64_t bs, int64_t seq, int64_t d, int dtype, int dir,
   out[2] = pl.cfg.steps;
   out[3] = period;
   out[4] = look;
-  out[5] = fss::look_span(static_cast<int>(pl.n_chunks), period, look);
+  out[5] = fss::kMaxSpan;
   out[6] = pl.cfg.vec;
   out[7] = pl.cfg.cols;
   return FSS_OK;
 }
 
-int32_t fss_debug_chain_anchor(int32_t chunk, int32_t period) {
-  if (chunk < 0 || period < 1) return -1;
-  return fss::chain_anchor(chunk, period);
+int32_t fss_debug_chain_anchor(int32_t chunk, int32_t period, int32_t stride) {
+  if (chunk < 0 || period < 1 || stride < 1) return -1;
+  return fss::chain_anchor(chunk, period, stride);
 }
 
 uint32_t fss_debug_set_spin_limit(uint32_t polls) {

@@ -203,7 +203,6 @@ __global__ __launch_bounds__(1024) void cm_scan_kernel(const ScanArgs p) {
   c.wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   c.n_waves = blockDim.x >> 6;
   c.look = p.look_waves;
-  c.span = p.span;
   float2 *const lds_maps = reinterpret_cast<float2 *>(lds);  // laid out as in scan_kernel with one slot per lane
   c.lds_pred = lds_maps + 2 * c.n_waves * 64;
   c.seq = p.seq;
@@ -230,7 +229,8 @@ __global__ __launch_bounds__(1024) void cm_scan_kernel(const ScanArgs p) {
     c.chunk = static_cast<int>(chunk);
     c.ctile = static_cast<int>(ctile);
     c.last = c.chunk == p.n_chunks - 1;
-    c.anchor = __builtin_amdgcn_readfirstlane(chain_anchor(c.chunk, p.period));
+    c.anchor = __builtin_amdgcn_readfirstlane(chain_anchor(c.chunk, p.period, p.look_waves * kMaxSpan));
+    c.span = __builtin_amdgcn_readfirstlane(chunk_span(c.chunk - c.anchor, p.look_waves));
     cm_tile<E, VEC, ROWS, BWD>(p, c, static_cast<int64_t>(ctile) * ROWS, p.d);
   }
   count_out(p, c);
@@ -308,7 +308,6 @@ int run_cm_scan(int dtype, int dir, const void *alpha, const void *in_b, const v
   args.wg_cols = 1;
   args.look_waves = look_waves(pl.waves, 1);
   args.period = chain_period(pl.n_rowtiles, pl.waves);
-  args.span = look_span(args.n_chunks, args.period, args.look_waves);
   args.spin_limit = __atomic_load_n(&g_spin_limit, __ATOMIC_RELAXED);
   args.hdr = static_cast<uint32_t *>(workspace);
   args.words = workspace ? reinterpret_cast<uint64_t *>(static_cast<char *>(workspace) + kHeaderBytes) : nullptr;

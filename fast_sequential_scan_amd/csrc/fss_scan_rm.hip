@@ -473,7 +473,6 @@ __global__ __launch_bounds__(MAXW * 64) void scan_kernel(const ScanArgs p, const
   c.wcol = COLS > 1 ? (wave_in_group & 1) : 0;
   c.wave = COLS > 1 ? (wave_in_group >> 1) : wave_in_group;
   c.look = p.look_waves;
-  c.span = p.span;
   // LDS: two sets of per-wave maps (tiles alternate between them, so a wave that runs
   // ahead into the next tile cannot overwrite a map a slower wave still reads), then
   // the slots the look-back waves fill
@@ -523,7 +522,8 @@ __global__ __launch_bounds__(MAXW * 64) void scan_kernel(const ScanArgs p, const
     c.chunk = static_cast<int>(chunk);
     c.ctile = static_cast<int>(ctile);
     c.last = c.chunk == p.n_chunks - 1;
-    c.anchor = __builtin_amdgcn_readfirstlane(chain_anchor(c.chunk, p.period));
+    c.anchor = __builtin_amdgcn_readfirstlane(chain_anchor(c.chunk, p.period, p.look_waves * kMaxSpan));
+    c.span = __builtin_amdgcn_readfirstlane(chunk_span(c.chunk - c.anchor, p.look_waves));
 
     const int64_t col0 = static_cast<int64_t>(coltile) * kLaneSlots;  // first channel of the tile
     c.col_ok = col0 + c.lane * VEC < p.d;

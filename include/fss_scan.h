@@ -186,18 +186,19 @@ int fss_debug_tile_groups(int32_t n_groups, int32_t grid, int32_t n_tiles, int32
 /*
  * Test hooks (host only, no device call): how a row-major scan of this shape chains its chunks.
  * The state entering chunk k of a sequence is composed from the maps of chunks k-1 .. a+1 and
- * the outgoing state of chunk a = fss_debug_chain_anchor(k, period), the chunks dealt out
- * nearest first to `look` waves, `span` consecutive chunks each (a longer chain repeats that);
- * each wave composes its chunks nearest first, then the waves' results are folded in wave
- * order.  None of this depends on timing, so a chained scan returns the same bits from run to
- * run.  out[0..7] = number of chunks, waves along time per chunk, timesteps per lane (a chunk
- * is their product), period, look, span, vec, cols.  The current cache policy counts (as in
- * fss_choose_config).  No counterpart in the reference, where one thread walks a channel in
- * order (csrc/include/sequential_scan_kernel_bf16.cuh:121-151).
+ * the outgoing state of chunk a = fss_debug_chain_anchor(k, period, look * max_span): the last
+ * chunk of the round of `period` chunks before k's, or the last multiple of look * max_span
+ * below k if that is nearer.  The k - a chunks are dealt out nearest first to `look` waves,
+ * ceil((k - a) / look) consecutive chunks each; each wave composes its chunks nearest first,
+ * then the waves' results are folded in wave order.  None of this depends on timing, so a
+ * chained scan returns the same bits from run to run.  out[0..7] = number of chunks, waves
+ * along time per chunk, timesteps per lane (a chunk is their product), period, look, max_span,
+ * vec, cols.  No counterpart in the reference, where one thread walks a channel in order
+ * (csrc/include/sequential_scan_kernel_bf16.cuh:121-151).
  */
 int fss_debug_chain_plan(int64_t bs, int64_t seq, int64_t d, int dtype, int dir, size_t align_bytes,
                          const fss_config *cfg, int32_t *out);
-int32_t fss_debug_chain_anchor(int32_t chunk, int32_t period);
+int32_t fss_debug_chain_anchor(int32_t chunk, int32_t period, int32_t stride);
 
 /* The configuration the library would choose for this shape (for reporting). */
 int fss_choose_config(int64_t bs, int64_t seq, int64_t d, int dtype, int dir,

@@ -16,10 +16,11 @@
  *           order, B = fma0(A_w, B, B_w), A = A*A_w, which also yields what the slices before
  *           slice w do to the chunk's incoming state (its prefix);
  *   chain   the state entering chunk k > 0 is composed from the maps of chunks k-1 .. a+1 and
- *           the outgoing state of chunk a = anchor(k): the chunks are dealt out nearest first
- *           to `look` waves, `span` consecutive chunks each (a longer chain repeats that);
- *           each wave composes its chunks nearest first, then the waves' results are folded in
- *           wave order;
+ *           the outgoing state of chunk a = anchor(k) (the last chunk of the round of `period`
+ *           chunks before, or the last multiple of look*span below k if nearer): the chunks are
+ *           dealt out nearest first to `look` waves, ceil((k-a)/look) <= `span` consecutive
+ *           chunks each; each wave composes its chunks nearest first, then the waves' results
+ *           are folded in wave order;
  *   steps   every slice finally re-runs the recurrence from its true incoming state,
  *           state = fmaf(a, state, b), and the outputs are the states rounded to storage.
  *
@@ -57,9 +58,12 @@ typedef struct {
   int steps, waves, period, look, span;
 } chain_cfg;
 
-static int chain_anchor(int chunk, int period) {
+/* the last chunk of the round before, or the last multiple of `stride` below the chunk if nearer */
+static int chain_anchor(int chunk, int period, int stride) {
   const int round_first = chunk - chunk % period;
-  return round_first > 0 ? round_first - 1 : 0;
+  const int by_round = round_first > 0 ? round_first - 1 : 0;
+  const int by_stride = (chunk - 1) / stride * stride;
+  return by_round > by_stride ? by_round : by_stride;
 }
 
 /* One channel.  a[r], b[r] for r = 0..n-1 in scan order (a[0] is ignored: no predecessor);
@@ -105,15 +109,18 @@ static void chained_channel(const float *a, const float *b, float *out, int64_t 
       if (k == 0) {
         chunk_out[0] = B; /* the sequence starts from 0 */
       } else {
-        const int anchor = chain_anchor((int)k, cfg->period);
-        const int reach = cfg->look * cfg->span;
+        const int anchor = chain_anchor((int)k, cfg->period, cfg->look * cfg->span);
+        /* chunks per look-back wave: as few as the waves allow (cfg->span is the most) */
+        int span = ((int)k - anchor + cfg->look - 1) / cfg->look;
+        span = span < 1 ? 1 : (span > cfg->span ? cfg->span : span);
+        const int reach = cfg->look * span;
         float accA = 1.0f, accB = 0.0f;
         for (int nearest = (int)k - 1; nearest >= anchor; nearest -= reach) {
-          for (int w = 0; w < cfg->look && nearest - w * cfg->span >= anchor; ++w) {
-            const int j = nearest - w * cfg->span;
+          for (int w = 0; w < cfg->look && nearest - w * span >= anchor; ++w) {
+            const int j = nearest - w * span;
             float qA = j == anchor ? 0.0f : chunk_A[j];
             float qB = j == anchor ? chunk_out[j] : chunk_B[j];
-            for (int kk = 1; kk < cfg->span && j - kk >= anchor; ++kk) {
+            for (int kk = 1; kk < span && j - kk >= anchor; ++kk) {
               const int jj = j - kk;
               const float rA = jj == anchor ? 0.0f : chunk_A[jj];
               const float rB = jj == anchor ? chunk_out[jj] : chunk_B[jj];

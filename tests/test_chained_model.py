@@ -5,7 +5,7 @@ Two things are pinned here without a GPU:
 * the host side of the order (`fss_debug_chain_plan`, `fss_debug_chain_anchor`): which earlier
   chunk's state a chunk starts from and which maps it composes depends on the chunk's index and
   the plan alone, covers every chunk in between exactly once, and never asks for more than one
-  period of maps;
+  period of maps nor for more than one round of the look-back reaches;
 * `oracle/chained_model.c`, the sequential C restatement of the kernels' composition order that
   the GPU tests demand bit-for-bit agreement with: one slice equals the fused sequential oracle
   exactly, exact-arithmetic inputs equal it exactly under every tiling (which pins the model's
@@ -25,7 +25,7 @@ import oracle
 from fast_sequential_scan_amd import _native
 
 TILINGS = [
-    # steps, waves, period, look, span
+    # steps, waves, period, look, most chunks per look-back wave
     (8, 1, 1, 1, 1),
     (8, 2, 1, 2, 1),
     (8, 2, 3, 2, 1),
@@ -42,15 +42,17 @@ def chain_plan(bs, seq, d, dtype, direction, cfg=None, align=16):
     out = (ctypes.c_int32 * 8)()
     rc = _native.lib().fss_debug_chain_plan(bs, seq, d, dtype, direction, align, _native.make_config(cfg), out)
     assert rc == 0, rc
-    keys = ("n_chunks", "waves", "steps", "period", "look", "span", "vec", "cols")
+    keys = ("n_chunks", "waves", "steps", "period", "look", "max_span", "vec", "cols")
     return dict(zip(keys, list(out)))
 
 
-def fold_items(chunk, period, look, span):
+def fold_items(chunk, period, look, max_span):
     """The order in which the kernels fold earlier chunks into the state entering `chunk`:
-    a list of groups (one per look-back wave and round), each a list of chunk indices, nearest
-    first; the very last index is the anchor, whose outgoing state is taken."""
-    anchor = _native.lib().fss_debug_chain_anchor(chunk, period)
+    a list of groups (one per look-back wave), each a list of chunk indices, nearest first; the
+    very last index is the anchor, whose outgoing state is taken."""
+    anchor = _native.lib().fss_debug_chain_anchor(chunk, period, look * max_span)
+    items = chunk - anchor
+    span = min(max_span, max(1, -(-items // look)))
     groups = []
     nearest = chunk - 1
     while nearest >= anchor:
@@ -63,27 +65,39 @@ def fold_items(chunk, period, look, span):
     return anchor, groups
 
 
-def test_anchor_is_a_function_of_chunk_and_period_only():
+def test_anchor_is_a_function_of_chunk_and_plan_only():
     lib = _native.lib()
     for period in (1, 2, 3, 4, 7, 64, 128, 1000):
-        for chunk in range(1, 600):
-            a = lib.fss_debug_chain_anchor(chunk, period)
-            assert 0 <= a < chunk
-            # the last chunk of the round before, or chunk 0 within the first round
-            first = chunk - chunk % period
-            assert a == (first - 1 if first > 0 else 0)
-            assert chunk - a <= period  # never more than one period of chunks to fold
-    assert lib.fss_debug_chain_anchor(-1, 4) == -1
-    assert lib.fss_debug_chain_anchor(3, 0) == -1
+        for stride in (1, 4, 8, 64, 52, 1 << 20):
+            for chunk in range(1, 600):
+                a = lib.fss_debug_chain_anchor(chunk, period, stride)
+                assert 0 <= a < chunk
+                # the last chunk of the round before (chunk 0 within the first round), or the last
+                # multiple of the stride below the chunk if that is nearer
+                first = chunk - chunk % period
+                by_round = first - 1 if first > 0 else 0
+                by_stride = (chunk - 1) // stride * stride
+                assert a == max(by_round, by_stride)
+                assert chunk - a <= min(period, stride)  # never more than that many chunks to fold
+                # an anchor's own chain ends at chunk 0 after finitely many hops
+                hops, k = 0, a
+                while k > 0:
+                    k = lib.fss_debug_chain_anchor(k, period, stride)
+                    hops += 1
+                assert hops <= chunk
+    assert lib.fss_debug_chain_anchor(-1, 4, 64) == -1
+    assert lib.fss_debug_chain_anchor(3, 0, 64) == -1
+    assert lib.fss_debug_chain_anchor(3, 4, 0) == -1
 
 
-@pytest.mark.parametrize("period,look,span", [(1, 1, 1), (4, 16, 1), (4, 2, 1), (128, 16, 4), (7, 2, 3), (300, 16, 4)])
-def test_fold_covers_every_chunk_between_once_nearest_first(period, look, span):
+@pytest.mark.parametrize("period,look,max_span", [(1, 1, 1), (4, 16, 4), (4, 2, 1), (128, 16, 4), (7, 2, 3), (300, 16, 4), (300, 5, 4)])
+def test_fold_covers_every_chunk_between_once_nearest_first(period, look, max_span):
     for chunk in range(1, 700):
-        anchor, groups = fold_items(chunk, period, look, span)
+        anchor, groups = fold_items(chunk, period, look, max_span)
         flat = [j for g in groups for j in g]
         assert flat == list(range(chunk - 1, anchor - 1, -1))
-        assert all(1 <= len(g) <= span for g in groups)
+        assert all(1 <= len(g) <= max_span for g in groups)
+        assert len(groups) <= look  # one round of the look-back always reaches the anchor
 
 
 def test_chain_plan_of_the_measured_workloads():
@@ -92,15 +106,17 @@ def test_chain_plan_of_the_measured_workloads():
     # 16 waves lie along time and a chunk is 256 steps)
     p = chain_plan(8, 4096, 1024, _native.FSS_BF16, _native.FSS_FWD)
     assert (p["steps"], p["waves"], p["vec"], p["cols"]) == (32, 8, 2, 2)
-    assert p["n_chunks"] == 16 and p["period"] == 8 and p["span"] == 1
+    assert p["n_chunks"] == 16 and p["period"] == 8 and p["max_span"] == 4
     p = chain_plan(8, 8192, 1024, _native.FSS_BF16, _native.FSS_FWD)
     assert (p["steps"], p["waves"], p["vec"], p["cols"]) == (32, 16, 2, 1)
-    assert p["n_chunks"] == 16 and p["period"] == 4 and p["span"] == 1
+    assert p["n_chunks"] == 16 and p["period"] == 4 and p["look"] == 16
     p = chain_plan(8, 4096, 1024, _native.FSS_BF16, _native.FSS_BWD)
     assert (p["steps"], p["waves"]) == (16, 16) and p["n_chunks"] == 16 and p["period"] == 4
     p = chain_plan(1, 65521, 256, _native.FSS_BF16, _native.FSS_FWD)
     # two column tiles of 128 channels, 128 chunks of 512 steps: every chunk is in flight at once
-    assert (p["n_chunks"], p["steps"] * p["waves"], p["period"], p["look"], p["span"]) == (128, 512, 128, 16, 4)
+    # (so every 64th chunk is an anchor as well: 16 look-back waves x 4 chunks)
+    assert (p["n_chunks"], p["steps"] * p["waves"], p["period"], p["look"], p["max_span"]) == (128, 512, 128, 16, 4)
+    assert _native.lib().fss_debug_chain_anchor(127, 128, 64) == 64 and _native.lib().fss_debug_chain_anchor(64, 128, 64) == 0
     # an explicit configuration and a grid cap: the cap does not enter the plan
     a = chain_plan(2, 4099, 256, _native.FSS_BF16, _native.FSS_FWD, cfg=(1, 8, 2))
     b = chain_plan(2, 4099, 256, _native.FSS_BF16, _native.FSS_FWD, cfg=(1, 8, 2, 3))

@@ -37,8 +37,8 @@ def chain_plan(shape, dtype, direction, cfg=None):
     out = (ctypes.c_int32 * 8)()
     rc = _native.lib().fss_debug_chain_plan(*shape, CODE[dtype], direction, 16, _native.make_config(cfg), out)
     assert rc == 0, rc
-    n_chunks, waves, steps, period, look, span, _vec, _cols = list(out)
-    return dict(n_chunks=n_chunks, steps=steps, waves=waves, period=period, look=look, span=span)
+    n_chunks, waves, steps, period, look, max_span, _vec, _cols = list(out)
+    return dict(n_chunks=n_chunks, steps=steps, waves=waves, period=period, look=look, span=max_span)
 
 
 def long_memory_inputs(recipe, shape, dtype, seed):
