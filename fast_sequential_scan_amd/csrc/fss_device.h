@@ -622,9 +622,8 @@ __device__ __forceinline__ void fold_arriving_maps(float2 *lds_map, const uint32
 // After the one barrier of the phase every wave folds what the look-back waves left in LDS into
 // the chunk's incoming state itself (a few multiply-adds: cheaper than another barrier and a
 // broadcast), wave 0 also publishes the chunk's outgoing state, and every wave applies the
-// composition of the waves before it (one LDS read).  A chain of more than look*span chunks
-// repeats the look-back.  Who looks at which chunk, and the order of every composition, depend
-// on the chunk's index and the plan alone.
+// composition of the waves before it (one LDS read).  Who looks at which chunk, and the order of
+// every composition, depend on the chunk's index and the plan alone.
 //
 // `mid` (only with HAS_MID) is called once by every wave, by the look-back waves right after their
 // first fetch has been issued: loads it issues travel while the chain is resolved and
@@ -694,7 +693,6 @@ __device__ __forceinline__ void chain_chunks(const ScanArgs &p, const TileCtx &c
     hin[v] = local_const(0.0f);
   }
   const int anchor = c.anchor;
-  const int reach = c.look * c.span;  // chunks one round of the look-back covers
   // Which wave asks which chunk: look index 0 asks the nearest chunk.  Where the waves issue loads
   // of their own inside this phase (`mid`), the look-back is the work of the LAST waves (look
   // index 0 = the last wave): wave 0 is busy composing and publishing the chunk's own map and
@@ -702,71 +700,60 @@ __device__ __forceinline__ void chain_chunks(const ScanArgs &p, const TileCtx &c
   // 54.0 us, 60.3 -> 58.4 us over tensor sets in rotation; the forward, which issues nothing
   // here, measured 0.3-0.6 us slower that way and keeps the first waves).
   const int li = HAS_MID ? c.n_waves - 1 - wave : wave;
-  int nearest = c.chunk - 1;          // nearest earlier chunk not folded yet (>= anchor)
-  // The first look goes out ahead of the loop, with `mid` in a straight line between the
-  // issue of its loads and their use: only so does the compiler wait for exactly those
-  // loads and not for the ones `mid` has issued behind them.
+  // The chunks chunk-1 .. anchor, `span` consecutive ones per look-back wave: one round always
+  // reaches the anchor (chain_anchor keeps it within look * kMaxSpan chunks, chunk_span deals
+  // them out).  This wave's are j, j-1, ..., down to the anchor at most.
+  const int j = c.chunk - 1 - li * c.span;
+  const bool looks = li < c.look && j >= anchor;
+  // The first look goes out with `mid` in a straight line between the issue of its loads and
+  // their use: only so does the compiler wait for exactly those loads and not for the ones
+  // `mid` has issued behind them.
   bool have0 = false;
-  float q0A[VEC], q0B[VEC];
+  float qA[VEC], qB[VEC];
 #pragma unroll
-  for (int v = 0; v < VEC; ++v) q0A[v] = q0B[v] = local_const(0.0f);
+  for (int v = 0; v < VEC; ++v) qA[v] = qB[v] = local_const(0.0f);
   // The look-back starts once every wave of the column tile has its rows (the chunks it asks run
   // in step with this one: asking earlier only polls for longer).  Waves with loads of their own
   // to issue here wait for that moment too (issued while the other waves' rows are still on
   // their way, those loads only delay them: bs 8 seq 4096 d 1024 backward 53.5 -> 56.4 us); the
   // rest go straight on to the barrier.
-  const bool looks = li < c.look && nearest - li * c.span >= anchor;
   if (looks || (HAS_MID && wave != 0)) await_all_maps(c.s_ready, lane, c.n_waves, c.tile_no);
   if constexpr (HAS_MID) {
-    const int j0 = nearest - li * c.span;
     if (looks && p.spin_limit != 0) {
       ChunkWords<VEC> w;
-      poll_issue<VEC>(p, c, j0, j0 == anchor, w);
+      poll_issue<VEC>(p, c, j, j == anchor, w);
       mid();
-      have0 = poll_eval<VEC>(c, j0 == anchor, w, q0A, q0B);
+      have0 = poll_eval<VEC>(c, j == anchor, w, qA, qB);
     } else {
       mid();
     }
   }
-  for (;;) {
-    const int j = nearest - li * c.span;
-    if (li < c.look && j >= anchor) {
-      float qA[VEC], qB[VEC];
+  if (looks) {
+    if (!have0) await_chunk<VEC>(p, c, j, j == anchor, qA, qB);
+    // long chains: the wave also takes the chunks before that one (by now they have nearly
+    // always published), so that the look-back reaches `span` times as far
+    for (int k = 1; k < c.span && j - k >= anchor; ++k) {
+      float rA[VEC], rB[VEC];
+      await_chunk<VEC>(p, c, j - k, j - k == anchor, rA, rB);
 #pragma unroll
       for (int v = 0; v < VEC; ++v) {
-        qA[v] = q0A[v];
-        qB[v] = q0B[v];
-      }
-      if (!have0) await_chunk<VEC>(p, c, j, j == anchor, qA, qB);
-      have0 = false;
-      // long chains: the wave also takes the chunks before that one (by now they have nearly
-      // always published), so that one round of the look-back reaches `span` times as far
-      for (int k = 1; k < c.span && j - k >= anchor; ++k) {
-        float rA[VEC], rB[VEC];
-        await_chunk<VEC>(p, c, j - k, j - k == anchor, rA, rB);
-#pragma unroll
-        for (int v = 0; v < VEC; ++v) {
-          qB[v] = fma0(qA[v], rB[v], qB[v]);
-          qA[v] *= rA[v];
-        }
-      }
-#pragma unroll
-      for (int v = 0; v < VEC; ++v) c.lds_pred[(li * VEC + v) * 64 + lane] = make_float2(qA[v], qB[v]);
-    }
-    __syncthreads();
-    // every wave folds what the look-back waves found (the same few LDS reads in each wave
-    // cost less than a second barrier and a broadcast by wave 0)
-    for (int w = 0; w < c.look && nearest - w * c.span >= anchor; ++w) {
-#pragma unroll
-      for (int v = 0; v < VEC; ++v) {
-        const float2 m = c.lds_pred[(w * VEC + v) * 64 + lane];
-        accB[v] = fma0(accA[v], m.y, accB[v]);
-        accA[v] *= m.x;
+        qB[v] = fma0(qA[v], rB[v], qB[v]);
+        qA[v] *= rA[v];
       }
     }
-    nearest -= reach;
-    if (nearest < anchor) break;
-    __syncthreads();  // the slots are about to be overwritten: wait until every wave has read them
+#pragma unroll
+    for (int v = 0; v < VEC; ++v) c.lds_pred[(li * VEC + v) * 64 + lane] = make_float2(qA[v], qB[v]);
+  }
+  __syncthreads();
+  // every wave folds what the look-back waves found (the same few LDS reads in each wave
+  // cost less than a second barrier and a broadcast by wave 0)
+  for (int w = 0; w < c.look && c.chunk - 1 - w * c.span >= anchor; ++w) {
+#pragma unroll
+    for (int v = 0; v < VEC; ++v) {
+      const float2 m = c.lds_pred[(w * VEC + v) * 64 + lane];
+      accB[v] = fma0(accA[v], m.y, accB[v]);
+      accA[v] *= m.x;
+    }
   }
   // (the last group folded ended with the anchor's state, the map x -> 0*x + s: accB is the state)
 #pragma unroll

@@ -23,20 +23,23 @@
 //     1. every lane issues all its loads at once (STEPS rows x 2 or 3 tensors:
 //        the memory-level parallelism that fills HBM), then folds its slice into
 //        the affine map x -> A*x + B it applies to the incoming state;
-//     2. wave 0 composes the waves' maps through LDS and publishes the chunk's map;
-//        at the same time up to 16 waves each fetch what one earlier chunk of the
-//        same channels offers (its outgoing state if it has one, else its map),
-//        so the look-back over the nearest chunks costs one memory round trip, not
-//        one per chunk (decoupled look-back over (A,B) pairs in global memory).
-//        Every wave folds what they found into the chunk's incoming state and
-//        applies the maps of the waves before it; wave 0 publishes the outgoing
-//        state.  The backward issues the loads of its third tensor, which only
-//        phase 3 needs, inside this phase, behind the look-back's fetch;
+//     2. wave 0 composes the waves' maps through LDS as they arrive and publishes the chunk's
+//        map; at the same time up to 16 waves fetch the maps of the earlier chunks the chunk is
+//        to compose and the outgoing state of the one it starts from (its "anchor"), up to four
+//        chunks per wave, so the look-back over the nearest chunks costs a few memory round
+//        trips, not one per chunk (a look-back over (A,B) pairs in global memory whose order of
+//        composition is fixed by the chunk's index: see chain_anchor in fss_device.h).
+//        Every wave folds what they found into the chunk's incoming state and applies the maps
+//        of the waves before it; wave 0 publishes the outgoing state.  The backward issues the
+//        loads of its third tensor, which only phase 3 needs, inside this phase;
 //     3. every lane re-runs the recurrence over its register-resident slice from
 //        its true incoming state, in sequential order, and stores the results.
 //   Because phase 3 restarts from the incoming state, only that state is
 //   computed by re-associated arithmetic; within a slice the operation order is
-//   exactly the sequential one.
+//   exactly the sequential one.  And because which chunks are composed, and in which
+//   grouping, depends on the chunk's index and the plan alone - never on which
+//   earlier chunk happens to have finished - the result is a function of the inputs
+//   and the launch configuration: the same bits on every run.
 //
 // Chaining across workgroups
 //   The grid is persistent: it holds no more workgroups than the device keeps
