@@ -152,7 +152,7 @@ def _declare(lib: ctypes.CDLL) -> None:
     lib.fss_scan_bwd_cm.argtypes = [_int, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _vp, _sz, _vp, _cfgp]
     lib.fss_copy_bytes.argtypes = [_vp, _vp, _sz, _vp]
     lib.fss_stream_mix.restype = _int
-    lib.fss_stream_mix.argtypes = [ctypes.POINTER(_vp), _int, ctypes.POINTER(_vp), _int, _sz, _int, _vp]
+    lib.fss_stream_mix.argtypes = [ctypes.POINTER(_vp), _int, ctypes.POINTER(_vp), _int, _sz, _int, ctypes.POINTER(_int), _vp]
 
 
 def lib() -> ctypes.CDLL:
@@ -185,12 +185,15 @@ def check(status: int) -> None:
         raise FssError(status, msg)
 
 
-def stream_mix(reads, writes, nbytes: int, nontemporal_writes: bool, stream_handle: int, sink: int = 0) -> None:
-    """fss_stream_mix over lists of device addresses; `sink`: 16 writable bytes for a read-only run."""
+def stream_mix(reads, writes, nbytes: int, nontemporal_writes: bool, stream_handle: int, sink: int = 0,
+               shape: Optional[Tuple[int, int, int, int]] = None) -> None:
+    """fss_stream_mix over lists of device addresses; `sink`: 16 writable bytes for a read-only run;
+    `shape`: (workgroups, threads, vectors per lane and iteration, non-temporal loads) or None."""
     rd = (_vp * len(reads))(*reads)
     wr_list = list(writes) if writes else [sink]
     wr = (_vp * len(wr_list))(*wr_list)
-    check(lib().fss_stream_mix(rd, len(reads), wr, len(writes), nbytes, int(nontemporal_writes), stream_handle))
+    sh = (_int * 4)(*shape) if shape is not None else None
+    check(lib().fss_stream_mix(rd, len(reads), wr, len(writes), nbytes, int(nontemporal_writes), sh, stream_handle))
 
 
 def make_config(cfg: Optional[Tuple[int, int, int]]):

@@ -38,34 +38,62 @@ struct StreamMixArgs {
   u32x4 *wr[2];
   size_t n_vec;
 };
-template <int R, int W, bool NT>
-__global__ __launch_bounds__(256) void stream_mix_kernel(const StreamMixArgs a) {
-  const size_t stride = static_cast<size_t>(gridDim.x) * blockDim.x;
-  for (size_t i = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x; i < a.n_vec; i += stride) {
-    u32x4 v = a.rd[0][i];
-    if (R > 1) v ^= a.rd[1][i];
-    if (R > 2) v ^= a.rd[2][i];
-    if (W > 0) {
-      if (NT) __builtin_nontemporal_store(v, a.wr[0] + i); else a.wr[0][i] = v;
-    }
-    if (W > 1) {
-      if (NT) __builtin_nontemporal_store(~v, a.wr[1] + i); else a.wr[1][i] = ~v;
-    }
-    if (W == 0) {
-      // read-only: the loads must not be optimised away; the store never happens in practice
-      // (the caller passes a 16-byte sink for the one value that would trigger it)
-      if (v.x == 0x9e3779b9u && v.y == 0x7f4a7c15u && v.z == 0xf39cc060u && v.w == 0x5cedc834u) a.wr[0][0] = v;
-    }
+template <bool NT>
+__device__ __forceinline__ u32x4 stream_load(const u32x4 *p) {
+  return NT ? __builtin_nontemporal_load(p) : *p;
+}
+template <int R, int W, bool NTW, bool NTR>
+__device__ __forceinline__ void stream_mix_finish(const StreamMixArgs &a, size_t i, u32x4 v) {
+  if (R > 1) v ^= stream_load<NTR>(a.rd[1] + i);
+  if (R > 2) v ^= stream_load<NTR>(a.rd[2] + i);
+  if (W > 0) {
+    if (NTW) __builtin_nontemporal_store(v, a.wr[0] + i); else a.wr[0][i] = v;
+  }
+  if (W > 1) {
+    if (NTW) __builtin_nontemporal_store(~v, a.wr[1] + i); else a.wr[1][i] = ~v;
+  }
+  if (W == 0) {
+    // read-only: the loads must not be optimised away; the store never happens in practice
+    // (the caller passes a 16-byte sink for the one value that would trigger it)
+    if (v.x == 0x9e3779b9u && v.y == 0x7f4a7c15u && v.z == 0xf39cc060u && v.w == 0x5cedc834u) a.wr[0][0] = v;
   }
 }
+// U vectors per lane and iteration, a grid stride apart: their first loads are issued together.
+template <int R, int W, bool NTW, bool NTR, int U>
+__global__ __launch_bounds__(1024) void stream_mix_kernel(const StreamMixArgs a) {
+  const size_t stride = static_cast<size_t>(gridDim.x) * blockDim.x;
+  size_t i = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+  for (; i + (U - 1) * stride < a.n_vec; i += U * stride) {
+    u32x4 v[U];
+#pragma unroll
+    for (int u = 0; u < U; ++u) v[u] = stream_load<NTR>(a.rd[0] + i + u * stride);
+#pragma unroll
+    for (int u = 0; u < U; ++u) stream_mix_finish<R, W, NTW, NTR>(a, i + u * stride, v[u]);
+  }
+  for (; i < a.n_vec; i += stride) stream_mix_finish<R, W, NTW, NTR>(a, i, stream_load<NTR>(a.rd[0] + i));
+}
 
-template <int R, int W>
-static void launch_stream_mix(const StreamMixArgs &a, bool nt, hipStream_t stream) {
-  const dim3 grid(2048), block(256);
-  if (nt)
-    hipLaunchKernelGGL((stream_mix_kernel<R, W, true>), grid, block, 0, stream, a);
+struct StreamMixShape {
+  int blocks, threads, per_lane;
+  bool nt_writes, nt_reads;
+};
+template <int R, int W, bool NTW, bool NTR>
+static void launch_stream_mix_u(const StreamMixArgs &a, const StreamMixShape &sh, hipStream_t stream) {
+  const dim3 grid(sh.blocks), block(sh.threads);
+  if (sh.per_lane == 2)
+    hipLaunchKernelGGL((stream_mix_kernel<R, W, NTW, NTR, 2>), grid, block, 0, stream, a);
   else
-    hipLaunchKernelGGL((stream_mix_kernel<R, W, false>), grid, block, 0, stream, a);
+    hipLaunchKernelGGL((stream_mix_kernel<R, W, NTW, NTR, 1>), grid, block, 0, stream, a);
+}
+template <int R, int W>
+static void launch_stream_mix(const StreamMixArgs &a, const StreamMixShape &sh, hipStream_t stream) {
+  if (sh.nt_writes) {
+    if (sh.nt_reads) launch_stream_mix_u<R, W, true, true>(a, sh, stream);
+    else launch_stream_mix_u<R, W, true, false>(a, sh, stream);
+  } else {
+    if (sh.nt_reads) launch_stream_mix_u<R, W, false, true>(a, sh, stream);
+    else launch_stream_mix_u<R, W, false, false>(a, sh, stream);
+  }
 }
 
 int g_cache_policy = FSS_CACHE_AUTO;  // fss_set_cache_policy
@@ -224,10 +252,14 @@ int run_scan(int dtype, int dir, const void *alpha, const void *in_b, const void
   args.period = chain_period(pl.n_groups, pl.cfg.waves);
   args.spin_limit = __atomic_load_n(&g_spin_limit, __ATOMIC_RELAXED);
   const int64_t tensor_bytes = bs * seq * d * static_cast<int64_t>(esize);
-  if (streaming)
-    pl.alt_policy = !gated && dir == FSS_BWD;
+  // (a forward kernel with fewer than 32 steps per lane has no variant 2 and runs as variant 0)
+  const bool large = streaming || tensor_bytes > kStreamDoutBytes;
+  if (gated)
+    pl.alt_policy = 0;
+  else if (dir == FSS_FWD)
+    pl.alt_policy = large ? 2 : (tensor_bytes <= kKeepOutBytes ? 1 : 0);
   else
-    pl.alt_policy = !gated && (dir == FSS_FWD ? tensor_bytes <= kKeepOutBytes : tensor_bytes > kStreamDoutBytes);
+    pl.alt_policy = large ? 1 : 0;
   const StateArgs<true> state = {state_in, state_out, h_before};
   args.hdr = static_cast<uint32_t *>(workspace);
   args.words = workspace ? reinterpret_cast<uint64_t *>(static_cast<char *>(workspace) + kHeaderBytes) : nullptr;
@@ -544,8 +576,18 @@ int fss_copy_bytes(const void *src, void *dst, size_t bytes, void *stream) {
 }
 
 int fss_stream_mix(const void *const *reads, int n_reads, void *const *writes, int n_writes, size_t bytes,
-                   int nontemporal_writes, void *stream) {
+                   int nontemporal_writes, const int *launch_shape, void *stream) {
   if (!reads || n_reads < 1 || n_reads > 3 || n_writes < 0 || n_writes > 2) return FSS_ERR_BAD_CONFIG;
+  fss::StreamMixShape sh = {2048, 256, 1, nontemporal_writes != 0, false};
+  if (launch_shape) {
+    sh.blocks = launch_shape[0];
+    sh.threads = launch_shape[1];
+    sh.per_lane = launch_shape[2];
+    sh.nt_reads = launch_shape[3] != 0;
+    if (sh.blocks < 1 || sh.blocks > (1 << 20) || sh.threads < 64 || sh.threads > 1024 || sh.threads % 64 != 0 ||
+        (sh.per_lane != 1 && sh.per_lane != 2) || (launch_shape[3] != 0 && launch_shape[3] != 1))
+      return FSS_ERR_BAD_CONFIG;
+  }
   if (!writes) return FSS_ERR_NULL_POINTER;  // (read-only runs still name one 16-byte sink)
   if (bytes % 16 != 0) return FSS_ERR_MISALIGNED;
   fss::StreamMixArgs a = {{nullptr, nullptr, nullptr}, {nullptr, nullptr}, bytes / 16};
@@ -561,17 +603,16 @@ int fss_stream_mix(const void *const *reads, int n_reads, void *const *writes, i
   }
   if (bytes == 0) return FSS_OK;
   hipStream_t s = static_cast<hipStream_t>(stream);
-  const bool nt = nontemporal_writes != 0;
   switch (n_reads * 10 + n_writes) {
-    case 10: fss::launch_stream_mix<1, 0>(a, nt, s); break;
-    case 11: fss::launch_stream_mix<1, 1>(a, nt, s); break;
-    case 12: fss::launch_stream_mix<1, 2>(a, nt, s); break;
-    case 20: fss::launch_stream_mix<2, 0>(a, nt, s); break;
-    case 21: fss::launch_stream_mix<2, 1>(a, nt, s); break;
-    case 22: fss::launch_stream_mix<2, 2>(a, nt, s); break;
-    case 30: fss::launch_stream_mix<3, 0>(a, nt, s); break;
-    case 31: fss::launch_stream_mix<3, 1>(a, nt, s); break;
-    default: fss::launch_stream_mix<3, 2>(a, nt, s); break;
+    case 10: fss::launch_stream_mix<1, 0>(a, sh, s); break;
+    case 11: fss::launch_stream_mix<1, 1>(a, sh, s); break;
+    case 12: fss::launch_stream_mix<1, 2>(a, sh, s); break;
+    case 20: fss::launch_stream_mix<2, 0>(a, sh, s); break;
+    case 21: fss::launch_stream_mix<2, 1>(a, sh, s); break;
+    case 22: fss::launch_stream_mix<2, 2>(a, sh, s); break;
+    case 30: fss::launch_stream_mix<3, 0>(a, sh, s); break;
+    case 31: fss::launch_stream_mix<3, 1>(a, sh, s); break;
+    default: fss::launch_stream_mix<3, 2>(a, sh, s); break;
   }
   const hipError_t e = hipGetLastError();
   if (e != hipSuccess) {

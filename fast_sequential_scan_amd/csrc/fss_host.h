@@ -229,7 +229,7 @@ inline void complete_config(fss_config &c, int64_t bs, int64_t seq, int64_t d, i
 
 struct Plan {
   fss_config cfg;
-  bool alt_policy = false;  // plain scan: the other cache policy (see kKeepOutBytes, kStreamDoutBytes)
+  int alt_policy = 0;  // plain scan: which cache hints the kernel carries (see kKeepOutBytes, kStreamDoutBytes)
   int64_t tiles_per_row, n_ctiles, n_chunks;
   int64_t n_groups;  // column groups per chunk: n_ctiles / cfg.cols
   int64_t n_tiles;   // what the workgroups walk: n_groups * n_chunks

@@ -84,7 +84,7 @@ namespace fss {
 // interior and every lane has channels, so nothing is predicated; otherwise every
 // access is guarded.  The two variants share no registers, so the guarded one
 // costs the fast one nothing.
-template <typename E, int VEC, int STEPS, bool BWD, bool STATE, bool FULL, bool ALT>
+template <typename E, int VEC, int STEPS, bool BWD, bool STATE, bool FULL, int ALT>
 __device__ __forceinline__ void scan_tile(const ScanArgs &p, const StateArgs<STATE> &st, const TileCtx &c) {
   using RowT = Row<E, VEC>;
   const int64_t seq = c.seq, row_bytes = c.row_bytes, r0 = c.r0;
@@ -117,7 +117,7 @@ __device__ __forceinline__ void scan_tile(const ScanArgs &p, const StateArgs<STA
       // of the sequence, so it loads the row before instead.
       const int row = (BWD && s == 0 && at_start) ? 1 : s;
       a[s].template load<(BWD ? kNtABwd : kNtAFwd)>(uniform_ptr(pa + row * step_bytes) + lane_off);
-      b[s].template load<(BWD ? (kNtBBwd || ALT) : kNtBFwd)>(uniform_ptr(pb + s * step_bytes) + lane_off);
+      b[s].template load<(BWD ? (kNtBBwd || ALT != 0) : (kNtBFwd || ALT == 2))>(uniform_ptr(pb + s * step_bytes) + lane_off);
     } else {
       // Outside the sequence the step is the identity map (a=1, b=0).  The first step
       // of the plain scan has no predecessor (a=0), whatever alpha holds there; with a
@@ -127,7 +127,7 @@ __device__ __forceinline__ void scan_tile(const ScanArgs &p, const StateArgs<STA
       if (c.col_ok && s < valid) {
         if (s >= 1 || !at_start || (STATE && !BWD && st.state_in))
           a[s].template load<(BWD ? kNtABwd : kNtAFwd)>(uniform_ptr(pa + s * step_bytes) + lane_off);
-        b[s].template load<(BWD ? (kNtBBwd || ALT) : kNtBFwd)>(uniform_ptr(pb + s * step_bytes) + lane_off);
+        b[s].template load<(BWD ? (kNtBBwd || ALT != 0) : (kNtBFwd || ALT == 2))>(uniform_ptr(pb + s * step_bytes) + lane_off);
       }
     }
   }
@@ -219,7 +219,7 @@ __device__ __forceinline__ void scan_tile(const ScanArgs &p, const StateArgs<STA
     if (FULL || (c.col_ok && s < valid)) {
       RowT o;
       o.pack(state);
-      o.template store<(BWD ? kNtOutBwd : (kNtOutFwd && !ALT))>(uniform_ptr(po0 + s * step_bytes) + lane_off);
+      o.template store<(BWD ? kNtOutBwd : (kNtOutFwd && ALT != 1))>(uniform_ptr(po0 + s * step_bytes) + lane_off);
       if (BWD) {
         if (!FULL && s + 1 == valid) {  // t = 0: grad_alpha[0] = g[0] * h[-1], 0 in the plain scan
 #pragma unroll
@@ -452,12 +452,14 @@ __device__ __forceinline__ void gated_tile(const ScanArgs &p, const StateArgs<ST
 
 // STATE: the variant that honours the optional incoming/outgoing state rows of ScanArgs;
 // the plain and the gated scan are compiled without them.  GATED: the gated scan.
-// ALT: the other cache policy of the plain scan - the forward for small outputs, which stores h
-// without the non-temporal hint; the backward for large tensors, which reads dout with it.
+// ALT: the cache policy of the plain scan (hints only, never the arithmetic).  Forward: 0 stores
+// h with the non-temporal hint, 1 without it (small outputs, left in the cache for their reader),
+// 2 = 0 and reads beta, which nothing reads again, with the hint (large tensors).  Backward:
+// 1 reads dout with the hint (large tensors).
 // COLS: column tiles a workgroup covers side by side (compile-time, so that the common
 // one-column kernels keep their compile-time LDS addresses and scalar register count).
 // MAXW: the most waves a workgroup may have (max_waves of the planner): what the registers are allotted for.
-template <typename E, int VEC, int STEPS, bool BWD, bool STATE, bool GATED, bool ALT, int COLS, int MAXW>
+template <typename E, int VEC, int STEPS, bool BWD, bool STATE, bool GATED, int ALT, int COLS, int MAXW>
 __global__ __launch_bounds__(MAXW * 64) void scan_kernel(const ScanArgs p, const StateArgs<STATE> st) {
   constexpr int kLaneSlots = 64 * VEC;  // channels per tile
 
@@ -562,7 +564,7 @@ __global__ __launch_bounds__(MAXW * 64) void scan_kernel(const ScanArgs p, const
 
 // ---- launching ---------------------------------------------------------------------
 
-template <typename E, int VEC, int STEPS, bool BWD, bool STATE, bool GATED = false, bool ALT = false, int COLS = 1>
+template <typename E, int VEC, int STEPS, bool BWD, bool STATE, bool GATED = false, int ALT = 0, int COLS = 1>
 int launch_one(const ScanArgs &args, const StateArgs<true> &state, const Plan &pl, hipStream_t stream) {
   // The kernel's waits are only safe if every workgroup of the grid is resident,
   // so the grid never exceeds what the device holds at once; workgroups loop.
@@ -605,8 +607,11 @@ int launch_two_columns(const ScanArgs &args, const StateArgs<true> &state, const
   switch (pl.cfg.steps) {
 #define FSS_CASE2(S)                                                                                   \
   case S:                                                                                              \
-    if (pl.alt_policy) return launch_one<E, V, S, BWD, false, false, true, 2>(args, state, pl, stream); \
-    return launch_one<E, V, S, BWD, false, false, false, 2>(args, state, pl, stream);
+    if constexpr (!BWD && S == 32) {                                                                   \
+      if (pl.alt_policy == 2) return launch_one<E, V, S, BWD, false, false, 2, 2>(args, state, pl, stream); \
+    }                                                                                                  \
+    if (pl.alt_policy == 1) return launch_one<E, V, S, BWD, false, false, 1, 2>(args, state, pl, stream); \
+    return launch_one<E, V, S, BWD, false, false, 0, 2>(args, state, pl, stream);
     FSS_CASE2(16)
     default:
       break;
@@ -632,7 +637,10 @@ int launch_typed(const ScanArgs &args, const StateArgs<true> &state, const Plan 
 #define FSS_CASE(V, S)                                                                            \
   case V * 100 + S:                                                                               \
     if constexpr (!STATE) {                                                                       \
-      if (pl.alt_policy) return launch_one<E, V, S, BWD, STATE, false, true>(args, state, pl, stream); \
+      if constexpr (!BWD && S == 32) {                                                            \
+        if (pl.alt_policy == 2) return launch_one<E, V, S, BWD, STATE, false, 2>(args, state, pl, stream); \
+      }                                                                                           \
+      if (pl.alt_policy == 1) return launch_one<E, V, S, BWD, STATE, false, 1>(args, state, pl, stream); \
     }                                                                                             \
     return launch_one<E, V, S, BWD, STATE>(args, state, pl, stream);
     FSS_CASE(1, 8)

@@ -250,12 +250,13 @@ int fss_scan_bwd_f32(const void *alpha, const void *h, const void *dout,
  * How the scans treat the memory-side cache (process-wide; no counterpart in the reference).
  *   FSS_CACHE_AUTO       (default) assumes that the tensors of a step are touched again soon,
  *                        as in a benchmark loop or a short pipeline: a small forward output is
- *                        left in the cache for its reader, and the backward reads dout with the
+ *                        left in the cache for its reader, and the tensors nothing reads again
+ *                        (beta in the forward, dout in the backward) are read with the
  *                        streaming hint only when the inputs of a step cannot fit the cache.
  *   FSS_CACHE_STREAMING  assumes that nothing is found in the cache again (a scan inside a
  *                        large model): the forward output always carries the streaming hint and
- *                        the backward always reads dout with it (measured 2-3 % faster then, 3 % slower in a loop
- *                        over one set of tensors).
+ *                        beta and dout are always read with it (measured 3-5 % faster then,
+ *                        3-5 % slower in a loop over one set of tensors).
  * The policy selects cache hints on loads and stores and nothing else - never the tiling - so
  * results are bit-identical under both.  Returns the previous policy, or -1 for an unknown one.
  */
@@ -401,17 +402,21 @@ int fss_copy_bytes(const void *src, void *dst, size_t bytes, void *stream);
 /*
  * Calibration kernel: the plainest kernel that moves a scan's mix of streams.  Reads `n_reads`
  * (1..3) buffers and writes `n_writes` (0..2) buffers of `bytes` bytes each (a multiple of 16;
- * all pointers 16-byte aligned), linearly, 16 bytes per lane, with no dependence between
- * elements; `nontemporal_writes` marks the stores as the scans mark theirs.  writes[0]
+ * all pointers 16-byte aligned), linearly, 16 bytes per lane and access, with no dependence
+ * between elements; `nontemporal_writes` marks the stores as the scans mark theirs.  writes[0]
  * receives the XOR of the reads, writes[1] its complement.  With n_writes = 0, writes[0] must
- * still name 16 writable bytes (a sink that is not written in practice).  The forward scan's
- * mix is 2 reads + 1 write, the backward's 3 reads + 2 writes: what this kernel reaches over
- * buffers that fit no cache is what the machine's memory system gives that mix, and
- * bench.py reports the scans against it next to the nominal 8 TB/s.  No counterpart in the
- * reference.
+ * still name 16 writable bytes (a sink that is not written in practice).  `launch_shape` is
+ * NULL (2048 workgroups of 256 threads, one vector per lane and iteration, ordinary loads) or
+ * names four ints: workgroups (1..2^20), threads per workgroup (a multiple of 64, at most
+ * 1024), vectors per lane and iteration (1 or 2, a grid stride apart, first loads issued
+ * together), non-temporal loads (0 or 1); which shape streams fastest depends on the mix, so a
+ * calibration tries a few and keeps the best.  The forward scan's mix is 2 reads + 1 write,
+ * the backward's 3 reads + 2 writes: what this kernel reaches over buffers that fit no cache is
+ * what the machine's memory system gives that mix, and bench.py reports the scans against it
+ * next to the nominal 8 TB/s.  No counterpart in the reference.
  */
 int fss_stream_mix(const void *const *reads, int n_reads, void *const *writes, int n_writes,
-                   size_t bytes, int nontemporal_writes, void *stream);
+                   size_t bytes, int nontemporal_writes, const int *launch_shape, void *stream);
 
 #ifdef __cplusplus
 }
