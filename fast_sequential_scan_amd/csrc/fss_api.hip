@@ -252,14 +252,15 @@ int run_scan(int dtype, int dir, const void *alpha, const void *in_b, const void
   args.period = chain_period(pl.n_groups, pl.cfg.waves);
   args.spin_limit = __atomic_load_n(&g_spin_limit, __ATOMIC_RELAXED);
   const int64_t tensor_bytes = bs * seq * d * static_cast<int64_t>(esize);
-  // (a forward kernel with fewer than 32 steps per lane has no variant 2 and runs as variant 0)
+  // (variant 2 exists for the kernels large shapes run - the forward with 32 steps per lane, the
+  // backward with 16 steps and 4 bytes per lane; elsewhere the forward runs as 0, the backward as 1)
   const bool large = streaming || tensor_bytes > kStreamDoutBytes;
   if (gated)
     pl.alt_policy = 0;
   else if (dir == FSS_FWD)
     pl.alt_policy = large ? 2 : (tensor_bytes <= kKeepOutBytes ? 1 : 0);
   else
-    pl.alt_policy = large ? 1 : 0;
+    pl.alt_policy = streaming ? 2 : (large ? 1 : 0);
   const StateArgs<true> state = {state_in, state_out, h_before};
   args.hdr = static_cast<uint32_t *>(workspace);
   args.words = workspace ? reinterpret_cast<uint64_t *>(static_cast<char *>(workspace) + kHeaderBytes) : nullptr;

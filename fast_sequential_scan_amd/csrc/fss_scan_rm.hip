@@ -116,7 +116,7 @@ __device__ __forceinline__ void scan_tile(const ScanArgs &p, const StateArgs<STA
       // below, whatever is loaded here.  The backward would find it one row past the end
       // of the sequence, so it loads the row before instead.
       const int row = (BWD && s == 0 && at_start) ? 1 : s;
-      a[s].template load<(BWD ? kNtABwd : kNtAFwd)>(uniform_ptr(pa + row * step_bytes) + lane_off);
+      a[s].template load<(BWD ? (kNtABwd || ALT == 2) : kNtAFwd)>(uniform_ptr(pa + row * step_bytes) + lane_off);
       b[s].template load<(BWD ? (kNtBBwd || ALT != 0) : (kNtBFwd || ALT == 2))>(uniform_ptr(pb + s * step_bytes) + lane_off);
     } else {
       // Outside the sequence the step is the identity map (a=1, b=0).  The first step
@@ -126,7 +126,7 @@ __device__ __forceinline__ void scan_tile(const ScanArgs &p, const StateArgs<STA
       b[s].fill(0.0f);
       if (c.col_ok && s < valid) {
         if (s >= 1 || !at_start || (STATE && !BWD && st.state_in))
-          a[s].template load<(BWD ? kNtABwd : kNtAFwd)>(uniform_ptr(pa + s * step_bytes) + lane_off);
+          a[s].template load<(BWD ? (kNtABwd || ALT == 2) : kNtAFwd)>(uniform_ptr(pa + s * step_bytes) + lane_off);
         b[s].template load<(BWD ? (kNtBBwd || ALT != 0) : (kNtBFwd || ALT == 2))>(uniform_ptr(pb + s * step_bytes) + lane_off);
       }
     }
@@ -455,7 +455,9 @@ __device__ __forceinline__ void gated_tile(const ScanArgs &p, const StateArgs<ST
 // ALT: the cache policy of the plain scan (hints only, never the arithmetic).  Forward: 0 stores
 // h with the non-temporal hint, 1 without it (small outputs, left in the cache for their reader),
 // 2 = 0 and reads beta, which nothing reads again, with the hint (large tensors).  Backward:
-// 1 reads dout with the hint (large tensors).
+// 1 reads dout with the hint (large tensors), 2 = 1 and reads alpha with it as well (its last
+// use in a step; only when the caller says that nothing is found in the cache again, because
+// the forward of a loop over one set of tensors does find it there).
 // COLS: column tiles a workgroup covers side by side (compile-time, so that the common
 // one-column kernels keep their compile-time LDS addresses and scalar register count).
 // MAXW: the most waves a workgroup may have (max_waves of the planner): what the registers are allotted for.
@@ -610,7 +612,8 @@ int launch_two_columns(const ScanArgs &args, const StateArgs<true> &state, const
     if constexpr (!BWD && S == 32) {                                                                   \
       if (pl.alt_policy == 2) return launch_one<E, V, S, BWD, false, false, 2, 2>(args, state, pl, stream); \
     }                                                                                                  \
-    if (pl.alt_policy == 1) return launch_one<E, V, S, BWD, false, false, 1, 2>(args, state, pl, stream); \
+    if (pl.alt_policy == 1 || (BWD && pl.alt_policy == 2))                                             \
+      return launch_one<E, V, S, BWD, false, false, 1, 2>(args, state, pl, stream);                    \
     return launch_one<E, V, S, BWD, false, false, 0, 2>(args, state, pl, stream);
     FSS_CASE2(16)
     default:
@@ -637,10 +640,11 @@ int launch_typed(const ScanArgs &args, const StateArgs<true> &state, const Plan 
 #define FSS_CASE(V, S)                                                                            \
   case V * 100 + S:                                                                               \
     if constexpr (!STATE) {                                                                       \
-      if constexpr (!BWD && S == 32) {                                                            \
+      if constexpr ((!BWD && S == 32) || (BWD && S == 16 && V * E::kBytes == 4)) {                \
         if (pl.alt_policy == 2) return launch_one<E, V, S, BWD, STATE, false, 2>(args, state, pl, stream); \
       }                                                                                           \
-      if (pl.alt_policy == 1) return launch_one<E, V, S, BWD, STATE, false, 1>(args, state, pl, stream); \
+      if (pl.alt_policy == 1 || (BWD && pl.alt_policy == 2))                                      \
+        return launch_one<E, V, S, BWD, STATE, false, 1>(args, state, pl, stream);                \
     }                                                                                             \
     return launch_one<E, V, S, BWD, STATE>(args, state, pl, stream);
     FSS_CASE(1, 8)

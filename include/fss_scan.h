@@ -254,9 +254,10 @@ int fss_scan_bwd_f32(const void *alpha, const void *h, const void *dout,
  *                        (beta in the forward, dout in the backward) are read with the
  *                        streaming hint only when the inputs of a step cannot fit the cache.
  *   FSS_CACHE_STREAMING  assumes that nothing is found in the cache again (a scan inside a
- *                        large model): the forward output always carries the streaming hint and
- *                        beta and dout are always read with it (measured 3-5 % faster then,
- *                        3-5 % slower in a loop over one set of tensors).
+ *                        large model): the forward output always carries the streaming hint,
+ *                        beta and dout are always read with it, and so is alpha at its last use,
+ *                        in the backward (measured 1-6 % faster then, 3-8 % slower in a loop
+ *                        over one set of tensors).
  * The policy selects cache hints on loads and stores and nothing else - never the tiling - so
  * results are bit-identical under both.  Returns the previous policy, or -1 for an unknown one.
  */
