@@ -99,6 +99,9 @@ def parse_args():
     ap.add_argument("--no-workloads", action="store_true",
                     help="skip the table of all ten workloads (profiler runs: its launches would be averaged "
                          "into the kernels' statistics)")
+    ap.add_argument("--stream-one-set", action="store_true",
+                    help="only the plain streaming kernel in the benchmark's protocol (one set of tensors of --case's "
+                         "size, forward's mix then backward's, --steps steps in each launch shape); for profiling")
     ap.add_argument("--copy-mb", type=int, default=0,
                     help="run only the library's plain copy kernel on this many MiB, --steps times "
                          "(hardware counters of the scan kernels are scaled by what they read for it)")
@@ -176,6 +179,27 @@ STREAM_SHAPES = ((2048, 256, 1, 0), (16384, 256, 1, 0), (1024, 1024, 1, 0), (819
                  (512, 256, 2, 1), (1024, 512, 2, 1), (512, 256, 1, 1), (2048, 256, 2, 0))
 
 
+def stream_one_set(_native, torch, p, tensor_bytes, sp, sink, warmup, steps):
+    """The benchmark's own protocol for the plain streaming kernel: the forward's mix and the
+    backward's alternating on ONE set of tensors (p: addresses of alpha, beta, dout, h, grad_alpha,
+    grad_beta), where the 256 MB memory-side cache returns part of every stream; both launches of
+    a step in the same launch shape.  Returns (best ms per step, its shape, ms per step by shape)."""
+    by_shape = {}
+    for shape in STREAM_SHAPES:
+        def run(n):
+            for _ in range(n):
+                _native.stream_mix([p[0], p[1]], [p[3]], tensor_bytes, True, sp, sink.data_ptr(), shape)
+                _native.stream_mix([p[0], p[3], p[2]], [p[4], p[5]], tensor_bytes, True, sp, sink.data_ptr(), shape)
+        run(warmup)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        run(steps)
+        torch.cuda.synchronize()
+        by_shape[shape] = (time.perf_counter() - t0) * 1e3 / steps
+    best = min(by_shape, key=by_shape.get)
+    return by_shape[best], best, by_shape
+
+
 def machine_stream_leg(lib, _native, torch, pointer_sets, tensor_bytes, sp):
     """What this machine streams: the library's plain streaming kernel (fss_stream_mix) over the
     tensor sets of the rotation - every launch meets buffers that were last touched seven launches
@@ -216,24 +240,7 @@ def machine_stream_leg(lib, _native, torch, pointer_sets, tensor_bytes, sp):
         out[name.replace("_GBps", "_ms_per_launch")] = round(best_ms, 5)
         out[name.replace("_GBps", "_shape")] = list(best_shape)
         out[name.replace("_GBps", "_first_shape_GBps")] = round(nbytes / (default_ms * 1e-3) / 1e9, 1)
-    # The benchmark's own protocol: the forward's mix and the backward's alternating on ONE set of
-    # tensors, where the 256 MB memory-side cache returns part of every stream (both launches of a
-    # step in the same shape; the best shape's step is the machine's for this protocol).
-    p = pointer_sets[0]
-    best_ms, best_shape = None, None
-    for shape in STREAM_SHAPES:
-        def steps(n):
-            for _ in range(n):
-                _native.stream_mix([p[0], p[1]], [p[3]], tensor_bytes, True, sp, sink.data_ptr(), shape)
-                _native.stream_mix([p[0], p[3], p[2]], [p[4], p[5]], tensor_bytes, True, sp, sink.data_ptr(), shape)
-        steps(10)
-        torch.cuda.synchronize()
-        t0 = time.perf_counter()
-        steps(50)
-        torch.cuda.synchronize()
-        ms = (time.perf_counter() - t0) * 1e3 / 50
-        if best_ms is None or ms < best_ms:
-            best_ms, best_shape = ms, shape
+    best_ms, best_shape, _ = stream_one_set(_native, torch, pointer_sets[0], tensor_bytes, sp, sink, 10, 50)
     out["one_set_step_ms"] = round(best_ms, 5)
     out["one_set_step_GBps"] = round(8 * tensor_bytes / (best_ms * 1e-3) / 1e9, 1)
     out["one_set_step_shape"] = list(best_shape)
@@ -378,6 +385,22 @@ def main() -> int:
         print(json.dumps({"metric": "plain copy kernel", "read_bytes": n, "written_bytes": n, "steps": args.steps,
                           "ms_per_launch": round(ms, 5), "value": round(2 * n / (ms * 1e-3) / 1e9, 1),
                           "unit": "GB/s (read+write)"}))
+        return 0
+
+    if args.stream_one_set:
+        _, bs, seq, d = BASELINE_CASES[args.case]
+        esize = 4 if args.dtype == "f32" else 2
+        nbytes = bs * seq * d * esize
+        tensors = [torch.full((nbytes,), i + 1, dtype=torch.uint8, device=dev) for i in range(6)]
+        sink = torch.zeros(16, dtype=torch.uint8, device=dev)
+        sp = torch.cuda.current_stream().cuda_stream
+        best_ms, best_shape, by_shape = stream_one_set(_native, torch, [t.data_ptr() for t in tensors], nbytes, sp, sink,
+                                                       args.warmup, args.steps)
+        print(json.dumps({"metric": "plain streaming kernel, forward's mix then backward's on one set of tensors",
+                          "case": args.case, "dtype": args.dtype, "bytes_per_stream": nbytes, "steps": args.steps,
+                          "ms_per_step": round(best_ms, 5), "launch_shape": list(best_shape),
+                          "value": round(8 * nbytes / (best_ms * 1e-3) / 1e9, 1), "unit": "GB/s",
+                          "ms_per_step_by_shape": {"x".join(map(str, k)): round(v, 5) for k, v in by_shape.items()}}))
         return 0
 
     ext.set_cache_policy(args.cache_policy)
