@@ -134,6 +134,31 @@ def test_entry_points_reject_bad_arguments_without_a_gpu():
     assert lib.fss_scan_fwd_ex(0, p, p, p, 1, 9, 8, None, 0, None, ctypes.byref(two_chunks)) == 4
 
 
+def test_calibration_kernel_checks_its_arguments_without_a_gpu():
+    """fss_stream_mix: stream counts, launch shape, pointers and sizes are checked before anything is
+    launched; zero bytes is a valid call that launches nothing."""
+    lib = _native.lib()
+    buf = (ctypes.c_char * 256)()
+    p = ctypes.addressof(buf)
+    p += (-p) % 16
+    vp = ctypes.c_void_p
+    reads, writes = (vp * 3)(p, p + 16, p + 32), (vp * 2)(p + 48, p + 64)
+    shape = lambda *v: (ctypes.c_int * 4)(*v)  # noqa: E731
+    assert lib.fss_stream_mix(reads, 3, writes, 2, 0, 1, None, None) == 0
+    assert lib.fss_stream_mix(reads, 3, writes, 2, 0, 1, shape(512, 256, 2, 1), None) == 0
+    assert lib.fss_stream_mix(reads, 0, writes, 1, 0, 1, None, None) == 5
+    assert lib.fss_stream_mix(reads, 4, writes, 1, 0, 1, None, None) == 5
+    assert lib.fss_stream_mix(reads, 1, writes, 3, 0, 1, None, None) == 5
+    for bad in ((0, 256, 1, 0), ((1 << 20) + 1, 256, 1, 0), (2048, 32, 1, 0), (2048, 100, 1, 0), (2048, 2048, 1, 0),
+                (2048, 256, 0, 0), (2048, 256, 3, 0), (2048, 256, 1, 2), (2048, 256, 1, -1)):
+        assert lib.fss_stream_mix(reads, 3, writes, 2, 0, 1, shape(*bad), None) == 5, bad
+    assert lib.fss_stream_mix(reads, 1, None, 0, 0, 1, None, None) == 1          # a read-only run still names a sink
+    assert lib.fss_stream_mix(reads, 3, writes, 2, 24, 1, None, None) == 3        # not a multiple of 16 bytes
+    assert lib.fss_stream_mix((vp * 3)(p, p + 8, p + 32), 3, writes, 2, 0, 1, None, None) == 3
+    assert lib.fss_stream_mix((vp * 3)(p, None, p + 32), 3, writes, 2, 0, 1, None, None) == 1
+    assert lib.fss_stream_mix(reads, 2, (vp * 2)(p + 48, None), 2, 0, 1, None, None) == 1
+
+
 def test_noalloc_entry_point_refuses_oversized_shapes_before_touching_a_device():
     lib = _native.lib()
     buf = (ctypes.c_char * 64)()
