@@ -602,7 +602,11 @@ int launch_two_columns(const ScanArgs &args, const StateArgs<true> &state, const
   if (pl.cfg.vec != V) return FSS_ERR_BAD_CONFIG;
   if constexpr (STATE) {
     if constexpr (!BWD) {
-      if (pl.cfg.steps == 32) return launch_one<E, V, 32, BWD, true, false, false, 2>(args, state, pl, stream);
+      if (pl.cfg.steps == 32) {
+        if (pl.alt_policy == 2) return launch_one<E, V, 32, BWD, true, false, 2, 2>(args, state, pl, stream);
+        if (pl.alt_policy == 1) return launch_one<E, V, 32, BWD, true, false, 1, 2>(args, state, pl, stream);
+        return launch_one<E, V, 32, BWD, true, false, 0, 2>(args, state, pl, stream);
+      }
     }
     return FSS_ERR_BAD_CONFIG;
   } else {
@@ -639,10 +643,11 @@ int launch_typed(const ScanArgs &args, const StateArgs<true> &state, const Plan 
   switch (key) {
 #define FSS_CASE(V, S)                                                                            \
   case V * 100 + S:                                                                               \
-    if constexpr (!STATE) {                                                                       \
-      if constexpr ((!BWD && S == 32) || (BWD && S == 16 && V * E::kBytes == 4)) {                \
-        if (pl.alt_policy == 2) return launch_one<E, V, S, BWD, STATE, false, 2>(args, state, pl, stream); \
-      }                                                                                           \
+    /* the scans with states carry the policy in the kernels large shapes run, the plain scan in all */ \
+    if constexpr ((!BWD && S == 32) || (BWD && S == 16 && V * E::kBytes == 4)) {                  \
+      if (pl.alt_policy == 2) return launch_one<E, V, S, BWD, STATE, false, 2>(args, state, pl, stream); \
+      if (pl.alt_policy == 1) return launch_one<E, V, S, BWD, STATE, false, 1>(args, state, pl, stream); \
+    } else if constexpr (!STATE) {                                                                \
       if (pl.alt_policy == 1 || (BWD && pl.alt_policy == 2))                                      \
         return launch_one<E, V, S, BWD, STATE, false, 1>(args, state, pl, stream);                \
     }                                                                                             \

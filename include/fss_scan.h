@@ -259,11 +259,11 @@ int fss_scan_bwd_f32(const void *alpha, const void *h, const void *dout,
  *                        in the backward (measured 1-6 % faster then, 3-8 % slower in a loop
  *                        over one set of tensors).
  * The policy selects cache hints on loads and stores and nothing else - never the tiling - so
- * results are bit-identical under both.  It acts on the plain scans over (bs, seq, d) tensors
- * (fss_scan_fwd_* / fss_scan_bwd_* by type, fss_scan_fwd_ex / fss_scan_bwd_ex,
- * fss_scan_fwd_noalloc); the scans with states, the gated and the channel-major scans carry the
- * same hints under both (outputs and the backward's reads of h streamed, everything else
- * cached).  Returns the previous policy, or -1 for an unknown one.
+ * results are bit-identical under both.  It acts on the plain scans over (bs, seq, d) tensors,
+ * with or without states (with states: in the kernels that large shapes run - 32 steps per lane
+ * in the forward, 16 steps and 4 bytes per lane in the backward); the gated and the channel-major
+ * scans carry the same hints under both (outputs and the backward's reads of h streamed,
+ * everything else cached).  Returns the previous policy, or -1 for an unknown one.
  */
 enum fss_cache_policy { FSS_CACHE_AUTO = 0, FSS_CACHE_STREAMING = 1 };
 int fss_set_cache_policy(int policy);

@@ -130,3 +130,28 @@ def test_scan_with_state_autograd():
     # and the plain entry point is untouched by all this
     out = scan_cu(alpha.to(torch.bfloat16).to(DEV), beta.to(torch.bfloat16).to(DEV))
     assert out.shape == (bs, seq, d)
+
+
+@pytest.mark.parametrize("shape", [(4, 1000, 512), (8, 4096, 1024)], ids=["small_output", "headline_shape"])
+def test_cache_policies_give_identical_results_with_states(shape):
+    """The scans with states follow the cache policy in the kernels large shapes run (hints on loads
+    and stores only): every output bit stays, on both sides of the sizes at which the automatic
+    policy switches its hints, with alphas near 1 so that the carried states matter."""
+    import fast_sequential_scan_amd as pkg
+
+    alpha, beta, dout = make_inputs("near_one", *shape, seed=21)
+    g = torch.Generator().manual_seed(22)
+    h0 = torch.randn(shape[0], shape[2], generator=g).to(DEV)
+    g_last = torch.randn(shape[0], shape[2], generator=g).to(DEV)
+    a, b, do = alpha.to(DEV), beta.to(DEV), dout.to(DEV)
+    results = {}
+    for policy in ("auto", "streaming"):
+        previous = pkg.set_cache_policy(policy)
+        try:
+            h, h_last = ext.scan_forward_state(a, b, h0)
+            results[policy] = (h, h_last, *ext.scan_backward_state(a, h, do, h0, g_last))
+        finally:
+            pkg.set_cache_policy(previous)
+    ext.workspace_status()
+    for x, y in zip(results["auto"], results["streaming"]):
+        assert torch.equal(x, y)
